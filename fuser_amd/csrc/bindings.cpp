@@ -1,0 +1,65 @@
+// Python module fuser_amd._C: submodule `nvf_cutlass` with the same six callables and argument
+// lists as the reference's nvfuser_direct.nvf_cutlass (python/python_direct/cutlass.cpp:17-117),
+// plus eager entry points for the block quantizers.
+#include <torch/extension.h>
+
+#include "nvf_cutlass.h"
+
+namespace py = pybind11;
+namespace ck = nvfuser::cutlass_kernels;
+namespace bq = nvfuser::block_quantization;
+
+PYBIND11_MODULE(_C, m) {
+  m.doc() = "MI355X implementation of nvFuser's quantized-GEMM path";
+  py::module_ cutlass = m.def_submodule("nvf_cutlass", "Block-scaled and grouped GEMMs (MI355X).");
+
+  // As in the reference bindings, the dense ops do not expose skip_checks.
+  cutlass.def(
+      "mxfp8_scaled_mm",
+      [](const torch::Tensor& a, const torch::Tensor& b, const torch::Tensor& scales_a, const torch::Tensor& scales_b,
+         const torch::Tensor& alpha, at::ScalarType out_dtype) { return ck::mxfp8_scaled_mm(a, b, scales_a, scales_b, alpha, out_dtype); },
+      "mxfp8_scaled_mm(a, b, scales_a, scales_b, alpha, out_dtype) -> Tensor");
+  cutlass.def(
+      "nvfp4_scaled_mm",
+      [](const torch::Tensor& a, const torch::Tensor& b, const torch::Tensor& scales_a, const torch::Tensor& scales_b,
+         const torch::Tensor& alpha, at::ScalarType out_dtype) { return ck::nvfp4_scaled_mm(a, b, scales_a, scales_b, alpha, out_dtype); },
+      "nvfp4_scaled_mm(a, b, scales_a, scales_b, alpha, out_dtype) -> Tensor");
+  cutlass.def("grouped_mm", &ck::grouped_mm,
+              "grouped_mm(a, b, ab_strides, c_strides, problem_sizes, expert_offsets) -> Tensor");
+  cutlass.def("nvfp4_scaled_grouped_mm", &ck::nvfp4_scaled_grouped_mm,
+              "nvfp4_scaled_grouped_mm(a, b, a_blockscale, b_blockscale, alphas, ab_strides, c_strides, "
+              "problem_sizes, expert_offsets, sf_offsets, out_dtype) -> Tensor");
+  cutlass.def(
+      "validate_inputs_nvfp4_scaled_mm",
+      [](const torch::Tensor& a, const torch::Tensor& b, const torch::Tensor& sa, const torch::Tensor& sb,
+         const torch::Tensor& alpha, bool skip_checks) { return ck::validateInputsNvfp4ScaledMm(a, b, sa, sb, alpha, skip_checks); },
+      py::arg("a"), py::arg("b"), py::arg("scales_a"), py::arg("scales_b"), py::arg("alpha"), py::arg("skip_checks") = false);
+  cutlass.def(
+      "validate_inputs_mxfp8_scaled_mm",
+      [](const torch::Tensor& a, const torch::Tensor& b, const torch::Tensor& sa, const torch::Tensor& sb,
+         const torch::Tensor& alpha, bool skip_checks) { return ck::validateInputsMxFp8ScaledMm(a, b, sa, sb, alpha, skip_checks); },
+      py::arg("a"), py::arg("b"), py::arg("scales_a"), py::arg("scales_b"), py::arg("alpha"), py::arg("skip_checks") = false);
+  cutlass.def("get_sm_version", &ck::getSMVersion);
+  cutlass.def("get_multiprocessor_count", &ck::getMultiProcessorCount);
+
+  m.def(
+      "nv_block_quantize",
+      [](const torch::Tensor& input, const c10::optional<torch::Tensor>& global_scale, bool swizzle_block_scales,
+         int64_t block_size, at::ScalarType dtype) {
+        auto r = bq::nv_block_quantize(input, global_scale, swizzle_block_scales, block_size, dtype);
+        return py::make_tuple(r.first, r.second);
+      },
+      py::arg("input"), py::arg("global_scale") = py::none(), py::arg("swizzle_block_scales") = false,
+      py::arg("block_size") = 16, py::arg("dtype") = at::ScalarType::Float4_e2m1fn_x2);
+  m.def(
+      "nv_grouped_block_quantize",
+      [](const torch::Tensor& input, const torch::Tensor& input_offsets, const torch::Tensor& output_offsets,
+         const c10::optional<torch::Tensor>& global_scale, int64_t block_size, at::ScalarType dtype) {
+        auto r = bq::nv_grouped_block_quantize(input, input_offsets, output_offsets, global_scale, block_size, dtype);
+        return py::make_tuple(r.first, r.second);
+      },
+      py::arg("input"), py::arg("input_offsets"), py::arg("output_offsets"), py::arg("global_scale") = py::none(),
+      py::arg("block_size") = 16, py::arg("dtype") = at::ScalarType::Float4_e2m1fn_x2);
+  m.def("preprocess_grouped_matmul_input_sf", &bq::preprocess_grouped_matmul_input_sf, py::arg("input"),
+        py::arg("input_offsets"), py::arg("output_offsets"));
+}

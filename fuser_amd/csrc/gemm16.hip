@@ -1,0 +1,367 @@
+// GEMMs whose MFMA operands are 16-bit floats, for gfx950:
+//   * nvfp4_scaled_mm          (cutlass/nvfp4_scaled_mm.cu:283-312)
+//   * nvfp4_scaled_grouped_mm  (cutlass/nvfp4_scaled_group_mm.cu:714-788, pointer rule :83-155)
+//   * grouped_mm               (cutlass/group_mm.cu:518-571, pointer rule :76-105)
+//
+// NVFP4 has one e4m3 scale per 16 elements, which the block-32 / e8m0 scaled MFMA of gfx950 cannot
+// express.  An e2m1 value times an e4m3 scale has at most 6 significant bits and an exponent range
+// of 2^-10 .. 2^11, so it is exactly representable in fp16: tiles are dequantised to fp16 while
+// they are staged into LDS and fed to v_mfma_f32_32x32x16_f16 with fp32 accumulation.  Every
+// product is exact; only the fp32 accumulation order differs from any other correct implementation.
+//
+// All three ops share one kernel: a persistent workgroup walks (group, m-tile, n-tile) work items
+// whose list is derived on the device from problem_sizes, so no host synchronisation is needed and
+// empty groups cost nothing.  The dense op is the one-group case.
+//
+// Output layout trick: the MFMA is issued with the B fragment as first operand, so that a lane's
+// accumulator registers hold 4 consecutive N-elements of one output row and are stored as 8 bytes.
+#include "nvf_internal.h"
+
+namespace nvf {
+namespace {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kMaxGroups = 1024;  // same bound as the reference's <<<1, num_experts>>> set-up kernel
+
+struct Params {
+  const uint8_t* a;
+  const uint8_t* b;
+  const uint8_t* sfa;
+  const uint8_t* sfb;
+  const float* alpha;
+  void* out;
+  const int32_t* problem_sizes;   // nullptr => dense
+  const int32_t* expert_offsets;
+  const int32_t* sf_offsets;
+  int groups;
+  int m, n, k;
+};
+
+__device__ __forceinline__ uint32_t pack2(float a, float b, bool out_bf16) {
+  if (out_bf16) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    bf16x2 v = {(__bf16)a, (__bf16)b};
+    return __builtin_bit_cast(uint32_t, v);
+  }
+  f16x2 v = {(_Float16)a, (_Float16)b};
+  return __builtin_bit_cast(uint32_t, v);
+}
+
+// 32 packed e2m1 values (16 bytes) times two e4m3 block scales -> 32 fp16 values (4 x 16 bytes)
+__device__ __forceinline__ void dequant32(const u32x4 q, uint32_t sf2, u32x4 out[4]) {
+  const _Float16 s0 = (_Float16)e4m3_to_f32(sf2 & 0xffu);
+  const _Float16 s1 = (_Float16)e4m3_to_f32((sf2 >> 8) & 0xffu);
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {  // dword w holds elements 8w .. 8w+7 ; block = w / 2
+    const _Float16 s = (w < 2) ? s0 : s1;
+    const f16x2 sv = {s, s};
+    f16x2 h0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(q[w], 1.0f, 0) * sv;
+    f16x2 h1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(q[w], 1.0f, 1) * sv;
+    f16x2 h2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(q[w], 1.0f, 2) * sv;
+    f16x2 h3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(q[w], 1.0f, 3) * sv;
+    out[w] = u32x4{__builtin_bit_cast(uint32_t, h0), __builtin_bit_cast(uint32_t, h1), __builtin_bit_cast(uint32_t, h2),
+                   __builtin_bit_cast(uint32_t, h3)};
+  }
+}
+
+// LDS tile: rows x 64 16-bit elements (128 bytes per row); 16-byte chunk c of row r sits at
+// chunk position c ^ (r & 7) so that both the staging writes and the MFMA fragment reads of
+// 8 consecutive lanes fall into distinct banks.
+__device__ __forceinline__ int lds_pos(int row, int chunk) { return row * 8 + (chunk ^ (row & 7)); }
+
+template <int BM, int BN, bool NVFP4, bool BF16_MMA, bool OUT_BF16>
+__global__ __launch_bounds__(256) void gemm16_kernel(const Params p) {
+  constexpr int BK = 64;
+  constexpr int WTM = BM / 2, WTN = BN / 2;  // wave tile
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  extern __shared__ u32x4 lds[];
+  u32x4* lds_a = lds;
+  u32x4* lds_b = lds + BM * 8;
+  __shared__ int tile_prefix[kMaxGroups + 1];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int tiles_n = (p.n + BN - 1) / BN;
+  const bool dense = p.problem_sizes == nullptr;
+
+  // ---- work list: prefix sums of tiles per group ----
+  if (dense) {
+    if (tid == 0) {
+      tile_prefix[0] = 0;
+      tile_prefix[1] = ((p.m + BM - 1) / BM) * tiles_n;
+    }
+  } else {
+    // serial scan by one wavefront in chunks of 64 groups
+    if (wave == 0) {
+      int running = 0;
+      for (int base = 0; base < p.groups; base += 64) {
+        const int g = base + lane;
+        int cnt = 0;
+        if (g < p.groups) {
+          const int mg = p.problem_sizes[g * 3];
+          cnt = mg > 0 ? ((mg + BM - 1) / BM) * tiles_n : 0;
+        }
+        int incl = cnt;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+          const int o = __shfl_up(incl, d, 64);
+          if (lane >= d) incl += o;
+        }
+        if (g < p.groups) tile_prefix[g + 1] = running + incl;
+        running += __shfl(incl, 63, 64);
+      }
+      if (lane == 0) tile_prefix[0] = 0;
+    }
+  }
+  __syncthreads();
+  const int total_tiles = tile_prefix[p.groups];
+
+  const int kbytes = NVFP4 ? p.k / 2 : p.k * 2;     // bytes per operand row
+  const int sf_cols = p.k / 16;
+  const int sf_padded = (sf_cols + 3) & ~3;
+  const int nk = (p.k + BK - 1) / BK;
+
+  for (int tile = blockIdx.x; tile < total_tiles; tile += gridDim.x) {
+    // ---- decode work item ----
+    int g = 0;
+    {
+      int lo = 0, hi = p.groups;
+      while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (tile < tile_prefix[mid]) hi = mid; else lo = mid;
+      }
+      g = lo;
+    }
+    const int m_g = dense ? p.m : p.problem_sizes[g * 3];
+    const int64_t row_off = dense ? 0 : p.expert_offsets[g];
+    const int tiles_m = (m_g + BM - 1) / BM;
+    const int local = tile - tile_prefix[g];
+    const int mt = local % tiles_m, nt = local / tiles_m;
+    const int m0 = mt * BM, n0 = nt * BN;
+
+    const uint8_t* a_base = p.a + (row_off + m0) * (int64_t)kbytes;
+    const uint8_t* b_base = p.b + ((int64_t)g * p.n + n0) * (int64_t)kbytes;
+    const uint8_t* sfa_base = nullptr;
+    const uint8_t* sfb_base = nullptr;
+    if constexpr (NVFP4) {
+      const int64_t sf_row_off = dense ? 0 : p.sf_offsets[g];
+      sfa_base = p.sfa + sf_row_off * sf_cols;           // group slab, swizzled on its own
+      sfb_base = p.sfb + (int64_t)g * p.n * sf_cols;
+    }
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    // ---- staging registers ----
+    constexpr int A_TOTAL = NVFP4 ? BM * 2 : BM * 8;  // 16-byte global chunks per tile
+    constexpr int B_TOTAL = NVFP4 ? BN * 2 : BN * 8;
+    constexpr int A_CH = (A_TOTAL + 255) / 256;       // ... per thread
+    constexpr int B_CH = (B_TOTAL + 255) / 256;
+    u32x4 sa[A_CH], sb[B_CH];
+    uint32_t ssa[NVFP4 ? A_CH : 1], ssb[NVFP4 ? B_CH : 1];
+
+    auto issue_loads = [&](int ks) {
+      const int kbyte0 = NVFP4 ? ks * (BK / 2) : ks * (BK * 2);
+#pragma unroll
+      for (int i = 0; i < A_CH; ++i) {
+        const int c = tid + 256 * i;
+        const int row = NVFP4 ? (c >> 1) : (c >> 3);
+        const int chunk = NVFP4 ? (c & 1) : (c & 7);
+        const bool ok = (c < A_TOTAL) && (m0 + row < m_g) && (kbyte0 + chunk * 16 < kbytes);
+        sa[i] = u32x4{0, 0, 0, 0};
+        if (ok) sa[i] = *reinterpret_cast<const u32x4*>(a_base + (int64_t)row * kbytes + kbyte0 + chunk * 16);
+        if constexpr (NVFP4) {
+          ssa[i] = 0;
+          if (ok)
+            ssa[i] = *reinterpret_cast<const uint16_t*>(sfa_base + swizzle_128x4(m0 + row, ks * 4, sf_padded) + chunk * 2);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < B_CH; ++i) {
+        const int c = tid + 256 * i;
+        const int row = NVFP4 ? (c >> 1) : (c >> 3);
+        const int chunk = NVFP4 ? (c & 1) : (c & 7);
+        const bool ok = (c < B_TOTAL) && (n0 + row < p.n) && (kbyte0 + chunk * 16 < kbytes);
+        sb[i] = u32x4{0, 0, 0, 0};
+        if (ok) sb[i] = *reinterpret_cast<const u32x4*>(b_base + (int64_t)row * kbytes + kbyte0 + chunk * 16);
+        if constexpr (NVFP4) {
+          ssb[i] = 0;
+          if (ok)
+            ssb[i] = *reinterpret_cast<const uint16_t*>(sfb_base + swizzle_128x4(n0 + row, ks * 4, sf_padded) + chunk * 2);
+        }
+      }
+    };
+
+    auto store_lds = [&]() {
+#pragma unroll
+      for (int i = 0; i < A_CH; ++i) {
+        const int c = tid + 256 * i;
+        if (c >= A_TOTAL) break;
+        if constexpr (NVFP4) {
+          const int row = c >> 1, half = c & 1;
+          u32x4 d[4];
+          dequant32(sa[i], ssa[i], d);
+#pragma unroll
+          for (int q = 0; q < 4; ++q) lds_a[lds_pos(row, half * 4 + q)] = d[q];
+        } else {
+          lds_a[lds_pos(c >> 3, c & 7)] = sa[i];
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < B_CH; ++i) {
+        const int c = tid + 256 * i;
+        if (c >= B_TOTAL) break;
+        if constexpr (NVFP4) {
+          const int row = c >> 1, half = c & 1;
+          u32x4 d[4];
+          dequant32(sb[i], ssb[i], d);
+#pragma unroll
+          for (int q = 0; q < 4; ++q) lds_b[lds_pos(row, half * 4 + q)] = d[q];
+        } else {
+          lds_b[lds_pos(c >> 3, c & 7)] = sb[i];
+        }
+      }
+    };
+
+    issue_loads(0);
+    for (int ks = 0; ks < nk; ++ks) {
+      __syncthreads();  // previous step's fragment reads are done
+      store_lds();
+      __syncthreads();
+      if (ks + 1 < nk) issue_loads(ks + 1);
+
+#pragma unroll
+      for (int kk = 0; kk < BK / 16; ++kk) {
+        u32x4 fa[TM], fb[TN];
+        const int chunk = kk * 2 + (lane >> 5);
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fa[i] = lds_a[lds_pos(wm * WTM + i * 32 + (lane & 31), chunk)];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fb[j] = lds_b[lds_pos(wn * WTN + j * 32 + (lane & 31), chunk)];
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j) {
+            if constexpr (BF16_MMA) {
+              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fb[j]),
+                                                                  __builtin_bit_cast(bf16x8, fa[i]), acc[i][j], 0, 0, 0);
+            } else {
+              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, fb[j]),
+                                                                 __builtin_bit_cast(f16x8, fa[i]), acc[i][j], 0, 0, 0);
+            }
+          }
+      }
+    }
+
+    // ---- epilogue: acc[i][j][r] = C[m = lane%32][n = (r/4)*8 + (lane/32)*4 + r%4] of its 32x32 tile ----
+    float alpha = 1.0f;
+    if constexpr (NVFP4) alpha = dense ? p.alpha[0] : p.alpha[g];
+    uint16_t* out = static_cast<uint16_t*>(p.out);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int mrow = m0 + wm * WTM + i * 32 + (lane & 31);
+      if (mrow >= m_g) continue;
+      uint16_t* orow = out + (row_off + mrow) * (int64_t)p.n;
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq) {
+          const int ncol = n0 + wn * WTN + j * 32 + rq * 8 + (lane >> 5) * 4;
+          if (ncol < p.n) {
+            u32x2 v;
+            v[0] = pack2(acc[i][j][rq * 4 + 0] * alpha, acc[i][j][rq * 4 + 1] * alpha, OUT_BF16);
+            v[1] = pack2(acc[i][j][rq * 4 + 2] * alpha, acc[i][j][rq * 4 + 3] * alpha, OUT_BF16);
+            *reinterpret_cast<u32x2*>(orow + ncol) = v;
+          }
+        }
+      }
+    }
+  }
+}
+
+template <int BM, int BN, bool NVFP4, bool BF16_MMA, bool OUT_BF16>
+int launch_cfg(const Params& p, int grid, hipStream_t stream) {
+  auto kern = gemm16_kernel<BM, BN, NVFP4, BF16_MMA, OUT_BF16>;
+  constexpr int lds_bytes = (BM + BN) * 128;
+  static bool configured = false;  // benign race: the attribute call is idempotent
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    if (e != hipSuccess) return fail(NVF_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    configured = true;
+  }
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_bytes, stream, p);
+  return check_launch("gemm16_kernel");
+}
+
+template <bool NVFP4, bool BF16_MMA, bool OUT_BF16>
+int launch_sized(const Params& p, int64_t m_hint, int cus, hipStream_t stream) {
+  // Pick the largest tile that still yields about one work item per compute unit.
+  auto tiles = [&](int bm, int bn) { return ceil_div(m_hint, bm) * ceil_div(p.n, bn); };
+  const bool dense = p.problem_sizes == nullptr;
+  if (tiles(256, 256) >= cus || (!dense && m_hint >= 256 * (int64_t)p.groups)) {
+    const int64_t upper = dense ? tiles(256, 256) : (ceil_div(p.m, 256) + p.groups) * ceil_div(p.n, 256);
+    return launch_cfg<256, 256, NVFP4, BF16_MMA, OUT_BF16>(p, (int)(upper < cus ? upper : cus), stream);
+  }
+  if (tiles(128, 128) >= cus || !dense) {
+    const int64_t upper = dense ? tiles(128, 128) : (ceil_div(p.m, 128) + p.groups) * ceil_div(p.n, 128);
+    const int64_t cap = 2 * (int64_t)cus;
+    return launch_cfg<128, 128, NVFP4, BF16_MMA, OUT_BF16>(p, (int)(upper < cap ? upper : cap), stream);
+  }
+  const int64_t upper = tiles(64, 64);
+  const int64_t cap = 4 * (int64_t)cus;
+  return launch_cfg<64, 64, NVFP4, BF16_MMA, OUT_BF16>(p, (int)(upper < cap ? upper : cap), stream);
+}
+
+int cu_count() {
+  static int cached = 0;
+  if (cached == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+      cached = n;
+    else
+      return 256;
+  }
+  return cached;
+}
+
+}  // namespace
+
+int launch_gemm16(int op, const Gemm16Args& a, hipStream_t stream) {
+  if (a.groups > kMaxGroups) return fail(NVF_ERR_UNSUPPORTED_SHAPE, "at most %d groups are supported, got %d", kMaxGroups, a.groups);
+  if (a.m > INT32_MAX || a.n > INT32_MAX || a.k > INT32_MAX) return fail(NVF_ERR_UNSUPPORTED_SHAPE, "dimension exceeds int32");
+  Params p;
+  p.a = static_cast<const uint8_t*>(a.a);
+  p.b = static_cast<const uint8_t*>(a.b);
+  p.sfa = static_cast<const uint8_t*>(a.sfa);
+  p.sfb = static_cast<const uint8_t*>(a.sfb);
+  p.alpha = a.alpha;
+  p.out = a.out;
+  p.problem_sizes = a.problem_sizes;
+  p.expert_offsets = a.expert_offsets;
+  p.sf_offsets = a.sf_offsets;
+  p.groups = op == 0 ? 1 : a.groups;
+  p.m = (int)a.m;
+  p.n = (int)a.n;
+  p.k = (int)a.k;
+  const int cus = cu_count();
+  const bool bf16 = a.dtype == NVF_BF16;
+  if (op == 0 || op == 1) {
+    return bf16 ? launch_sized<true, false, true>(p, a.m, cus, stream) : launch_sized<true, false, false>(p, a.m, cus, stream);
+  }
+  return bf16 ? launch_sized<false, true, true>(p, a.m, cus, stream) : launch_sized<false, false, false>(p, a.m, cus, stream);
+}
+
+}  // namespace nvf

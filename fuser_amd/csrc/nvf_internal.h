@@ -1,0 +1,105 @@
+// Internal helpers shared by the HIP translation units of libnvf_hip.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <cstdarg>
+#include <cstdio>
+
+#include "nvf_hip.h"
+
+namespace nvf {
+
+// Records a message for nvf_last_error() and returns `status`.
+int fail(int status, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
+// Checks the launch that was just issued on the calling thread.
+int check_launch(const char* what);
+
+inline int64_t ceil_div(int64_t x, int64_t y) { return (x + y - 1) / y; }
+inline int64_t round_up(int64_t x, int64_t y) { return ceil_div(x, y) * y; }
+
+#define NVF_REQUIRE(cond, status, ...) \
+  do {                                 \
+    if (!(cond)) return ::nvf::fail((status), __VA_ARGS__); \
+  } while (0)
+
+// ---- launchers implemented in the kernel translation units ----
+int launch_nvfp4_quantize(const void* in, int in_dtype, int64_t rows, int64_t cols, const float* gs, int layout,
+                          const int32_t* in_off, const int32_t* out_off, int groups, void* out_fp4, void* out_sf,
+                          hipStream_t stream);
+int launch_preprocess_sf(const void* in, int elem_size, int64_t rows, int64_t cols, const int32_t* in_off,
+                         const int32_t* out_off, int groups, void* out, hipStream_t stream);
+int launch_mxfp8_quantize(const void* in, int in_dtype, int64_t rows, int64_t cols, int swizzle, void* out_fp8,
+                          void* out_sf, hipStream_t stream);
+int launch_cast(int kind, const float* in, int64_t n, uint8_t* out, hipStream_t stream);
+
+// op: 0 dense NVFP4, 1 grouped NVFP4, 2 grouped bf16/f16
+struct Gemm16Args {
+  const void* a;
+  const void* b;
+  const void* sfa;
+  const void* sfb;
+  const float* alpha;  // dense: scalar; grouped NVFP4: [groups]; grouped 16-bit: nullptr
+  void* out;
+  const int32_t* problem_sizes;
+  const int32_t* expert_offsets;
+  const int32_t* sf_offsets;
+  int groups;
+  int64_t m, n, k;
+  int dtype;  // out dtype (NVFP4 ops) or in/out dtype (grouped_mm)
+};
+int launch_gemm16(int op, const Gemm16Args& args, hipStream_t stream);
+int launch_mxfp8_gemm(const void* a, const void* b, const void* sfa, const void* sfb, const float* alpha, void* out,
+                      int64_t m, int64_t n, int64_t k, int out_dtype, hipStream_t stream);
+
+}  // namespace nvf
+
+// ------------------------------------------------------------------------------------------------
+// Device-side narrow-float codecs (gfx950).
+// ------------------------------------------------------------------------------------------------
+#if defined(__HIPCC__)
+namespace nvf {
+
+__device__ __forceinline__ float bits_to_f32(uint32_t u) { return __uint_as_float(u); }
+__device__ __forceinline__ uint32_t f32_to_bits(float f) { return __float_as_uint(f); }
+
+// 128x4 scale layout: byte offset of (row, col) in a buffer with `padded_cols` columns.
+__device__ __forceinline__ int64_t swizzle_128x4(int64_t row, int64_t col, int64_t padded_cols) {
+  return (row >> 7) * (padded_cols << 7) + ((col >> 2) << 9) + ((row & 31) << 4) + (((row >> 5) & 3) << 2) + (col & 3);
+}
+
+// e4m3fn decode, exact (hardware convert, verified for all 256 codes).
+__device__ __forceinline__ float e4m3_to_f32(uint32_t code) { return __builtin_amdgcn_cvt_f32_fp8((int)code, 0); }
+
+// e4m3fn encode, round-to-nearest-even, saturating to +-448, NaN -> 0x7F.
+// The hardware convert rounds correctly but turns overflow into NaN, hence the clamp.
+__device__ __forceinline__ uint32_t f32_to_e4m3_satfinite(float x) {
+  if (x != x) return 0x7fu;
+  float c = fminf(fmaxf(x, -448.0f), 448.0f);
+  return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(c, c, 0, false) & 0xffu;
+}
+
+// e2m1 encode of two values into one byte (first value in the low nibble), RNE, saturating to
+// +-6.  The hardware convert does exactly that for every non-NaN input; NaN is mapped to +6.
+__device__ __forceinline__ uint32_t f32x2_to_e2m1_byte(float lo, float hi) {
+  uint32_t r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(0u, lo, hi, 1.0f, 0) & 0xffu;
+  if (lo != lo) r = (r & 0xf0u) | 0x07u;
+  if (hi != hi) r = (r & 0x0fu) | 0x70u;
+  return r;
+}
+
+// ue8m0 encode, round toward +inf (smallest power of two >= x), saturating; NaN -> 0xFF;
+// zero and negative inputs -> 0.
+__device__ __forceinline__ uint32_t f32_to_e8m0_rp(float x) {
+  uint32_t b = f32_to_bits(x);
+  if (x != x) return 0xffu;
+  if ((b >> 31) || b == 0) return 0u;
+  uint32_t e = b >> 23, m = b & 0x7fffffu;
+  if (e == 255) return 0xfeu;
+  if (e == 0) return m > 0x400000u ? 1u : 0u;  // denormal: 2^-127 is e8m0 code 0
+  uint32_t r = e + (m != 0);
+  return r > 254u ? 254u : r;
+}
+
+}  // namespace nvf
+#endif
