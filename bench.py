@@ -1,0 +1,288 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-GEMM hot path on one MI355X.
+
+A step is one ``mxfp8_scaled_mm`` of M=N=K=8192 (BASELINE config 2, the shape the metric is quoted
+on): e4m3 operands with e8m0 per-32 scales in the 128x4 layout, bf16 output, inputs resident in HBM.
+``value`` is its throughput in TFLOP/s (2*M*N*K per step).  The same JSON line carries
+  roofline      the MXFP8 GEMM kernel against the dense fp8 MFMA peak (5.0 PFLOP/s),
+  cpu_baseline  the PyTorch-CPU dequantize + fp32 matmul reference on a bounded sample,
+  extra         the other workloads of the metric: NVFP4 block quantize GB/s at the config-5
+                activation size (with its own HBM roofline), NVFP4 GEMM 8192^3, the dense-LLM
+                shapes of config 3, and the grouped GEMMs of configs 4 and 5.
+Synthetic data: seeded N(0,1) / N(0,0.02) bf16 tensors quantized by the library's own quantizers.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP8_TFLOPS = 5000.0   # MI355X dense fp8 MFMA
+PEAK_F16_TFLOPS = 2500.0   # dense bf16 / fp16 MFMA
+PEAK_HBM_GBS = 8000.0      # HBM3E
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg (profiling runs)")
+    ap.add_argument("--no-extra", action="store_true", help="only the headline MXFP8 workload")
+    ap.add_argument("--calib", action="store_true", help="profiling aid: also run a plain 1 GiB device copy a few times, "
+                    "so that a counter run shows what FETCH_SIZE / WRITE_SIZE read for a kernel of known traffic")
+    ap.add_argument("--only", default="", help="profiling aid: run just this extra workload "
+                    "(quant | nvfp4 | llm | grouped | gnvfp4) and print its line")
+    return ap.parse_args()
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU; every kernel of the path is single-device "
+              "(run with --gpus 1).", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from fuser_amd import nvf_cutlass, ops
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    one = torch.tensor(1.0, device=dev)
+
+    def timed(fn, steps, warmup):
+        """Average milliseconds per call: HIP events on the launch stream around `steps` calls."""
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        wall = (time.perf_counter() - t0) * 1e3 / steps
+        return e0.elapsed_time(e1) / steps, wall
+
+    def ru(x, y):
+        return (x + y - 1) // y * y
+
+    def moe_top2(tokens, experts, seed):
+        gen = torch.Generator().manual_seed(seed)
+        logits = torch.randn(tokens, experts, generator=gen) + torch.linspace(-1.5, 1.5, experts)
+        return torch.bincount(logits.topk(2, dim=1).indices.flatten(), minlength=experts)
+
+    def moe_zipf(tokens, topk, experts, s, seed):
+        gen = torch.Generator().manual_seed(seed)
+        p = 1.0 / torch.arange(1, experts + 1).float() ** s
+        p = p[torch.randperm(experts, generator=gen)]
+        idx = torch.multinomial(p.expand(tokens, experts), topk, replacement=False, generator=gen).flatten()
+        return torch.bincount(idx, minlength=experts)
+
+    extra = {}
+    gen = torch.Generator(device=dev).manual_seed(0)
+
+    # ------------------------------------------------------------------ extras
+    def run_quant():
+        m, k = 65536, 7168
+        x = torch.randn(m, k, device=dev, generator=gen).bfloat16()
+        gs = (2688.0 / x.float().abs().max()).float()
+        ms, _ = timed(lambda: ops.nv_block_quantize(x, gs, True, 16), 30, 5)
+        gbs = m * k * 2.5625 / ms / 1e6
+        extra["nvfp4_quantize"] = {"workload": "bf16 [65536,7168] -> NVFP4, 128x4 swizzled scales (config 5 activations)",
+                                   "ms": round(ms, 4), "GB/s": round(gbs, 1),
+                                   "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                                "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None}}
+        sizes = moe_zipf(8192, 8, 256, 1.1, 0).int()
+        padded = (sizes + 127) // 128 * 128
+        eo = (torch.cumsum(sizes, 0) - sizes).int().to(dev)
+        so = (torch.cumsum(padded, 0) - padded).int().to(dev)
+        ms, _ = timed(lambda: ops.nv_grouped_block_quantize(x, eo, so, None, 16), 30, 5)
+        extra["nvfp4_grouped_quantize"] = {"workload": "same tensor, 256 Zipf(1.1) groups", "ms": round(ms, 4),
+                                           "GB/s": round(m * k * 2.5625 / ms / 1e6, 1)}
+        for (mm, kk) in ((256, 1024), (2048, 4096)):
+            xs = torch.randn(mm, kk, device=dev, generator=gen).bfloat16()
+            ms, _ = timed(lambda: ops.nv_block_quantize(xs, gs, True, 16), 50, 5)
+            extra[f"nvfp4_quantize_{mm}x{kk}"] = {"us": round(ms * 1e3, 2), "GB/s": round(mm * kk * 2.5625 / ms / 1e6, 1)}
+
+    def quantized_nvfp4(rows, k, std):
+        x = (torch.randn(rows, k, device=dev, generator=gen) * std).bfloat16()
+        gs = (2688.0 / x.float().abs().max()).float()
+        q, s = ops.nv_block_quantize(x, gs, True, 16)
+        return q, s, gs
+
+    def run_nvfp4():
+        m = n = k = 8192
+        a, sa, ga = quantized_nvfp4(m, k, 1.0)
+        b, sb, gb = quantized_nvfp4(n, k, 1.0)
+        alpha = (1.0 / (ga * gb)).float()
+        ms, _ = timed(lambda: nvf_cutlass.nvfp4_scaled_mm(a, b, sa, sb, alpha, torch.bfloat16), 20, 3)
+        tf = 2.0 * m * n * k / ms / 1e9
+        extra["nvfp4_gemm_8192"] = {"ms": round(ms, 4), "TFLOP/s": round(tf, 1),
+                                    "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
+                                                 "frac": round(tf / PEAK_F16_TFLOPS, 4), "traffic": None,
+                                                 "note": "fp16 MFMA issued (exact fp16 dequantisation of e2m1 x e4m3)"}}
+
+    def run_llm():
+        res = {}
+        for (n, k) in ((4096, 4096), (14336, 4096), (4096, 14336)):
+            w, sw, gw = quantized_nvfp4(n, k, 0.02)
+            for m in (16, 128, 2048):
+                x = torch.randn(m, k, device=dev, generator=gen).bfloat16()
+                gx = (2688.0 / x.float().abs().max()).float()
+                alpha = (1.0 / (gx * gw)).float()
+                qx, sx = ops.nv_block_quantize(x, gx, True, 16)
+                ms_q, _ = timed(lambda: ops.nv_block_quantize(x, gx, True, 16), 50, 5)
+                ms_g, _ = timed(lambda: nvf_cutlass.nvfp4_scaled_mm(qx, w, sx, sw, alpha, torch.bfloat16), 50, 5)
+
+                def seq():
+                    q, s = ops.nv_block_quantize(x, gx, True, 16)
+                    return nvf_cutlass.nvfp4_scaled_mm(q, w, s, sw, alpha, torch.bfloat16)
+
+                ms_s, _ = timed(seq, 50, 5)
+                byts = n * k * 0.5625 + m * k * 0.5625 + 2 * m * n
+                res[f"M{m}_N{n}_K{k}"] = {"quant_us": round(ms_q * 1e3, 2), "gemm_us": round(ms_g * 1e3, 2), "seq_us": round(ms_s * 1e3, 2),
+                                          "gemm_TFLOP/s": round(2.0 * m * n * k / ms_g / 1e9, 1), "gemm_GB/s": round(byts / ms_g / 1e6, 1)}
+        extra["nvfp4_gemm_llm_shapes"] = res
+
+    def run_grouped():
+        g, k, n = 8, 4096, 14336
+        sizes = moe_top2(4096, g, 0).int()
+        rows = int(sizes.sum())
+        a = torch.randn(rows, k, device=dev, generator=gen).bfloat16()
+        b = (torch.randn(g, n, k, device=dev, generator=gen) * 0.02).bfloat16()
+        ps = torch.stack([sizes, torch.full_like(sizes, n), torch.full_like(sizes, k)], 1).int().to(dev)
+        eo = (torch.cumsum(sizes, 0) - sizes).int().to(dev)
+        st = torch.full((g,), k, dtype=torch.int64, device=dev)
+        ct = torch.full((g,), n, dtype=torch.int64, device=dev)
+        ms, _ = timed(lambda: nvf_cutlass.grouped_mm(a, b, st, ct, ps, eo), 15, 3)
+        tf = 2.0 * rows * n * k / ms / 1e9
+        extra["grouped_mm_bf16"] = {"workload": f"config 4: 8 experts, sizes {sizes.tolist()}, K=4096, N=14336", "ms": round(ms, 4),
+                                    "TFLOP/s": round(tf, 1), "frac_of_bf16_peak": round(tf / PEAK_F16_TFLOPS, 4)}
+
+    def run_gnvfp4():
+        g, rows = 256, 65536
+        sizes = moe_zipf(8192, 8, g, 1.1, 0).int()
+        padded = (sizes + 127) // 128 * 128
+        eo = (torch.cumsum(sizes, 0) - sizes).int().to(dev)
+        so = (torch.cumsum(padded, 0) - padded).int().to(dev)
+        res = {"group_sizes_min_median_max": [int(sizes.min()), int(sizes.median()), int(sizes.max())]}
+        for (k, n) in ((7168, 2048), (2048, 7168)):
+            x = torch.randn(rows, k, device=dev, generator=gen).bfloat16()
+            aq, asf = ops.nv_grouped_block_quantize(x, eo, so, None, 16)
+            bq = torch.empty(g, n, k // 2, dtype=torch.uint8, device=dev)
+            bsf = torch.empty(g, n, k // 16, dtype=torch.uint8, device=dev)
+            alphas = torch.empty(g, device=dev)
+            for e in range(g):
+                w = (torch.randn(n, k, device=dev, generator=gen) * 0.02).bfloat16()
+                gs = (2688.0 / w.float().abs().max()).float()
+                q, s = ops.nv_block_quantize(w, gs, True, 16)
+                bq[e], bsf[e], alphas[e] = q.view(torch.uint8), s.view(torch.uint8), 1.0 / gs
+            bq4, bsf8 = bq.view(torch.float4_e2m1fn_x2), bsf.view(torch.float8_e4m3fn)
+            ps = torch.stack([sizes, torch.full_like(sizes, n), torch.full_like(sizes, k)], 1).int().to(dev)
+            st = torch.full((g,), k, dtype=torch.int64, device=dev)
+            ct = torch.full((g,), n, dtype=torch.int64, device=dev)
+            ms, _ = timed(lambda: nvf_cutlass.nvfp4_scaled_grouped_mm(aq, bq4, asf, bsf8, alphas, st, ct, ps, eo, so, torch.bfloat16), 10, 2)
+            tf = 2.0 * rows * n * k / ms / 1e9
+            res[f"K{k}_N{n}"] = {"ms": round(ms, 4), "useful_TFLOP/s": round(tf, 1), "frac_of_f16_peak": round(tf / PEAK_F16_TFLOPS, 4)}
+            del bq, bsf, bq4, bsf8, x, aq, asf
+        extra["nvfp4_grouped_mm"] = res
+
+    if args.calib:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 256)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
+    runners = {"quant": run_quant, "nvfp4": run_nvfp4, "llm": run_llm, "grouped": run_grouped, "gnvfp4": run_gnvfp4}
+    if args.only:
+        runners[args.only]()
+        print(json.dumps({"only": args.only, "extra": extra}))
+        return
+
+    # ------------------------------------------------------------------ headline: MXFP8 8192^3
+    m = n = k = 8192
+    a = torch.randn(m, k, device=dev, generator=gen).bfloat16()
+    b = torch.randn(n, k, device=dev, generator=gen).bfloat16()
+    qa, sa = ops.nv_block_quantize(a, None, True, 32, torch.float8_e4m3fn)
+    qb, sb = ops.nv_block_quantize(b, None, True, 32, torch.float8_e4m3fn)
+    del a, b
+    flops = 2.0 * m * n * k
+    ms, wall_ms = timed(lambda: nvf_cutlass.mxfp8_scaled_mm(qa, qb, sa, sb, one, torch.bfloat16), args.steps, args.warmup)
+    tflops = flops / ms / 1e9
+
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tpath):
+        traffic = json.load(open(tpath)).get("mxfp8_gemm_8192_bytes_per_launch")
+
+    # ------------------------------------------------------------------ CPU baseline (bounded sample)
+    cpu = None
+    if not args.no_cpu:
+        from oracle import nvf_oracle as O
+
+        threads = os.cpu_count() or 1
+        threads = min(threads, 16)
+        torch.set_num_threads(threads)
+        ha, hsa = qa.view(torch.uint8).cpu(), sa.view(torch.uint8).cpu()
+        hb, hsb = qb.view(torch.uint8).cpu(), sb.view(torch.uint8).cpu()
+        runs = []
+        for _ in range(5):
+            t0 = time.perf_counter()
+            da = O.dequantize_mxfp8_fast(ha, hsa)
+            db = O.dequantize_mxfp8_fast(hb, hsb)
+            t1 = time.perf_counter()
+            ref = torch.matmul(da, db.t())
+            t2 = time.perf_counter()
+            runs.append((t2 - t0, t1 - t0, t2 - t1))
+            if sum(r[0] for r in runs) > 25.0:
+                break
+        runs.sort()
+        tot, tdq, tmm = runs[len(runs) // 2]
+        got = nvf_cutlass.mxfp8_scaled_mm(qa, qb, sa, sb, one, torch.bfloat16)
+        rows = torch.arange(0, m, 61)
+        err = ((got[rows.to(dev)].float().cpu() - ref[rows]).abs().max() / ref[rows].abs().max()).item()
+        cpu = {"value": round(flops / tot / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+               "sample": f"the whole 8192^3 workload, median of {len(runs)} runs: torch-CPU dequantize ({tdq:.2f} s) + fp32 matmul "
+                         f"({tmm:.2f} s)",
+               "gpu_vs_cpu_max_rel": round(err, 6)}
+        del da, db, ref, got
+
+    if not args.no_extra:
+        for name in ("quant", "nvfp4", "llm", "grouped", "gnvfp4"):
+            runners[name]()
+
+    line = {
+        "metric": "mxfp8_scaled_mm TFLOP/s, M=N=K=8192, bf16 out (+ NVFP4 quantize GB/s and NVFP4 GEMM TFLOP/s in extra)",
+        "value": round(tflops, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms, 5),
+        "wall_ms_per_step": round(wall_ms, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "fp8_e4m3 x fp8_e4m3 -> f32 accumulate -> bf16",
+        "data": "synthetic: seeded N(0,1) bf16 quantized to MXFP8 on the GPU",
+        "config": {"workload": "BASELINE config 2: MXFP8 scaled GEMM M=N=K=8192, e8m0 per-32 scales in 128x4 layout, A row-major, B K-major"},
+        "roofline": {"bound": "mfma", "achieved": round(tflops, 2), "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(tflops / PEAK_FP8_TFLOPS, 4), "traffic": traffic,
+                     "kernel": "mxfp8_gemm_kernel", "flops_per_launch": flops},
+        "cpu_baseline": cpu,
+        "extra": extra,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
