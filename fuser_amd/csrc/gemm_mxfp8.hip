@@ -195,6 +195,208 @@ __global__ __launch_bounds__(256) void mxfp8_gemm_kernel(const Params p) {
   }
 }
 
+
+// -------------------------------------------------------------------------------------------------
+// Fast path: 256x256 tile, M % 256 == N % 256 == K % 128 == 0.
+//   * Tiles travel global -> LDS with 16-byte LDS-direct loads (no staging registers) into a double
+//     buffer.  They are issued from inline assembly so that the compiler does not serialise them
+//     against the LDS reads of the other buffer; completion is enforced by the explicit
+//     s_waitcnt vmcnt(0) in front of the one barrier per 128-deep K step.
+//   * MFMA fragments are double-buffered in registers: the LDS reads of the next half step are in
+//     flight under the 16 MFMAs of the current one.
+//   * A load issued in the middle of step ks is consumed after the barrier in the middle of step
+//     ks+1, i.e. it has 32 MFMAs (~2000 cycles) to land.
+// LDS layout per operand tile: 256 rows x 128 bytes; 16-byte chunk c of row r at chunk position
+// c ^ ((r >> 1) & 7): conflict-free for the fragment reads (16 consecutive lanes = 16 consecutive
+// rows, one chunk) on the 64-bank LDS.
+// -------------------------------------------------------------------------------------------------
+__device__ __forceinline__ int lds_pos2(int row, int chunk) { return row * 8 + (chunk ^ ((row >> 1) & 7)); }
+
+__device__ __forceinline__ void lds_dma16(uint32_t lds_byte_addr, const uint8_t* base, uint32_t voff) {
+  // lds_byte_addr and base are wave-uniform; lane L's 16 bytes land at lds_byte_addr + 16 * L
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_byte_addr), "v"(voff), "s"(base) : "memory");
+}
+
+template <bool OUT_BF16>
+__global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) {
+  constexpr int BM = 256, BN = 256;
+  constexpr int TILE_UNITS = 2048;            // 16-byte units per operand tile (256 rows x 8 chunks)
+  constexpr int BUF_UNITS = 2 * TILE_UNITS;   // A + B
+  extern __shared__ u32x4 lds[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int li = lane & 31, lg = lane >> 5;
+
+  // ---- tile assignment: consecutive workgroup ids land on different XCDs (id % 8), so give each
+  // XCD a contiguous range of tiles, walked in 8 (m) x 4 (n) blocks that share A / B tiles in its L2.
+  const int tiles_m = p.m / BM, tiles_n = p.n / BN;
+  int t = blockIdx.x;
+  const int nb = gridDim.x;
+  if ((nb & 7) == 0) t = (t & 7) * (nb >> 3) + (t >> 3);
+  int mt, nt;
+  if ((tiles_m & 7) == 0 && (tiles_n & 3) == 0) {
+    const int sb = t >> 5, w = t & 31;
+    const int sbm = sb % (tiles_m >> 3), sbn = sb / (tiles_m >> 3);
+    mt = sbm * 8 + (w & 7);
+    nt = sbn * 4 + (w >> 3);
+  } else {
+    mt = t % tiles_m;
+    nt = t / tiles_m;
+  }
+  const int m0 = mt * BM, n0 = nt * BN;
+  const int nk = p.k >> 7;
+  const int sf_tiles_k = (p.k >> 5) >> 2;  // 512-byte scale tiles per 128-row tile (K % 128 == 0)
+
+  // ---- LDS-direct load addressing.  Wave w issues 8 loads per operand per K step; load j covers LDS
+  // units [(w*8+j)*64, +64) = rows (w*8+j)*8 .. +7; lane L lands at unit +L, i.e. row +(L>>3), chunk
+  // position L&7, which must hold global chunk (L&7) ^ ((row>>1)&7) = (L&7) ^ ((L>>4) | ((j&1)<<2)).
+  const uint8_t* a_tile = p.a + ((int64_t)m0 + wave * 64) * p.k;  // uniform
+  const uint8_t* b_tile = p.b + ((int64_t)n0 + wave * 64) * p.k;
+  const uint32_t row_off = (uint32_t)(lane >> 3) * (uint32_t)p.k;
+  const uint32_t voff_even = row_off + (uint32_t)(((lane & 7) ^ (lane >> 4)) << 4);
+  const uint32_t voff_odd = row_off + (uint32_t)(((lane & 7) ^ ((lane >> 4) | 4)) << 4);
+  const uint32_t lds_base = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)lds);
+  const uint32_t step8 = 8u * (uint32_t)p.k;  // 8 rows
+
+  auto issue_tile_loads = [&](int ks, int buf) {
+    const uint32_t la = lds_base + (uint32_t)(buf * BUF_UNITS + wave * 512) * 16u;
+    const uint32_t lb = la + TILE_UNITS * 16u;
+    const uint8_t* ga = a_tile + ((int64_t)ks << 7);
+    const uint8_t* gb = b_tile + ((int64_t)ks << 7);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const uint32_t v = ((j & 1) ? voff_odd : voff_even) + (uint32_t)j * step8;
+      lds_dma16(la + j * 1024u, ga, v);
+      lds_dma16(lb + j * 1024u, gb, v);
+    }
+  };
+  // ---- scales: one 16-byte load per lane per K step = rows {li, li+32, li+64, li+96} of the wave's
+  // 128-row scale tile x 4 K-blocks
+  const uint8_t* psa = p.sfa + ((int64_t)((m0 >> 7) + wm) * sf_tiles_k) * 512 + li * 16;
+  const uint8_t* psb = p.sfb + ((int64_t)((n0 >> 7) + wn) * sf_tiles_k) * 512 + li * 16;
+  auto load_scales = [&](int ks, u32x4& wa, u32x4& wb) {
+    wa = *reinterpret_cast<const u32x4*>(psa + (int64_t)ks * 512);
+    wb = *reinterpret_cast<const u32x4*>(psb + (int64_t)ks * 512);
+  };
+  auto load_frags = [&](int buf, int sub, i32x8 (&fa)[4], i32x8 (&fb)[4]) {
+    const u32x4* la = lds + buf * BUF_UNITS;
+    const u32x4* lb = la + TILE_UNITS;
+    const int c_lo = sub * 4 + lg, c_hi = c_lo + 2;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = wm * 128 + i * 32 + li;
+      const u32x4 lo = la[lds_pos2(row, c_lo)], hi = la[lds_pos2(row, c_hi)];
+      fa[i] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int row = wn * 128 + j * 32 + li;
+      const u32x4 lo = lb[lds_pos2(row, c_lo)], hi = lb[lds_pos2(row, c_hi)];
+      fb[j] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+    }
+  };
+
+  f32x16 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  i32x8 fa0[4], fb0[4], fa1[4], fb1[4];
+  u32x4 sca, scb, sca_n, scb_n;
+
+  issue_tile_loads(0, 0);
+  if (nk > 1) issue_tile_loads(1, 1);
+  load_scales(0, sca, scb);
+  sca_n = sca; scb_n = scb;
+  if (nk > 1) load_scales(1, sca_n, scb_n);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  load_frags(0, 0, fa0, fb0);
+  const int sh = lg * 8;  // lane group 1 supplies K-blocks 1 and 3 of a step
+
+  // Keeps the 16 accumulator tiles "used" at this point of the program, so that the MFMAs producing
+  // them cannot be moved past the statement that follows (they have no side effects of their own).
+#define NVF_PIN_ACC()                                                                                          \
+  do {                                                                                                         \
+    asm volatile("" : "+a"(acc[0][0]), "+a"(acc[0][1]), "+a"(acc[0][2]), "+a"(acc[0][3]), "+a"(acc[1][0]),     \
+                 "+a"(acc[1][1]), "+a"(acc[1][2]), "+a"(acc[1][3]));                                           \
+    asm volatile("" : "+a"(acc[2][0]), "+a"(acc[2][1]), "+a"(acc[2][2]), "+a"(acc[2][3]), "+a"(acc[3][0]),     \
+                 "+a"(acc[3][1]), "+a"(acc[3][2]), "+a"(acc[3][3]));                                           \
+  } while (0)
+
+  for (int ks = 0; ks < nk; ++ks) {
+    const int buf = ks & 1;
+    u32x4 wa, wb;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { wa[i] = sca[i] >> sh; wb[i] = scb[i] >> sh; }
+    load_frags(buf, 1, fa1, fb1);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb0[j], fa0[i], acc[i][j], 0, 0, 0, (int)wb[j], 0, (int)wa[i]);
+    NVF_PIN_ACC();
+    // Everything this wave loaded into buf^1 has landed, and its reads of buf are complete; after the
+    // barrier that holds for every wave, so buf^1 may be read and buf may be overwritten.
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    load_frags(buf ^ 1, 0, fa0, fb0);  // on the last step this reads stale data that is never used
+    if (ks + 2 < nk) issue_tile_loads(ks + 2, buf);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb1[j], fa1[i], acc[i][j], 0, 0, 2, (int)wb[j], 2, (int)wa[i]);
+    NVF_PIN_ACC();
+    sca = sca_n; scb = scb_n;
+    if (ks + 2 < nk) load_scales(ks + 2, sca_n, scb_n);
+  }
+#undef NVF_PIN_ACC
+
+  const float alpha = p.alpha[0];
+  uint16_t* out = static_cast<uint16_t*>(p.out);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int mrow = m0 + wm * 128 + i * 32 + li;
+    uint16_t* orow = out + (int64_t)mrow * p.n;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+      for (int rq = 0; rq < 4; ++rq) {
+        const int ncol = n0 + wn * 128 + j * 32 + rq * 8 + lg * 4;
+        u32x2 v;
+        v[0] = pack2(acc[i][j][rq * 4 + 0] * alpha, acc[i][j][rq * 4 + 1] * alpha, OUT_BF16);
+        v[1] = pack2(acc[i][j][rq * 4 + 2] * alpha, acc[i][j][rq * 4 + 3] * alpha, OUT_BF16);
+        *reinterpret_cast<u32x2*>(orow + ncol) = v;
+      }
+    }
+  }
+}
+
+template <bool OUT_BF16>
+int launch_fast(const Params& p, hipStream_t stream) {
+  auto kern = mxfp8_gemm_256_kernel<OUT_BF16>;
+  constexpr int lds_bytes = 2 * 2 * 2048 * 16;  // 128 KiB
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    if (e != hipSuccess) return fail(NVF_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    configured = true;
+  }
+  const int64_t tiles = (int64_t)(p.m / 256) * (p.n / 256);
+  hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(256), lds_bytes, stream, p);
+  return check_launch("mxfp8_gemm_256_kernel");
+}
+
 template <int BM, int BN, bool OUT_BF16>
 int launch_cfg(const Params& p, hipStream_t stream) {
   auto kern = mxfp8_gemm_kernel<BM, BN, OUT_BF16>;
@@ -213,6 +415,8 @@ int launch_cfg(const Params& p, hipStream_t stream) {
 template <bool OUT_BF16>
 int launch_sized(const Params& p, hipStream_t stream) {
   auto tiles = [&](int bm, int bn) { return ceil_div(p.m, bm) * ceil_div(p.n, bn); };
+  if (tiles(256, 256) >= 128 && (p.k & 127) == 0 && (p.m & 255) == 0 && (p.n & 255) == 0 && (int64_t)p.k * 256 < (1ll << 31))
+    return launch_fast<OUT_BF16>(p, stream);
   if (tiles(256, 256) >= 256) return launch_cfg<256, 256, OUT_BF16>(p, stream);
   if (tiles(128, 128) >= 256) return launch_cfg<128, 128, OUT_BF16>(p, stream);
   return launch_cfg<64, 64, OUT_BF16>(p, stream);
