@@ -230,56 +230,83 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
   const int wm = wave >> 1, wn = wave & 1;
   const int li = lane & 31, lg = lane >> 5;
 
-  // ---- tile assignment: consecutive workgroup ids land on different XCDs (id % 8), so give each
-  // XCD a contiguous range of tiles, walked in 8 (m) x 4 (n) blocks that share A / B tiles in its L2.
+  // ---- persistent tile walk.  Workgroup ids are dealt round-robin to the 8 XCDs, so XCD x owns the
+  // contiguous tile range [x*chunk, (x+1)*chunk) and its workgroups take consecutive tiles of it in
+  // each round: with the 8 (m) x 4 (n) blocked tile numbering below, the 32 tiles an XCD works on at
+  // any time share 8 A panels and 4 B panels in that XCD's L2.
   const int tiles_m = p.m / BM, tiles_n = p.n / BN;
-  int t = blockIdx.x;
-  const int nb = gridDim.x;
-  if ((nb & 7) == 0) t = (t & 7) * (nb >> 3) + (t >> 3);
-  int mt, nt;
-  if ((tiles_m & 7) == 0 && (tiles_n & 3) == 0) {
-    const int sb = t >> 5, w = t & 31;
-    const int sbm = sb % (tiles_m >> 3), sbn = sb / (tiles_m >> 3);
-    mt = sbm * 8 + (w & 7);
-    nt = sbn * 4 + (w >> 3);
-  } else {
-    mt = t % tiles_m;
-    nt = t / tiles_m;
-  }
-  const int m0 = mt * BM, n0 = nt * BN;
+  const int total = tiles_m * tiles_n;
+  const int chunk_tiles = (total + 7) >> 3;
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, slots = gridDim.x >> 3;
+  const int range_end = min((xcd + 1) * chunk_tiles, total);
+  const bool blocked = (tiles_m & 7) == 0 && (tiles_n & 3) == 0;
+  auto tile_coords = [&](int t, int& m0, int& n0) {
+    int mt, nt;
+    if (blocked) {
+      const int sb = t >> 5, w = t & 31;
+      mt = (sb % (tiles_m >> 3)) * 8 + (w & 7);
+      nt = (sb / (tiles_m >> 3)) * 4 + (w >> 3);
+    } else {
+      mt = t % tiles_m;
+      nt = t / tiles_m;
+    }
+    m0 = mt * BM;
+    n0 = nt * BN;
+  };
+  const int first_tile = xcd * chunk_tiles + slot;
+  if (first_tile >= range_end) return;
+  const int my_tiles = (range_end - first_tile + slots - 1) / slots;
+
   const int nk = p.k >> 7;
   const int sf_tiles_k = (p.k >> 5) >> 2;  // 512-byte scale tiles per 128-row tile (K % 128 == 0)
 
   // ---- LDS-direct load addressing.  Wave w issues 8 loads per operand per K step; load j covers LDS
   // units [(w*8+j)*64, +64) = rows (w*8+j)*8 .. +7; lane L lands at unit +L, i.e. row +(L>>3), chunk
   // position L&7, which must hold global chunk (L&7) ^ ((row>>1)&7) = (L&7) ^ ((L>>4) | ((j&1)<<2)).
-  const uint8_t* a_tile = p.a + ((int64_t)m0 + wave * 64) * p.k;  // uniform
-  const uint8_t* b_tile = p.b + ((int64_t)n0 + wave * 64) * p.k;
   const uint32_t row_off = (uint32_t)(lane >> 3) * (uint32_t)p.k;
   const uint32_t voff_even = row_off + (uint32_t)(((lane & 7) ^ (lane >> 4)) << 4);
   const uint32_t voff_odd = row_off + (uint32_t)(((lane & 7) ^ ((lane >> 4) | 4)) << 4);
   const uint32_t lds_base = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)lds);
   const uint32_t step8 = 8u * (uint32_t)p.k;  // 8 rows
 
-  auto issue_tile_loads = [&](int ks, int buf) {
+  // ---- load stream state: the (tile, K step) the next loads are issued for
+  int l_tile = first_tile, l_ks = 0, l_count = 0;  // l_count: steps issued so far
+  const int total_steps = my_tiles * nk;
+  const uint8_t *l_a, *l_b, *l_sa, *l_sb;  // all wave-uniform
+  const uint32_t sc_lane_off = (uint32_t)li * 16u;
+  auto set_load_tile = [&](int t) {
+    int m0, n0;
+    tile_coords(t, m0, n0);
+    l_a = p.a + ((int64_t)m0 + wave * 64) * p.k;  // uniform
+    l_b = p.b + ((int64_t)n0 + wave * 64) * p.k;
+    // one 16-byte scale load per lane per K step: rows {li, li+32, li+64, li+96} of the wave's 128-row
+    // scale tile x 4 K-blocks
+    l_sa = p.sfa + ((int64_t)((m0 >> 7) + wm) * sf_tiles_k) * 512;
+    l_sb = p.sfb + ((int64_t)((n0 >> 7) + wn) * sf_tiles_k) * 512;
+  };
+  set_load_tile(l_tile);
+  u32x4 sc_la, sc_lb;  // scales in flight (for step l_count - 1)
+  auto issue_step_loads = [&]() {
+    if (l_count >= total_steps) return;
+    const int buf = l_count & 1;
     const uint32_t la = lds_base + (uint32_t)(buf * BUF_UNITS + wave * 512) * 16u;
     const uint32_t lb = la + TILE_UNITS * 16u;
-    const uint8_t* ga = a_tile + ((int64_t)ks << 7);
-    const uint8_t* gb = b_tile + ((int64_t)ks << 7);
+    const uint8_t* ga = l_a + ((int64_t)l_ks << 7);
+    const uint8_t* gb = l_b + ((int64_t)l_ks << 7);
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const uint32_t v = ((j & 1) ? voff_odd : voff_even) + (uint32_t)j * step8;
       lds_dma16(la + j * 1024u, ga, v);
       lds_dma16(lb + j * 1024u, gb, v);
     }
-  };
-  // ---- scales: one 16-byte load per lane per K step = rows {li, li+32, li+64, li+96} of the wave's
-  // 128-row scale tile x 4 K-blocks
-  const uint8_t* psa = p.sfa + ((int64_t)((m0 >> 7) + wm) * sf_tiles_k) * 512 + li * 16;
-  const uint8_t* psb = p.sfb + ((int64_t)((n0 >> 7) + wn) * sf_tiles_k) * 512 + li * 16;
-  auto load_scales = [&](int ks, u32x4& wa, u32x4& wb) {
-    wa = *reinterpret_cast<const u32x4*>(psa + (int64_t)ks * 512);
-    wb = *reinterpret_cast<const u32x4*>(psb + (int64_t)ks * 512);
+    sc_la = *reinterpret_cast<const u32x4*>(l_sa + (int64_t)l_ks * 512 + sc_lane_off);
+    sc_lb = *reinterpret_cast<const u32x4*>(l_sb + (int64_t)l_ks * 512 + sc_lane_off);
+    ++l_count;
+    if (++l_ks == nk) {
+      l_ks = 0;
+      l_tile += slots;
+      if (l_count < total_steps) set_load_tile(l_tile);
+    }
   };
   auto load_frags = [&](int buf, int sub, i32x8 (&fa)[4], i32x8 (&fb)[4]) {
     const u32x4* la = lds + buf * BUF_UNITS;
@@ -300,25 +327,15 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
   };
 
   f32x16 acc[4][4];
+  auto zero_acc = [&]() {
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+      for (int j = 0; j < 4; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
-
-  i32x8 fa0[4], fb0[4], fa1[4], fb1[4];
-  u32x4 sca, scb, sca_n, scb_n;
-
-  issue_tile_loads(0, 0);
-  if (nk > 1) issue_tile_loads(1, 1);
-  load_scales(0, sca, scb);
-  sca_n = sca; scb_n = scb;
-  if (nk > 1) load_scales(1, sca_n, scb_n);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __builtin_amdgcn_s_barrier();
-  load_frags(0, 0, fa0, fb0);
-  const int sh = lg * 8;  // lane group 1 supplies K-blocks 1 and 3 of a step
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+  };
+  zero_acc();
 
   // Keeps the 16 accumulator tiles "used" at this point of the program, so that the MFMAs producing
   // them cannot be moved past the statement that follows (they have no side effects of their own).
@@ -330,56 +347,75 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
                  "+a"(acc[3][1]), "+a"(acc[3][2]), "+a"(acc[3][3]));                                           \
   } while (0)
 
-  for (int ks = 0; ks < nk; ++ks) {
-    const int buf = ks & 1;
-    u32x4 wa, wb;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) { wa[i] = sca[i] >> sh; wb[i] = scb[i] >> sh; }
-    load_frags(buf, 1, fa1, fb1);
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb0[j], fa0[i], acc[i][j], 0, 0, 0, (int)wb[j], 0, (int)wa[i]);
-    NVF_PIN_ACC();
-    // Everything this wave loaded into buf^1 has landed, and its reads of buf are complete; after the
-    // barrier that holds for every wave, so buf^1 may be read and buf may be overwritten.
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-    load_frags(buf ^ 1, 0, fa0, fb0);  // on the last step this reads stale data that is never used
-    if (ks + 2 < nk) issue_tile_loads(ks + 2, buf);
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb1[j], fa1[i], acc[i][j], 0, 0, 2, (int)wb[j], 2, (int)wa[i]);
-    NVF_PIN_ACC();
-    sca = sca_n; scb = scb_n;
-    if (ks + 2 < nk) load_scales(ks + 2, sca_n, scb_n);
-  }
-#undef NVF_PIN_ACC
-
   const float alpha = p.alpha[0];
-  uint16_t* out = static_cast<uint16_t*>(p.out);
+  const int sh = lg * 8;  // lane group 1 supplies K-blocks 1 and 3 of a step
+
+  i32x8 fa0[4], fb0[4], fa1[4], fb1[4];
+  u32x4 wa, wb;      // scales of the step being computed, shifted for this lane group
+  u32x4 na, nb;      // scales of the next step
+
+  issue_step_loads();  // step 0
+  na = sc_la; nb = sc_lb;
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int mrow = m0 + wm * 128 + i * 32 + li;
-    uint16_t* orow = out + (int64_t)mrow * p.n;
+  for (int i = 0; i < 4; ++i) { wa[i] = na[i] >> sh; wb[i] = nb[i] >> sh; }
+  issue_step_loads();  // step 1
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  load_frags(0, 0, fa0, fb0);
+
+  int g = 0;
+  for (int c_tile = first_tile; c_tile < range_end; c_tile += slots) {
+    for (int c_ks = 0; c_ks < nk; ++c_ks, ++g) {
+      const int buf = g & 1;
+      load_frags(buf, 1, fa1, fb1);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+      for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int rq = 0; rq < 4; ++rq) {
-        const int ncol = n0 + wn * 128 + j * 32 + rq * 8 + lg * 4;
-        u32x2 v;
-        v[0] = pack2(acc[i][j][rq * 4 + 0] * alpha, acc[i][j][rq * 4 + 1] * alpha, OUT_BF16);
-        v[1] = pack2(acc[i][j][rq * 4 + 2] * alpha, acc[i][j][rq * 4 + 3] * alpha, OUT_BF16);
-        *reinterpret_cast<u32x2*>(orow + ncol) = v;
+        for (int j = 0; j < 4; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb0[j], fa0[i], acc[i][j], 0, 0, 0, (int)wb[j], 0, (int)wa[i]);
+      NVF_PIN_ACC();
+      // Everything this wave loaded for step g+1 has landed and its reads of buf are complete; after
+      // the barrier that holds for every wave, so buf^1 may be read and buf may be overwritten.
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      na = sc_la; nb = sc_lb;              // scales of step g+1 (landed: covered by the wait above)
+      load_frags(buf ^ 1, 0, fa0, fb0);    // after the last step this reads stale data that is never used
+      issue_step_loads();                  // step g+2 -> buf, and its scales -> sc_la / sc_lb
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb1[j], fa1[i], acc[i][j], 0, 0, 2, (int)wb[j], 2, (int)wa[i]);
+      NVF_PIN_ACC();
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { wa[i] = na[i] >> sh; wb[i] = nb[i] >> sh; }
+    }
+    // ---- epilogue of this tile; the loads of the next tile's first two steps are already in flight.
+    // acc[i][j][r] = C[m = li][n = (r/4)*8 + lg*4 + r%4] of its 32x32 sub-tile.
+    int m0, n0;
+    tile_coords(c_tile, m0, n0);
+    uint16_t* out = static_cast<uint16_t*>(p.out);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      uint16_t* orow = out + (int64_t)(m0 + wm * 128 + i * 32 + li) * p.n + n0 + wn * 128 + lg * 4;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq) {
+          u32x2 v;
+          v[0] = pack2(acc[i][j][rq * 4 + 0] * alpha, acc[i][j][rq * 4 + 1] * alpha, OUT_BF16);
+          v[1] = pack2(acc[i][j][rq * 4 + 2] * alpha, acc[i][j][rq * 4 + 3] * alpha, OUT_BF16);
+          *reinterpret_cast<u32x2*>(orow + j * 32 + rq * 8) = v;
+        }
       }
     }
+    zero_acc();
   }
+#undef NVF_PIN_ACC
 }
 
 template <bool OUT_BF16>
@@ -393,7 +429,9 @@ int launch_fast(const Params& p, hipStream_t stream) {
     configured = true;
   }
   const int64_t tiles = (int64_t)(p.m / 256) * (p.n / 256);
-  hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(256), lds_bytes, stream, p);
+  const int cus = 256;
+  const unsigned grid = (unsigned)(tiles >= cus ? cus : ((tiles + 7) / 8) * 8);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_bytes, stream, p);
   return check_launch("mxfp8_gemm_256_kernel");
 }
 
