@@ -286,44 +286,41 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
   };
   set_load_tile(l_tile);
   u32x4 sc_la, sc_lb;  // scales in flight (for step l_count - 1)
-  auto issue_step_loads = [&]() {
-    if (l_count >= total_steps) return;
+  // Unit q (0..15) of a step's tile loads: operand q&1, rows (wave*8 + q/2)*8 .. +7.
+  // Past the end of the stream the last step is loaded again (into a buffer nobody reads any more), so
+  // that the hot loop stays free of branches.
+  auto issue_step_unit = [&](int q) {
     const int buf = l_count & 1;
-    const uint32_t la = lds_base + (uint32_t)(buf * BUF_UNITS + wave * 512) * 16u;
-    const uint32_t lb = la + TILE_UNITS * 16u;
-    const uint8_t* ga = l_a + ((int64_t)l_ks << 7);
-    const uint8_t* gb = l_b + ((int64_t)l_ks << 7);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const uint32_t v = ((j & 1) ? voff_odd : voff_even) + (uint32_t)j * step8;
-      lds_dma16(la + j * 1024u, ga, v);
-      lds_dma16(lb + j * 1024u, gb, v);
-    }
+    const int j = q >> 1;
+    const uint32_t l = lds_base + (uint32_t)(buf * BUF_UNITS + (q & 1) * TILE_UNITS + wave * 512) * 16u + j * 1024u;
+    const uint8_t* gp = ((q & 1) ? l_b : l_a) + ((int64_t)l_ks << 7);
+    lds_dma16(l, gp, ((j & 1) ? voff_odd : voff_even) + (uint32_t)j * step8);
+  };
+  // After the 16 units: the step's scale loads, then advance the stream.
+  auto issue_step_tail = [&]() {
     sc_la = *reinterpret_cast<const u32x4*>(l_sa + (int64_t)l_ks * 512 + sc_lane_off);
     sc_lb = *reinterpret_cast<const u32x4*>(l_sb + (int64_t)l_ks * 512 + sc_lane_off);
     ++l_count;
-    if (++l_ks == nk) {
+    if (l_ks + 1 < nk) {
+      ++l_ks;
+    } else if (l_count < total_steps) {
       l_ks = 0;
       l_tile += slots;
-      if (l_count < total_steps) set_load_tile(l_tile);
+      set_load_tile(l_tile);
     }
   };
-  auto load_frags = [&](int buf, int sub, i32x8 (&fa)[4], i32x8 (&fb)[4]) {
-    const u32x4* la = lds + buf * BUF_UNITS;
-    const u32x4* lb = la + TILE_UNITS;
-    const int c_lo = sub * 4 + lg, c_hi = c_lo + 2;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int row = wm * 128 + i * 32 + li;
-      const u32x4 lo = la[lds_pos2(row, c_lo)], hi = la[lds_pos2(row, c_hi)];
-      fa[i] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
-    }
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int row = wn * 128 + j * 32 + li;
-      const u32x4 lo = lb[lds_pos2(row, c_lo)], hi = lb[lds_pos2(row, c_hi)];
-      fb[j] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
-    }
+  // Fragment storage: [operand: 0 = A, 1 = B][sub-tile][half].  Unit q (0..15) of a half step is one
+  // ds_read_b128: operand q>>3, sub-tile (q>>1)&3, half q&1.
+  struct Frags { u32x4 h[2][4][2]; };
+  auto load_unit = [&](int buf, int sub, int q, Frags& f) {
+    const int op = q >> 3, t = (q >> 1) & 3, half = q & 1;
+    const u32x4* base = lds + buf * BUF_UNITS + op * TILE_UNITS;
+    const int row = (op ? wn : wm) * 128 + t * 32 + li;
+    f.h[op][t][half] = base[lds_pos2(row, sub * 4 + lg + 2 * half)];
+  };
+  auto frag = [&](const Frags& f, int op, int t) {
+    const u32x4 lo = f.h[op][t][0], hi = f.h[op][t][1];
+    return i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
   };
 
   f32x16 acc[4][4];
@@ -350,46 +347,57 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
   const float alpha = p.alpha[0];
   const int sh = lg * 8;  // lane group 1 supplies K-blocks 1 and 3 of a step
 
-  i32x8 fa0[4], fb0[4], fa1[4], fb1[4];
+  Frags f0, f1;      // fragments of the first / second half (K 0..63 / 64..127) of a step
   u32x4 wa, wb;      // scales of the step being computed, shifted for this lane group
   u32x4 na, nb;      // scales of the next step
 
-  issue_step_loads();  // step 0
+#pragma unroll
+  for (int q = 0; q < 16; ++q) issue_step_unit(q);  // step 0
+  issue_step_tail();
   na = sc_la; nb = sc_lb;
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
   for (int i = 0; i < 4; ++i) { wa[i] = na[i] >> sh; wb[i] = nb[i] >> sh; }
-  issue_step_loads();  // step 1
+#pragma unroll
+  for (int q = 0; q < 16; ++q) issue_step_unit(q);  // step 1
+  issue_step_tail();
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
-  load_frags(0, 0, fa0, fb0);
+#pragma unroll
+  for (int q = 0; q < 16; ++q) load_unit(0, 0, q, f0);
 
   int g = 0;
   for (int c_tile = first_tile; c_tile < range_end; c_tile += slots) {
     for (int c_ks = 0; c_ks < nk; ++c_ks, ++g) {
       const int buf = g & 1;
-      load_frags(buf, 1, fa1, fb1);
+      // ---- first half: MFMAs on f0, interleaved one-to-one with the LDS reads that fill f1
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb0[j], fa0[i], acc[i][j], 0, 0, 0, (int)wb[j], 0, (int)wa[i]);
+      for (int q = 0; q < 16; ++q) {
+        const int i = q >> 2, j = q & 3;
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(frag(f0, 1, j), frag(f0, 0, i), acc[i][j], 0, 0, 0, (int)wb[j], 0, (int)wa[i]);
+        load_unit(buf, 1, q, f1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
       NVF_PIN_ACC();
       // Everything this wave loaded for step g+1 has landed and its reads of buf are complete; after
       // the barrier that holds for every wave, so buf^1 may be read and buf may be overwritten.
       asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
       __builtin_amdgcn_s_barrier();
       asm volatile("" ::: "memory");
-      na = sc_la; nb = sc_lb;              // scales of step g+1 (landed: covered by the wait above)
-      load_frags(buf ^ 1, 0, fa0, fb0);    // after the last step this reads stale data that is never used
-      issue_step_loads();                  // step g+2 -> buf, and its scales -> sc_la / sc_lb
+      na = sc_la; nb = sc_lb;  // scales of step g+1 (landed: covered by the wait above)
+      // ---- second half: MFMAs on f1, interleaved with the LDS reads of the next step's f0 (from buf^1;
+      // after the last step they read stale data that is never used) and the loads of step g+2 into buf
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb1[j], fa1[i], acc[i][j], 0, 0, 2, (int)wb[j], 2, (int)wa[i]);
+      for (int q = 0; q < 16; ++q) {
+        const int i = q >> 2, j = q & 3;
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(frag(f1, 1, j), frag(f1, 0, i), acc[i][j], 0, 0, 2, (int)wb[j], 2, (int)wa[i]);
+        load_unit(buf ^ 1, 0, q, f0);
+        issue_step_unit(q);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      issue_step_tail();
       NVF_PIN_ACC();
 #pragma unroll
       for (int i = 0; i < 4; ++i) { wa[i] = na[i] >> sh; wb[i] = nb[i] >> sh; }
@@ -415,6 +423,7 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
     }
     zero_acc();
   }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no LDS-direct load may outlive the workgroup
 #undef NVF_PIN_ACC
 }
 
