@@ -10,6 +10,7 @@
 // (rows r, r+32, r+64, r+96) x (4 consecutive K-blocks): one 16-byte load per lane fetches every
 // scale a 128-row wave tile needs for a 128-deep K step.
 #include "nvf_internal.h"
+#include <cstdlib>
 
 namespace nvf {
 namespace {
@@ -28,6 +29,8 @@ struct Params {
   const float* alpha;
   void* out;
   int m, n, k;
+  int stag_mode = 0, stag_mul = 0;
+  unsigned long long* clk = nullptr;
 };
 
 __device__ __forceinline__ uint32_t pack2(float a, float b, bool out_bf16) {
@@ -217,7 +220,7 @@ __device__ __forceinline__ void lds_dma16(uint32_t lds_byte_addr, const uint8_t*
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_byte_addr), "v"(voff), "s"(base) : "memory");
 }
 
-template <bool OUT_BF16>
+template <bool OUT_BF16, int DBG = 0>
 __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) {
   constexpr int BM = 256, BN = 256;
   constexpr int TILE_UNITS = 2048;            // 16-byte units per operand tile (256 rows x 8 chunks)
@@ -255,7 +258,7 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
   };
   const int first_tile = xcd * chunk_tiles + slot;
   if (first_tile >= range_end) return;
-  const int my_tiles = (range_end - first_tile + slots - 1) / slots;
+  unsigned long long t_core0 = __builtin_readcyclecounter(), t_real0 = wall_clock64();
 
   const int nk = p.k >> 7;
   const int sf_tiles_k = (p.k >> 5) >> 2;  // 512-byte scale tiles per 128-row tile (K % 128 == 0)
@@ -270,44 +273,48 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
   const uint32_t step8 = 8u * (uint32_t)p.k;  // 8 rows
 
   // ---- load stream state: the (tile, K step) the next loads are issued for
-  int l_tile = first_tile, l_ks = 0, l_count = 0;  // l_count: steps issued so far
-  const int total_steps = my_tiles * nk;
-  const uint8_t *l_a, *l_b, *l_sa, *l_sb;  // all wave-uniform
-  const uint32_t sc_lane_off = (uint32_t)li * 16u;
-  auto set_load_tile = [&](int t) {
+  // ---- load stream: the loads of step g+2 are issued while step g is computed, so the stream runs
+  // ahead of the compute loop and crosses into the next tile two steps early.  All of its state is
+  // wave-uniform and it advances without branches (the next tile's base pointers are prepared at the
+  // top of the tile loop), so that the hot loop stays one basic block.
+  struct TilePtrs { const uint8_t *a, *b, *sa, *sb; };
+  auto tile_ptrs = [&](int t) {
     int m0, n0;
     tile_coords(t, m0, n0);
-    l_a = p.a + ((int64_t)m0 + wave * 64) * p.k;  // uniform
-    l_b = p.b + ((int64_t)n0 + wave * 64) * p.k;
+    TilePtrs r;
+    r.a = p.a + ((int64_t)m0 + wave * 64) * p.k;
+    r.b = p.b + ((int64_t)n0 + wave * 64) * p.k;
     // one 16-byte scale load per lane per K step: rows {li, li+32, li+64, li+96} of the wave's 128-row
     // scale tile x 4 K-blocks
-    l_sa = p.sfa + ((int64_t)((m0 >> 7) + wm) * sf_tiles_k) * 512;
-    l_sb = p.sfb + ((int64_t)((n0 >> 7) + wn) * sf_tiles_k) * 512;
+    r.sa = p.sfa + ((int64_t)((m0 >> 7) + wm) * sf_tiles_k) * 512;
+    r.sb = p.sfb + ((int64_t)((n0 >> 7) + wn) * sf_tiles_k) * 512;
+    return r;
   };
-  set_load_tile(l_tile);
+  TilePtrs lp = tile_ptrs(first_tile);  // tile the stream is in
+  TilePtrs np = lp;                     // tile it enters next
+  int l_ks = 0, l_count = 0;            // K step inside lp; steps issued so far
+  const uint32_t sc_lane_off = (uint32_t)li * 16u;
   u32x4 sc_la, sc_lb;  // scales in flight (for step l_count - 1)
-  // Unit q (0..15) of a step's tile loads: operand q&1, rows (wave*8 + q/2)*8 .. +7.
-  // Past the end of the stream the last step is loaded again (into a buffer nobody reads any more), so
-  // that the hot loop stays free of branches.
+  // Unit q (0..15) of a step's tile loads: operand q&1, rows (wave*8 + q/2)*8 .. +7.  Past the end of
+  // the stream the last tile is loaded again (into a buffer nobody reads any more).
   auto issue_step_unit = [&](int q) {
     const int buf = l_count & 1;
     const int j = q >> 1;
     const uint32_t l = lds_base + (uint32_t)(buf * BUF_UNITS + (q & 1) * TILE_UNITS + wave * 512) * 16u + j * 1024u;
-    const uint8_t* gp = ((q & 1) ? l_b : l_a) + ((int64_t)l_ks << 7);
+    const uint8_t* gp = ((q & 1) ? lp.b : lp.a) + ((int64_t)l_ks << 7);
     lds_dma16(l, gp, ((j & 1) ? voff_odd : voff_even) + (uint32_t)j * step8);
   };
-  // After the 16 units: the step's scale loads, then advance the stream.
+  // After the 16 units: the step's scale loads, then advance the stream (selects only).
   auto issue_step_tail = [&]() {
-    sc_la = *reinterpret_cast<const u32x4*>(l_sa + (int64_t)l_ks * 512 + sc_lane_off);
-    sc_lb = *reinterpret_cast<const u32x4*>(l_sb + (int64_t)l_ks * 512 + sc_lane_off);
+    sc_la = *reinterpret_cast<const u32x4*>(lp.sa + (int64_t)l_ks * 512 + sc_lane_off);
+    sc_lb = *reinterpret_cast<const u32x4*>(lp.sb + (int64_t)l_ks * 512 + sc_lane_off);
     ++l_count;
-    if (l_ks + 1 < nk) {
-      ++l_ks;
-    } else if (l_count < total_steps) {
-      l_ks = 0;
-      l_tile += slots;
-      set_load_tile(l_tile);
-    }
+    const bool wrap = (l_ks + 1 == nk);
+    l_ks = wrap ? 0 : l_ks + 1;
+    lp.a = wrap ? np.a : lp.a;
+    lp.b = wrap ? np.b : lp.b;
+    lp.sa = wrap ? np.sa : lp.sa;
+    lp.sb = wrap ? np.sb : lp.sb;
   };
   // Fragment storage: [operand: 0 = A, 1 = B][sub-tile][half].  Unit q (0..15) of a half step is one
   // ds_read_b128: operand q>>3, sub-tile (q>>1)&3, half q&1.
@@ -368,6 +375,8 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
 
   int g = 0;
   for (int c_tile = first_tile; c_tile < range_end; c_tile += slots) {
+    // the stream is inside this tile by now; prepare the tile it will enter two steps before the end
+    np = (c_tile + slots < range_end) ? tile_ptrs(c_tile + slots) : lp;
     for (int c_ks = 0; c_ks < nk; ++c_ks, ++g) {
       const int buf = g & 1;
       // ---- first half: MFMAs on f0, interleaved one-to-one with the LDS reads that fill f1
@@ -375,29 +384,33 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
 #pragma unroll
       for (int q = 0; q < 16; ++q) {
         const int i = q >> 2, j = q & 3;
+        if (!(DBG & 2)) load_unit(buf, 1, q, f1);
         acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(frag(f0, 1, j), frag(f0, 0, i), acc[i][j], 0, 0, 0, (int)wb[j], 0, (int)wa[i]);
-        load_unit(buf, 1, q, f1);
         __builtin_amdgcn_sched_barrier(0);
       }
       NVF_PIN_ACC();
       // Everything this wave loaded for step g+1 has landed and its reads of buf are complete; after
       // the barrier that holds for every wave, so buf^1 may be read and buf may be overwritten.
+      if (!(DBG & 4)) {
       asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
       __builtin_amdgcn_s_barrier();
-      asm volatile("" ::: "memory");
-      na = sc_la; nb = sc_lb;  // scales of step g+1 (landed: covered by the wait above)
+      }
+      // The scale words of step g+1 are consumed here and nowhere earlier: their load is covered by the
+      // wait above, and any wait placed before it would also stall on the tile loads just issued.
+      asm volatile("" : "+v"(sc_la), "+v"(sc_lb) : : "memory");
+      na = sc_la; nb = sc_lb;
       // ---- second half: MFMAs on f1, interleaved with the LDS reads of the next step's f0 (from buf^1;
       // after the last step they read stale data that is never used) and the loads of step g+2 into buf
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int q = 0; q < 16; ++q) {
         const int i = q >> 2, j = q & 3;
+        if (!(DBG & 2)) load_unit(buf ^ 1, 0, q, f0);
+        if (!(DBG & 1)) issue_step_unit(q);
+        if (q == 15) issue_step_tail();  // scalar bookkeeping in the shadow of the MFMAs already queued
         acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(frag(f1, 1, j), frag(f1, 0, i), acc[i][j], 0, 0, 2, (int)wb[j], 2, (int)wa[i]);
-        load_unit(buf ^ 1, 0, q, f0);
-        issue_step_unit(q);
         __builtin_amdgcn_sched_barrier(0);
       }
-      issue_step_tail();
       NVF_PIN_ACC();
 #pragma unroll
       for (int i = 0; i < 4; ++i) { wa[i] = na[i] >> sh; wb[i] = nb[i] >> sh; }
@@ -424,12 +437,24 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
     zero_acc();
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no LDS-direct load may outlive the workgroup
+  if (p.clk && tid == 0) { p.clk[blockIdx.x * 2] = __builtin_readcyclecounter() - t_core0; p.clk[blockIdx.x * 2 + 1] = wall_clock64() - t_real0; }
 #undef NVF_PIN_ACC
 }
 
 template <bool OUT_BF16>
 int launch_fast(const Params& p, hipStream_t stream) {
   auto kern = mxfp8_gemm_256_kernel<OUT_BF16>;
+  if (const char* d = getenv("NVF_DBG")) {
+    switch (atoi(d)) {
+      case 1: kern = mxfp8_gemm_256_kernel<OUT_BF16, 1>; break;
+      case 2: kern = mxfp8_gemm_256_kernel<OUT_BF16, 2>; break;
+      case 3: kern = mxfp8_gemm_256_kernel<OUT_BF16, 3>; break;
+      case 4: kern = mxfp8_gemm_256_kernel<OUT_BF16, 4>; break;
+      case 5: kern = mxfp8_gemm_256_kernel<OUT_BF16, 5>; break;
+      case 7: kern = mxfp8_gemm_256_kernel<OUT_BF16, 7>; break;
+    }
+    hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 131072);
+  }
   constexpr int lds_bytes = 2 * 2 * 2048 * 16;  // 128 KiB
   static bool configured = false;
   if (!configured) {
@@ -437,10 +462,13 @@ int launch_fast(const Params& p, hipStream_t stream) {
     if (e != hipSuccess) return fail(NVF_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
     configured = true;
   }
+  Params q = p;
+  if (const char* e = getenv("NVF_CLKBUF")) q.clk = (unsigned long long*)strtoull(e, nullptr, 16);
+  if (const char* e = getenv("NVF_STAG")) { q.stag_mode = e[0] == 'A' ? 1 : 2; q.stag_mul = atoi(e + 1); }
   const int64_t tiles = (int64_t)(p.m / 256) * (p.n / 256);
   const int cus = 256;
   const unsigned grid = (unsigned)(tiles >= cus ? cus : ((tiles + 7) / 8) * 8);
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_bytes, stream, p);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_bytes, stream, q);
   return check_launch("mxfp8_gemm_256_kernel");
 }
 
@@ -462,7 +490,7 @@ int launch_cfg(const Params& p, hipStream_t stream) {
 template <bool OUT_BF16>
 int launch_sized(const Params& p, hipStream_t stream) {
   auto tiles = [&](int bm, int bn) { return ceil_div(p.m, bm) * ceil_div(p.n, bn); };
-  if (tiles(256, 256) >= 128 && (p.k & 127) == 0 && (p.m & 255) == 0 && (p.n & 255) == 0 && (int64_t)p.k * 256 < (1ll << 31))
+  if (tiles(256, 256) >= 128 && (p.k & 127) == 0 && p.k >= 256 && (p.m & 255) == 0 && (p.n & 255) == 0 && (int64_t)p.k * 256 < (1ll << 31))
     return launch_fast<OUT_BF16>(p, stream);
   if (tiles(256, 256) >= 256) return launch_cfg<256, 256, OUT_BF16>(p, stream);
   if (tiles(128, 128) >= 256) return launch_cfg<128, 128, OUT_BF16>(p, stream);
