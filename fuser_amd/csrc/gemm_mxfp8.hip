@@ -10,7 +10,6 @@
 // (rows r, r+32, r+64, r+96) x (4 consecutive K-blocks): one 16-byte load per lane fetches every
 // scale a 128-row wave tile needs for a 128-deep K step.
 #include "nvf_internal.h"
-#include <cstdlib>
 
 namespace nvf {
 namespace {
@@ -29,8 +28,6 @@ struct Params {
   const float* alpha;
   void* out;
   int m, n, k;
-  int stag_mode = 0, stag_mul = 0;
-  unsigned long long* clk = nullptr;
 };
 
 __device__ __forceinline__ uint32_t pack2(float a, float b, bool out_bf16) {
@@ -220,7 +217,7 @@ __device__ __forceinline__ void lds_dma16(uint32_t lds_byte_addr, const uint8_t*
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_byte_addr), "v"(voff), "s"(base) : "memory");
 }
 
-template <bool OUT_BF16, int DBG = 0>
+template <bool OUT_BF16>
 __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) {
   constexpr int BM = 256, BN = 256;
   constexpr int TILE_UNITS = 2048;            // 16-byte units per operand tile (256 rows x 8 chunks)
@@ -258,7 +255,6 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
   };
   const int first_tile = xcd * chunk_tiles + slot;
   if (first_tile >= range_end) return;
-  unsigned long long t_core0 = __builtin_readcyclecounter(), t_real0 = wall_clock64();
 
   const int nk = p.k >> 7;
   const int sf_tiles_k = (p.k >> 5) >> 2;  // 512-byte scale tiles per 128-row tile (K % 128 == 0)
@@ -384,17 +380,15 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
 #pragma unroll
       for (int q = 0; q < 16; ++q) {
         const int i = q >> 2, j = q & 3;
-        if (!(DBG & 2)) load_unit(buf, 1, q, f1);
+        load_unit(buf, 1, q, f1);
         acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(frag(f0, 1, j), frag(f0, 0, i), acc[i][j], 0, 0, 0, (int)wb[j], 0, (int)wa[i]);
         __builtin_amdgcn_sched_barrier(0);
       }
       NVF_PIN_ACC();
       // Everything this wave loaded for step g+1 has landed and its reads of buf are complete; after
       // the barrier that holds for every wave, so buf^1 may be read and buf may be overwritten.
-      if (!(DBG & 4)) {
       asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
       __builtin_amdgcn_s_barrier();
-      }
       // The scale words of step g+1 are consumed here and nowhere earlier: their load is covered by the
       // wait above, and any wait placed before it would also stall on the tile loads just issued.
       asm volatile("" : "+v"(sc_la), "+v"(sc_lb) : : "memory");
@@ -405,8 +399,8 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
 #pragma unroll
       for (int q = 0; q < 16; ++q) {
         const int i = q >> 2, j = q & 3;
-        if (!(DBG & 2)) load_unit(buf ^ 1, 0, q, f0);
-        if (!(DBG & 1)) issue_step_unit(q);
+        load_unit(buf ^ 1, 0, q, f0);
+        issue_step_unit(q);
         if (q == 15) issue_step_tail();  // scalar bookkeeping in the shadow of the MFMAs already queued
         acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(frag(f1, 1, j), frag(f1, 0, i), acc[i][j], 0, 0, 2, (int)wb[j], 2, (int)wa[i]);
         __builtin_amdgcn_sched_barrier(0);
@@ -437,24 +431,12 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
     zero_acc();
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no LDS-direct load may outlive the workgroup
-  if (p.clk && tid == 0) { p.clk[blockIdx.x * 2] = __builtin_readcyclecounter() - t_core0; p.clk[blockIdx.x * 2 + 1] = wall_clock64() - t_real0; }
 #undef NVF_PIN_ACC
 }
 
 template <bool OUT_BF16>
 int launch_fast(const Params& p, hipStream_t stream) {
   auto kern = mxfp8_gemm_256_kernel<OUT_BF16>;
-  if (const char* d = getenv("NVF_DBG")) {
-    switch (atoi(d)) {
-      case 1: kern = mxfp8_gemm_256_kernel<OUT_BF16, 1>; break;
-      case 2: kern = mxfp8_gemm_256_kernel<OUT_BF16, 2>; break;
-      case 3: kern = mxfp8_gemm_256_kernel<OUT_BF16, 3>; break;
-      case 4: kern = mxfp8_gemm_256_kernel<OUT_BF16, 4>; break;
-      case 5: kern = mxfp8_gemm_256_kernel<OUT_BF16, 5>; break;
-      case 7: kern = mxfp8_gemm_256_kernel<OUT_BF16, 7>; break;
-    }
-    hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 131072);
-  }
   constexpr int lds_bytes = 2 * 2 * 2048 * 16;  // 128 KiB
   static bool configured = false;
   if (!configured) {
@@ -462,13 +444,10 @@ int launch_fast(const Params& p, hipStream_t stream) {
     if (e != hipSuccess) return fail(NVF_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
     configured = true;
   }
-  Params q = p;
-  if (const char* e = getenv("NVF_CLKBUF")) q.clk = (unsigned long long*)strtoull(e, nullptr, 16);
-  if (const char* e = getenv("NVF_STAG")) { q.stag_mode = e[0] == 'A' ? 1 : 2; q.stag_mul = atoi(e + 1); }
   const int64_t tiles = (int64_t)(p.m / 256) * (p.n / 256);
   const int cus = 256;
   const unsigned grid = (unsigned)(tiles >= cus ? cus : ((tiles + 7) / 8) * 8);
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_bytes, stream, q);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_bytes, stream, p);
   return check_launch("mxfp8_gemm_256_kernel");
 }
 

@@ -173,6 +173,24 @@ def test_mxfp8_gemm_ragged_shapes_alpha_and_scale_spread(dev, shape):
         assert err <= GEMM_MAX_REL, (shape, dtype, err)
 
 
+@pytest.mark.parametrize("shape", [(4096, 2048, 512), (2560, 3328, 384), (2048, 4096, 256), (8192, 1024, 1152)])
+def test_mxfp8_gemm_persistent_256_tile_kernel_full_compare(dev, shape):
+    """Shapes with M % 256 == N % 256 == K % 128 == 0 and at least 128 tiles take the persistent
+    LDS-direct kernel; every output element is compared with the oracle.  (2560, 3328) has a tile grid
+    that is not a multiple of the 8 x 4 blocking, (8192, 1024) gives some workgroups two tiles and K
+    steps that wrap the load stream across tiles."""
+    m, n, k = shape
+    gen = torch.Generator().manual_seed(k)
+    a, sa = _mxfp8_operand(m, k, gen, 1.0)
+    b, sb = _mxfp8_operand(n, k, gen, 1.0)
+    ref = O.ref_mxfp8_scaled_mm(a, b, sa, sb, 1.5)
+    out = _run_mxfp8(a, b, sa, sb, 1.5, torch.bfloat16, dev)
+    scale = ref.abs().amax(dim=1, keepdim=True).clamp(min=1e-30)
+    assert ((out.float().cpu() - ref).abs() / scale).max().item() <= GEMM_MAX_REL
+    out2 = _run_mxfp8(a, b, sa, sb, 1.5, torch.bfloat16, dev)
+    assert torch.equal(out, out2)
+
+
 def test_mxfp8_gemm_8192_cubed_sampled_against_oracle(dev):
     """BASELINE config 2 at full size.  The CPU oracle is applied to a sample of output rows/columns;
     determinism and the K-split additivity property are checked on the whole output."""
