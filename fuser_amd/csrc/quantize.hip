@@ -1,15 +1,11 @@
-// NVFP4 / MXFP8 block quantizers for gfx950: one HBM pass, 16-byte coalesced loads, amax reduced
-// across lanes with DPP, packed payload and block scales written in place (linear, 128x4 swizzled,
-// or per-group padded 128x4).
+// NVFP4 / MXFP8 block quantizers for gfx950: one HBM pass, 16-byte loads, packed payload and block
+// scales written in place (linear, 128x4 swizzled, or per-group padded 128x4).
 //
 // Semantics restated from runtime/block_quantization_kernels.cu:142-186 (MXFP8), :194-319 (NVFP4),
 // :321-361 (scale-layout copy), :363-413 (grouped NVFP4) and the casts of runtime/casts.cu.
 //
-// Work decomposition (all kernels): a wavefront owns one row segment of 512 consecutive elements,
-// lane l holding elements [8l, 8l+8) -> a 1 KiB contiguous read and a 256 B (fp4) / 512 B (fp8)
-// contiguous payload write per wavefront.  A 256-thread workgroup walks a band of 32*ROW_ITERS rows;
-// with ROW_ITERS == 4 a lane visits rows r, r+32, r+64, r+96 so that the four scale words it
-// gathers are the 16 contiguous bytes the 128x4 layout gives those rows.
+// Work decomposition: a wavefront owns one row segment of 1024 elements, 16 per lane (one NVFP4 block,
+// half an MXFP8 block); a workgroup is 4 consecutive rows of one segment; details at each kernel.
 #include "nvf_internal.h"
 
 #include <cfloat>
@@ -19,9 +15,7 @@ namespace {
 
 enum { LAYOUT_LINEAR = 0, LAYOUT_SWIZZLED = 1, LAYOUT_GROUPED = 2 };
 
-constexpr int kSegCols = 512;  // elements per wavefront row segment
-
-// lane i <- lane i^1 / i^2 within a quad, lane i <- lane i+4 / i+8 within a row of 16
+// lane i <- lane i^1 / i^2 within a quad, lane i <- lane i+4 within a row of 16
 __device__ __forceinline__ uint32_t dpp_xor1(uint32_t v) {
   return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xf, 0xf, true);  // quad_perm [1,0,3,2]
 }
@@ -31,55 +25,12 @@ __device__ __forceinline__ uint32_t dpp_xor2(uint32_t v) {
 __device__ __forceinline__ uint32_t dpp_shl4(uint32_t v) {
   return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x104, 0xf, 0xf, true);  // row_shl:4
 }
-__device__ __forceinline__ uint32_t dpp_shl8(uint32_t v) {
-  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x108, 0xf, 0xf, true);  // row_shl:8
-}
 
-// ---- loading 8 consecutive elements as fp32, with a cheap "contains Inf or NaN" flag ----
 struct bf16_t { uint16_t v; };
 struct f16_t { uint16_t v; };
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
-
-__device__ __forceinline__ void load8(const bf16_t* p, float x[8], bool& nan) {
-  const u32x4 u = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
-  uint32_t f = 0;
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    x[2 * j] = bits_to_f32(u[j] << 16);
-    x[2 * j + 1] = bits_to_f32(u[j] & 0xffff0000u);
-    f |= ((u[j] & 0x7fff7fffu) + 0x00800080u);  // bit 15 / 31 set <=> that half is Inf or NaN
-  }
-  nan = (f & 0x80008000u) != 0;
-}
-__device__ __forceinline__ void load8(const f16_t* p, float x[8], bool& nan) {
-  const u32x4 u = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
-  uint32_t f = 0;
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    x[2 * j] = (float)__builtin_bit_cast(_Float16, (uint16_t)(u[j] & 0xffffu));
-    x[2 * j + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(u[j] >> 16));
-    f |= ((u[j] & 0x7fff7fffu) + 0x04000400u);
-  }
-  nan = (f & 0x80008000u) != 0;
-}
-__device__ __forceinline__ void load8(const float* p, float x[8], bool& nan) {
-  const f32x4 a = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p));
-  const f32x4 b = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p) + 1);
-#pragma unroll
-  for (int j = 0; j < 4; ++j) { x[j] = a[j]; x[4 + j] = b[j]; }
-  nan = false;
-#pragma unroll
-  for (int j = 0; j < 8; ++j) nan |= !(fabsf(x[j]) < INFINITY);
-}
-
-// amax of 8 values, NaN ignored (fmaxf), start -inf: block_quantization_kernels.cu:124-128
-__device__ __forceinline__ float amax8(const float x[8]) {
-  float m = -INFINITY;
-#pragma unroll
-  for (int j = 0; j < 8; ++j) m = fmaxf(m, fabsf(x[j]));
-  return m;
-}
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 // last group g with offsets[g] <= row (what the reference's linear scan returns for sorted offsets)
 __device__ __forceinline__ int find_group(const int32_t* __restrict__ offsets, int groups, int64_t row) {
@@ -92,232 +43,285 @@ __device__ __forceinline__ int find_group(const int32_t* __restrict__ offsets, i
 }
 
 // -------------------------------------------------------------------------------------------------
-// NVFP4
+// NVFP4: one lane quantizes one 16-element block.
+//   * A wavefront owns a row segment of 1024 elements; lane l loads elements [16l, 16l+16) with 16-byte
+//     loads (two for 16-bit inputs, four for fp32), so a wavefront reads 2 KiB contiguous and writes
+//     512 contiguous payload bytes; no cross-lane reduction and no duplicated scale arithmetic.
+//   * A workgroup is 4 consecutive rows of one segment and lives for one such step: many short
+//     workgroups in row-major order keep the HBM stream close to linear (5.8 TB/s on 65536 x 7168 bf16,
+//     against 5.0 TB/s for workgroups that walk 128-row bands).
+//   * The scale bytes of 4 neighbouring lanes are merged into one dword with two DPP steps; the dwords
+//     of the 32 rows that share a 128-byte line of the 128x4 layout come from different workgroups and
+//     are merged by the caches before they reach HBM.
+//   * amax/6 and 1/x use a 3-instruction division (reciprocal constant resp. v_rcp_f32, one fused
+//     residual correction); for biased exponents in [2, 250] it returns exactly the IEEE quotient for
+//     every fp32 input (checked exhaustively on the GPU); anything else (zero, denormal, huge, Inf, NaN)
+//     makes the wavefront redo the block scale with true divisions.
 // -------------------------------------------------------------------------------------------------
-template <typename T, int LAYOUT, int ROW_ITERS>
+// 16 consecutive elements: the raw 16-byte loads are issued first and decoded to fp32 later, so that
+// address-independent work (group lookup, global scale) overlaps the memory latency. Inactive lanes load
+// from a valid dummy address and decode to zeros; `nonfinite` flags Inf or NaN among the 16.
+template <typename T>
+struct Raw16 {
+  u32x4 q[sizeof(T) * 2];
+};
+template <typename T>
+__device__ __forceinline__ Raw16<T> issue16(const T* p) {
+  Raw16<T> r;
+#pragma unroll
+  for (int q = 0; q < (int)sizeof(T) * 2; ++q) r.q[q] = *(reinterpret_cast<const u32x4*>(p) + q);
+  return r;
+}
+__device__ __forceinline__ void decode16(const Raw16<bf16_t>& r, bool active, float x[16], bool& nonfinite) {
+  const uint32_t mask = active ? 0xffffffffu : 0u;
+  uint32_t f = 0;
+#pragma unroll
+  for (int q = 0; q < 2; ++q) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t u = r.q[q][j] & mask;
+      x[8 * q + 2 * j] = bits_to_f32(u << 16);
+      x[8 * q + 2 * j + 1] = bits_to_f32(u & 0xffff0000u);
+      f |= (u & 0x7fff7fffu) + 0x00800080u;  // bit 15 / 31 set <=> that half is Inf or NaN
+    }
+  }
+  nonfinite = (f & 0x80008000u) != 0;
+}
+__device__ __forceinline__ void decode16(const Raw16<f16_t>& r, bool active, float x[16], bool& nonfinite) {
+  const uint32_t mask = active ? 0xffffffffu : 0u;
+  uint32_t f = 0;
+#pragma unroll
+  for (int q = 0; q < 2; ++q) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t u = r.q[q][j] & mask;
+      x[8 * q + 2 * j] = (float)__builtin_bit_cast(_Float16, (uint16_t)(u & 0xffffu));
+      x[8 * q + 2 * j + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(u >> 16));
+      f |= (u & 0x7fff7fffu) + 0x04000400u;
+    }
+  }
+  nonfinite = (f & 0x80008000u) != 0;
+}
+__device__ __forceinline__ void decode16(const Raw16<float>& r, bool active, float x[16], bool& nonfinite) {
+  const uint32_t mask = active ? 0xffffffffu : 0u;
+  nonfinite = false;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      x[4 * q + j] = bits_to_f32(r.q[q][j] & mask);
+      nonfinite |= !(fabsf(x[4 * q + j]) < INFINITY);
+    }
+  }
+}
+
+// true when the 3-instruction divisions below are exact for this operand
+__device__ __forceinline__ bool fast_div_ok(float v) { return ((f32_to_bits(v) >> 23) & 0xffu) - 2u <= 248u; }
+__device__ __forceinline__ float fast_div6(float m) {
+  const float r6 = 0x1.555556p-3f;  // RN(1/6)
+  const float q0 = m * r6;
+  return __builtin_fmaf(__builtin_fmaf(-6.0f, q0, m), r6, q0);
+}
+__device__ __forceinline__ float fast_rcp(float v) {
+  const float r0 = __builtin_amdgcn_rcpf(v);
+  return __builtin_fmaf(__builtin_fmaf(-v, r0, 1.0f), r0, r0);
+}
+
+constexpr int kSegCols = 1024;  // elements per wavefront row segment
+
+template <typename T, int LAYOUT>
 __global__ __launch_bounds__(256) void nvfp4_quantize_kernel(const T* __restrict__ in, int64_t rows, int64_t cols,
                                                              const float* __restrict__ gs_ptr,
                                                              const int32_t* __restrict__ in_off,
                                                              const int32_t* __restrict__ out_off, int groups,
-                                                             uint8_t* __restrict__ out_fp4,
+                                                             uint32_t segs, uint8_t* __restrict__ out_fp4,
                                                              uint8_t* __restrict__ out_sf) {
-  constexpr int kBandRows = 32 * ROW_ITERS;
+  // workgroup = 4 consecutive rows of one 1024-column segment; consecutive workgroups walk the segments
+  // of the same 4 rows, so the chip streams the input almost linearly
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const int64_t row0 = (int64_t)blockIdx.y * kBandRows;
-  const int64_t col = (int64_t)blockIdx.x * kSegCols + lane * 8;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t band = blockIdx.x / segs;
+  const uint32_t seg = blockIdx.x - band * segs;
+  const int64_t row = (int64_t)band * 4 + wave;
+  const int64_t col = (int64_t)seg * kSegCols + lane * 16;
   const bool col_ok = col < cols;
+  const bool active = col_ok && row < rows;
   const int64_t sf_cols = cols >> 4;
   const int64_t padded = (sf_cols + 3) & ~(int64_t)3;
   const int64_t sf_col = col >> 4;  // scale column of this lane's block
+  const bool word_scales = !(LAYOUT == LAYOUT_LINEAR && (sf_cols & 3) != 0);
+
+  const Raw16<T> raw = issue16(active ? in + row * cols + col : in);
 
   const bool use_gs = gs_ptr != nullptr;
   const float gs = use_gs ? *gs_ptr : 1.0f;
   const float decode = 1.0f / gs;  // :236
 
-  __shared__ int64_t row_sf_base[kBandRows];
+  int64_t sf_row_base = 0;  // byte offset of (row, scale column 0) in the scale buffer
   if constexpr (LAYOUT == LAYOUT_GROUPED) {
-    if (threadIdx.x < kBandRows) {
-      const int64_t r = row0 + threadIdx.x;
-      int64_t base = 0;
-      if (r < rows) {
-        const int g = find_group(in_off, groups, r);
-        base = (int64_t)out_off[g] * padded + swizzle_128x4(r - in_off[g], 0, padded);
-      }
-      row_sf_base[threadIdx.x] = base;
+    if (row < rows) {
+      // row is wavefront-uniform: the search runs on the scalar unit and its cache while the loads fly
+      const int g = find_group(in_off, groups, row);
+      sf_row_base = (int64_t)out_off[g] * padded + swizzle_128x4(row - in_off[g], 0, padded);
     }
-    __syncthreads();
+  } else if constexpr (LAYOUT == LAYOUT_SWIZZLED) {
+    sf_row_base = swizzle_128x4(row, 0, padded);  // rows past `rows` inside the last tile receive zeros
+  } else {
+    sf_row_base = row * sf_cols;
   }
 
-#pragma unroll 1
-  for (int t = 0; t < 8; ++t) {
-    const int rb = t * 4 + wave;  // row inside a 32-row group
-    uint32_t sfw[ROW_ITERS];
-    float x[ROW_ITERS][8];
-    bool nan = false;
-#pragma unroll
-    for (int i = 0; i < ROW_ITERS; ++i) {
-      const int64_t row = row0 + rb + 32 * i;
-      if (col_ok && row < rows) {
-        bool n;
-        load8(in + row * cols + col, x[i], n);
-        nan |= n;
-      } else {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) x[i][j] = 0.0f;
-      }
-    }
-    const bool wave_has_nan = __builtin_amdgcn_ballot_w64(nan) != 0;  // any non-finite input in the wavefront
+  float x[16];
+  bool nonfinite;
+  decode16(raw, active, x, nonfinite);
+  const bool wave_nonfinite = __builtin_amdgcn_ballot_w64(nonfinite) != 0;
 
+  // amax, NaN ignored (fmaxf), start -inf: block_quantization_kernels.cu:124-128
+  float m = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < ROW_ITERS; ++i) {
-      const int64_t row = row0 + rb + 32 * i;
-      float m = amax8(x[i]);
-      m = fmaxf(m, bits_to_f32(dpp_xor1(f32_to_bits(m))));  // the two lanes of a 16-element block
-      float s = m / 6.0f;                                    // :224
-      if (use_gs) s = s * gs;                                // :226
-      s = fminf(s, FLT_MAX);                                 // :228
-      const uint32_t q8 = f32_to_e4m3_satfinite(s);          // :230
-      const float sf = e4m3_to_f32(q8);                      // :233
-      const float r = use_gs ? fminf(1.0f / (sf * decode), FLT_MAX) : fminf(1.0f / sf, FLT_MAX);  // :237/:239
+  for (int j = 0; j < 16; ++j) m = fmaxf(m, fabsf(x[j]));
+  float s = fast_div6(m);                 // :224  amax / 6
+  if (use_gs) s = s * gs;                 // :226
+  s = fminf(s, FLT_MAX);                  // :228
+  uint32_t q8 = f32_to_e4m3_satfinite(s); // :230
+  float sf = e4m3_to_f32(q8);             // :233
+  float den = use_gs ? sf * decode : sf;  // :237 / :239
+  float r = fminf(fast_rcp(den), FLT_MAX);
+  if (__builtin_amdgcn_ballot_w64(active && (!fast_div_ok(m) || !fast_div_ok(den))) != 0) {
+    s = m / 6.0f;
+    if (use_gs) s = s * gs;
+    s = fminf(s, FLT_MAX);
+    q8 = f32_to_e4m3_satfinite(s);
+    sf = e4m3_to_f32(q8);
+    den = use_gs ? sf * decode : sf;
+    r = fminf(1.0f / den, FLT_MAX);
+  }
 
-      uint32_t p = 0;
-      if (!wave_has_nan) {
-        p = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(p, x[i][0] * r, x[i][1] * r, 1.0f, 0);
-        p = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(p, x[i][2] * r, x[i][3] * r, 1.0f, 1);
-        p = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(p, x[i][4] * r, x[i][5] * r, 1.0f, 2);
-        p = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(p, x[i][6] * r, x[i][7] * r, 1.0f, 3);
-      } else {
+  uint32_t p0 = 0, p1 = 0;
+  if (!wave_nonfinite) {
+    p0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(p0, x[0] * r, x[1] * r, 1.0f, 0);
+    p0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(p0, x[2] * r, x[3] * r, 1.0f, 1);
+    p0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(p0, x[4] * r, x[5] * r, 1.0f, 2);
+    p0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(p0, x[6] * r, x[7] * r, 1.0f, 3);
+    p1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(p1, x[8] * r, x[9] * r, 1.0f, 0);
+    p1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(p1, x[10] * r, x[11] * r, 1.0f, 1);
+    p1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(p1, x[12] * r, x[13] * r, 1.0f, 2);
+    p1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(p1, x[14] * r, x[15] * r, 1.0f, 3);
+  } else {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) p |= f32x2_to_e2m1_byte(x[i][2 * j] * r, x[i][2 * j + 1] * r) << (8 * j);
-      }
-      const bool active = col_ok && row < rows;
-      if (active) *reinterpret_cast<uint32_t*>(out_fp4 + ((row * cols + col) >> 1)) = p;
-
-      if (LAYOUT == LAYOUT_LINEAR && (sf_cols & 3) != 0) {
-        // scale rows are not word aligned: one byte per block, written by its even lane
-        if (active && !(lane & 1)) out_sf[row * sf_cols + sf_col] = (uint8_t)q8;
-        sfw[i] = 0;
-      } else {
-        // gather the 4 scale bytes of 64 consecutive elements into lane 0 of each 8-lane group
-        uint32_t v = ((lane & 1) || !active) ? 0u : (q8 << (8 * ((lane >> 1) & 3)));
-        v |= dpp_xor2(v);
-        v |= dpp_shl4(v);
-        sfw[i] = v;
-      }
-    }
-
-    if ((lane & 7) == 0 && col_ok && !(LAYOUT == LAYOUT_LINEAR && (sf_cols & 3) != 0)) {
-      if constexpr (LAYOUT == LAYOUT_SWIZZLED && ROW_ITERS == 4) {
-        // rows rb, rb+32, rb+64, rb+96 of one 128-row tile: 16 contiguous bytes
-        uint8_t* dst = out_sf + (int64_t)blockIdx.y * (padded << 7) + ((sf_col >> 2) << 9) + (rb << 4);
-        *reinterpret_cast<uint4*>(dst) = make_uint4(sfw[0], sfw[1], sfw[2], sfw[3]);
-      } else {
-#pragma unroll
-        for (int i = 0; i < ROW_ITERS; ++i) {
-          const int64_t row = row0 + rb + 32 * i;
-          if constexpr (LAYOUT == LAYOUT_SWIZZLED) {
-            // rows past `rows` inside the last 128-row tile receive zeros
-            *reinterpret_cast<uint32_t*>(out_sf + swizzle_128x4(row, sf_col, padded)) = sfw[i];
-          } else if constexpr (LAYOUT == LAYOUT_GROUPED) {
-            if (row < rows)
-              *reinterpret_cast<uint32_t*>(out_sf + row_sf_base[rb + 32 * i] + ((sf_col >> 2) << 9)) = sfw[i];
-          } else {
-            if (row < rows) *reinterpret_cast<uint32_t*>(out_sf + row * sf_cols + sf_col) = sfw[i];
-          }
-        }
-      }
+    for (int j = 0; j < 4; ++j) {
+      p0 |= f32x2_to_e2m1_byte(x[2 * j] * r, x[2 * j + 1] * r) << (8 * j);
+      p1 |= f32x2_to_e2m1_byte(x[8 + 2 * j] * r, x[8 + 2 * j + 1] * r) << (8 * j);
     }
   }
+  if (active) __builtin_nontemporal_store(u32x2{p0, p1}, reinterpret_cast<u32x2*>(out_fp4 + ((row * cols + col) >> 1)));
+
+  if (!word_scales) {
+    if (active) out_sf[sf_row_base + sf_col] = (uint8_t)q8;  // scale rows are not word aligned
+    return;
+  }
+  // merge the scale bytes of 4 neighbouring blocks; the quad leader stores the dword
+  uint32_t v = active ? (q8 << (8 * (lane & 3))) : 0u;
+  v |= dpp_xor1(v);
+  v |= dpp_xor2(v);
+  if ((lane & 3) == 0 && col_ok) {
+    if constexpr (LAYOUT == LAYOUT_SWIZZLED) {
+      *reinterpret_cast<uint32_t*>(out_sf + sf_row_base + ((sf_col >> 2) << 9)) = v;
+    } else if constexpr (LAYOUT == LAYOUT_GROUPED) {
+      if (row < rows) *reinterpret_cast<uint32_t*>(out_sf + sf_row_base + ((sf_col >> 2) << 9)) = v;
+    } else {
+      if (row < rows) *reinterpret_cast<uint32_t*>(out_sf + sf_row_base + sf_col) = v;
+    }
+  }
+}
+
+template <typename T, int LAYOUT>
+int launch_nvfp4_layout(const T* in, int64_t rows, int64_t cols, const float* gs, const int32_t* in_off,
+                        const int32_t* out_off, int groups, uint8_t* out_fp4, uint8_t* out_sf, hipStream_t stream) {
+  const int64_t segs = ceil_div(cols, kSegCols);
+  // rows the grid must cover: the swizzled layout also zero-fills the padding rows of the last tile
+  const int64_t cover = LAYOUT == LAYOUT_SWIZZLED ? round_up(rows, 128) : rows;
+  const int64_t wgs = ceil_div(cover, 4) * segs;
+  if (wgs >= ((int64_t)1 << 31)) return fail(NVF_ERR_UNSUPPORTED_SHAPE, "tensor of %lld x %lld is too large for one launch",
+                                             (long long)rows, (long long)cols);
+  hipLaunchKernelGGL((nvfp4_quantize_kernel<T, LAYOUT>), dim3((unsigned)wgs), dim3(256), 0, stream, in, rows, cols, gs,
+                     in_off, out_off, groups, (uint32_t)segs, out_fp4, out_sf);
+  return check_launch("nvfp4_quantize_kernel");
 }
 
 template <typename T>
 int launch_nvfp4_typed(const T* in, int64_t rows, int64_t cols, const float* gs, int layout, const int32_t* in_off,
                        const int32_t* out_off, int groups, uint8_t* out_fp4, uint8_t* out_sf, hipStream_t stream) {
-  const unsigned gx = (unsigned)ceil_div(cols, kSegCols);
-  // Large inputs: 128-row bands (16-byte scale stores).  Small inputs: 32-row bands so that more
-  // compute units get work.
-  const bool big = rows * cols >= ((int64_t)1 << 24);
-  if (layout == LAYOUT_SWIZZLED) {
-    if (big) {
-      dim3 grid(gx, (unsigned)ceil_div(rows, 128));
-      hipLaunchKernelGGL((nvfp4_quantize_kernel<T, LAYOUT_SWIZZLED, 4>), grid, dim3(256), 0, stream, in, rows, cols, gs,
-                         in_off, out_off, groups, out_fp4, out_sf);
-    } else {
-      dim3 grid(gx, (unsigned)(round_up(rows, 128) / 32));
-      hipLaunchKernelGGL((nvfp4_quantize_kernel<T, LAYOUT_SWIZZLED, 1>), grid, dim3(256), 0, stream, in, rows, cols, gs,
-                         in_off, out_off, groups, out_fp4, out_sf);
-    }
-  } else if (layout == LAYOUT_GROUPED) {
-    if (big) {
-      dim3 grid(gx, (unsigned)ceil_div(rows, 128));
-      hipLaunchKernelGGL((nvfp4_quantize_kernel<T, LAYOUT_GROUPED, 4>), grid, dim3(256), 0, stream, in, rows, cols, gs,
-                         in_off, out_off, groups, out_fp4, out_sf);
-    } else {
-      dim3 grid(gx, (unsigned)ceil_div(rows, 32));
-      hipLaunchKernelGGL((nvfp4_quantize_kernel<T, LAYOUT_GROUPED, 1>), grid, dim3(256), 0, stream, in, rows, cols, gs,
-                         in_off, out_off, groups, out_fp4, out_sf);
-    }
-  } else {
-    if (big) {
-      dim3 grid(gx, (unsigned)ceil_div(rows, 128));
-      hipLaunchKernelGGL((nvfp4_quantize_kernel<T, LAYOUT_LINEAR, 4>), grid, dim3(256), 0, stream, in, rows, cols, gs,
-                         in_off, out_off, groups, out_fp4, out_sf);
-    } else {
-      dim3 grid(gx, (unsigned)ceil_div(rows, 32));
-      hipLaunchKernelGGL((nvfp4_quantize_kernel<T, LAYOUT_LINEAR, 1>), grid, dim3(256), 0, stream, in, rows, cols, gs,
-                         in_off, out_off, groups, out_fp4, out_sf);
-    }
-  }
-  return check_launch("nvfp4_quantize_kernel");
+  if (layout == LAYOUT_SWIZZLED)
+    return launch_nvfp4_layout<T, LAYOUT_SWIZZLED>(in, rows, cols, gs, in_off, out_off, groups, out_fp4, out_sf, stream);
+  if (layout == LAYOUT_GROUPED)
+    return launch_nvfp4_layout<T, LAYOUT_GROUPED>(in, rows, cols, gs, in_off, out_off, groups, out_fp4, out_sf, stream);
+  return launch_nvfp4_layout<T, LAYOUT_LINEAR>(in, rows, cols, gs, in_off, out_off, groups, out_fp4, out_sf, stream);
 }
 
 // -------------------------------------------------------------------------------------------------
-// MXFP8: 32-element blocks (4 lanes), scale = ue8m0_rp(amax * (1/448)), payload = e4m3(x * 2^-(e-127))
+// MXFP8: 32-element blocks, scale = ue8m0_rp(amax * (1/448)), payload = e4m3(x * 2^-(e-127)).
+// A lane holds 16 elements (half a block, amax merged with its neighbour by one DPP step) and stores 16
+// payload bytes; a wavefront owns a 1024-element row segment, a workgroup 4 consecutive rows of it, in
+// the same row-major order of short workgroups as the NVFP4 kernel.
 // -------------------------------------------------------------------------------------------------
 template <typename T, bool SWIZZLE>
 __global__ __launch_bounds__(256) void mxfp8_quantize_kernel(const T* __restrict__ in, int64_t rows, int64_t cols,
-                                                             uint8_t* __restrict__ out_fp8,
+                                                             uint32_t segs, uint8_t* __restrict__ out_fp8,
                                                              uint8_t* __restrict__ out_sf) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const int64_t row0 = (int64_t)blockIdx.y * 32;
-  const int64_t col = (int64_t)blockIdx.x * kSegCols + lane * 8;
-  const bool col_ok = col < cols;
+  const uint32_t band = blockIdx.x / segs;
+  const uint32_t seg = blockIdx.x - band * segs;
+  const int64_t row = (int64_t)band * 4 + wave;
+  const int64_t col = (int64_t)seg * kSegCols + lane * 16;
+  const bool col_ok = col < cols;  // cols % 32 == 0, so both lanes of a block agree
+  const bool active = col_ok && row < rows;
   const int64_t sf_cols = cols >> 5;
   const int64_t padded = (sf_cols + 3) & ~(int64_t)3;
   const int64_t sf_col = col >> 5;
   const bool word_stores = SWIZZLE || (sf_cols & 3) == 0;
 
-#pragma unroll 1
-  for (int t = 0; t < 8; ++t) {
-    const int64_t row = row0 + t * 4 + wave;
-    const bool active = col_ok && row < rows;
-    float x[8];
-    bool nan = false;
-    if (active) {
-      load8(in + row * cols + col, x, nan);
-    } else {
+  const Raw16<T> raw = issue16(active ? in + row * cols + col : in);
+  float x[16];
+  bool nonfinite;
+  decode16(raw, active, x, nonfinite);
+  const bool wave_nonfinite = __builtin_amdgcn_ballot_w64(nonfinite) != 0;
+  // amax, NaN ignored (fmaxf), start -inf: block_quantization_kernels.cu:124-128
+  float m = -INFINITY;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) x[j] = 0.0f;
+  for (int j = 0; j < 16; ++j) m = fmaxf(m, fabsf(x[j]));
+  m = fmaxf(m, bits_to_f32(dpp_xor1(f32_to_bits(m))));
+  const uint32_t e = f32_to_e8m0_rp(m * (1.0f / 448));                   // :168-169
+  const float inv = (e == 0) ? 1.0f : bits_to_f32((254u - e) << 23);     // :134-140
+  uint32_t w[4] = {0, 0, 0, 0};
+  if (!wave_nonfinite) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      w[j] = __builtin_amdgcn_cvt_pk_fp8_f32(__builtin_amdgcn_fmed3f(x[4 * j] * inv, -448.0f, 448.0f),
+                                             __builtin_amdgcn_fmed3f(x[4 * j + 1] * inv, -448.0f, 448.0f), w[j], false);
+      w[j] = __builtin_amdgcn_cvt_pk_fp8_f32(__builtin_amdgcn_fmed3f(x[4 * j + 2] * inv, -448.0f, 448.0f),
+                                             __builtin_amdgcn_fmed3f(x[4 * j + 3] * inv, -448.0f, 448.0f), w[j], true);
     }
-    const bool wave_has_nan = __builtin_amdgcn_ballot_w64(nan) != 0;  // any non-finite input in the wavefront
-    float m = amax8(x);
-    m = fmaxf(m, bits_to_f32(dpp_xor1(f32_to_bits(m))));
-    m = fmaxf(m, bits_to_f32(dpp_xor2(f32_to_bits(m))));
-    const uint32_t e = f32_to_e8m0_rp(m * (1.0f / 448));                   // :168-169
-    const float inv = (e == 0) ? 1.0f : bits_to_f32((254u - e) << 23);     // :134-140
-    uint32_t lo = 0, hi = 0;
-    if (!wave_has_nan) {
-      float y[8];
+  } else {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) y[j] = __builtin_amdgcn_fmed3f(x[j] * inv, -448.0f, 448.0f);
-      lo = __builtin_amdgcn_cvt_pk_fp8_f32(y[0], y[1], lo, false);
-      lo = __builtin_amdgcn_cvt_pk_fp8_f32(y[2], y[3], lo, true);
-      hi = __builtin_amdgcn_cvt_pk_fp8_f32(y[4], y[5], hi, false);
-      hi = __builtin_amdgcn_cvt_pk_fp8_f32(y[6], y[7], hi, true);
-    } else {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        lo |= f32_to_e4m3_satfinite(x[j] * inv) << (8 * j);
-        hi |= f32_to_e4m3_satfinite(x[4 + j] * inv) << (8 * j);
-      }
-    }
-    if (active) *reinterpret_cast<uint2*>(out_fp8 + row * cols + col) = make_uint2(lo, hi);
+    for (int j = 0; j < 16; ++j) w[j >> 2] |= f32_to_e4m3_satfinite(x[j] * inv) << (8 * (j & 3));
+  }
+  if (active)
+    __builtin_nontemporal_store(u32x4{w[0], w[1], w[2], w[3]}, reinterpret_cast<u32x4*>(out_fp8 + row * cols + col));
 
-    if (word_stores) {
-      uint32_t v = ((lane & 3) || !active) ? 0u : (e << (8 * ((lane >> 2) & 3)));
-      v |= dpp_shl4(v);
-      v |= dpp_shl8(v);
-      if ((lane & 15) == 0 && col_ok) {
-        if constexpr (SWIZZLE) {
-          *reinterpret_cast<uint32_t*>(out_sf + swizzle_128x4(row, sf_col, padded)) = v;
-        } else {
-          if (row < rows) *reinterpret_cast<uint32_t*>(out_sf + row * sf_cols + sf_col) = v;
-        }
-      }
+  if (!word_stores) {
+    if (active && !(lane & 1)) out_sf[row * sf_cols + sf_col] = (uint8_t)e;  // scale rows are not word aligned
+    return;
+  }
+  // the scale bytes of 4 neighbouring blocks (8 lanes) merged into lane 0 of every 8
+  uint32_t v = ((lane & 1) || !active) ? 0u : (e << (8 * ((lane >> 1) & 3)));
+  v |= dpp_xor2(v);
+  v |= dpp_shl4(v);
+  if ((lane & 7) == 0 && col_ok) {
+    if constexpr (SWIZZLE) {
+      *reinterpret_cast<uint32_t*>(out_sf + swizzle_128x4(row, sf_col, padded)) = v;  // padding rows: zeros
     } else {
-      if (active && !(lane & 3)) out_sf[row * sf_cols + sf_col] = (uint8_t)e;
+      if (row < rows) *reinterpret_cast<uint32_t*>(out_sf + row * sf_cols + sf_col) = v;
     }
   }
 }
@@ -325,13 +329,17 @@ __global__ __launch_bounds__(256) void mxfp8_quantize_kernel(const T* __restrict
 template <typename T>
 int launch_mxfp8_typed(const T* in, int64_t rows, int64_t cols, int swizzle, uint8_t* out_fp8, uint8_t* out_sf,
                        hipStream_t stream) {
-  const unsigned gx = (unsigned)ceil_div(cols, kSegCols);
+  const int64_t segs = ceil_div(cols, kSegCols);
+  const int64_t cover = swizzle ? round_up(rows, 128) : rows;
+  const int64_t wgs = ceil_div(cover, 4) * segs;
+  if (wgs >= ((int64_t)1 << 31)) return fail(NVF_ERR_UNSUPPORTED_SHAPE, "tensor of %lld x %lld is too large for one launch",
+                                             (long long)rows, (long long)cols);
   if (swizzle) {
-    dim3 grid(gx, (unsigned)(round_up(rows, 128) / 32));
-    hipLaunchKernelGGL((mxfp8_quantize_kernel<T, true>), grid, dim3(256), 0, stream, in, rows, cols, out_fp8, out_sf);
+    hipLaunchKernelGGL((mxfp8_quantize_kernel<T, true>), dim3((unsigned)wgs), dim3(256), 0, stream, in, rows, cols,
+                       (uint32_t)segs, out_fp8, out_sf);
   } else {
-    dim3 grid(gx, (unsigned)ceil_div(rows, 32));
-    hipLaunchKernelGGL((mxfp8_quantize_kernel<T, false>), grid, dim3(256), 0, stream, in, rows, cols, out_fp8, out_sf);
+    hipLaunchKernelGGL((mxfp8_quantize_kernel<T, false>), dim3((unsigned)wgs), dim3(256), 0, stream, in, rows, cols,
+                       (uint32_t)segs, out_fp8, out_sf);
   }
   return check_launch("mxfp8_quantize_kernel");
 }
