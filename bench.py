@@ -87,6 +87,10 @@ def main():
 
     extra = {}
     gen = torch.Generator(device=dev).manual_seed(0)
+    measured_traffic = {}
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tpath):
+        measured_traffic = json.load(open(tpath))
 
     # ------------------------------------------------------------------ extras
     def run_quant():
@@ -98,7 +102,10 @@ def main():
         extra["nvfp4_quantize"] = {"workload": "bf16 [65536,7168] -> NVFP4, 128x4 swizzled scales (config 5 activations)",
                                    "ms": round(ms, 4), "GB/s": round(gbs, 1),
                                    "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                                                "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None}}
+                                                "frac": round(gbs / PEAK_HBM_GBS, 4),
+                                                "traffic": measured_traffic.get("nvfp4_quantize_65536x7168_bytes_per_launch"),
+                                                "kernel": "nvfp4_quantize_kernel",
+                                                "bytes_per_launch": m * k * 2.5625}}
         sizes = moe_zipf(8192, 8, 256, 1.1, 0).int()
         padded = (sizes + 127) // 128 * 128
         eo = (torch.cumsum(sizes, 0) - sizes).int().to(dev)
@@ -219,10 +226,7 @@ def main():
     ms, wall_ms = timed(lambda: nvf_cutlass.mxfp8_scaled_mm(qa, qb, sa, sb, one, torch.bfloat16), args.steps, args.warmup)
     tflops = flops / ms / 1e9
 
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "traffic.json")
-    if os.path.exists(tpath):
-        traffic = json.load(open(tpath)).get("mxfp8_gemm_8192_bytes_per_launch")
+    traffic = measured_traffic.get("mxfp8_gemm_8192_bytes_per_launch")
 
     # ------------------------------------------------------------------ CPU baseline (bounded sample)
     cpu = None
@@ -277,7 +281,7 @@ def main():
         "config": {"workload": "BASELINE config 2: MXFP8 scaled GEMM M=N=K=8192, e8m0 per-32 scales in 128x4 layout, A row-major, B K-major"},
         "roofline": {"bound": "mfma", "achieved": round(tflops, 2), "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(tflops / PEAK_FP8_TFLOPS, 4), "traffic": traffic,
-                     "kernel": "mxfp8_gemm_kernel", "flops_per_launch": flops},
+                     "kernel": "mxfp8_gemm_256_kernel", "flops_per_launch": flops},
         "cpu_baseline": cpu,
         "extra": extra,
     }
