@@ -292,6 +292,243 @@ __global__ __launch_bounds__(256) void gemm16_kernel(const Params p) {
   }
 }
 
+// -------------------------------------------------------------------------------------------------
+// NVFP4 fast path: dense, 256x256 tile, M % 256 == N % 256 == 0, K % 128 == 0.
+//   * Persistent workgroups walk the tiles in an XCD-aware order; the operand stream (global -> registers
+//     -> fp16 in LDS) runs continuously across tile borders, two 64-deep K steps ahead of the MFMAs.
+//   * Thread t owns row t of both operand tiles: per step it loads 32 payload bytes and one scale dword
+//     (the 128x4 layout keeps a row's four K-blocks of a step in one dword) per operand, two steps
+//     before use; the conversion to fp16 (one v_cvt_scalef32_pk_f16_fp4 and one v_pk_mul_f16 per two
+//     elements) and the LDS writes for step g+1 are spread between the MFMAs of step g.
+//   * e4m3 -> fp16 of a scale is a shift: (s & 0x7f) << 7 is s * 2^-8 as fp16 (also for subnormal s);
+//     the 2^8 is given back by the payload conversion's power-of-two scale operand.
+//   * One barrier per step, placed before the last quarter of its MFMAs: by then every wave has written
+//     its share of the next step and holds this step's last fragments in registers.
+// LDS: two buffers of (A tile + B tile), each tile 256 rows x 128 bytes with 16-byte chunk c of row r at
+// chunk position c ^ ((r >> 1) & 7): conflict-free for the row-per-lane writes and the fragment reads.
+// -------------------------------------------------------------------------------------------------
+__device__ __forceinline__ int lds_pos2(int row, int chunk) { return row * 8 + (chunk ^ ((row >> 1) & 7)); }
+
+template <bool OUT_BF16>
+__global__ __launch_bounds__(256, 1) void nvfp4_gemm_256_kernel(const Params p) {
+  constexpr int BM = 256, BN = 256;
+  constexpr int TILE_UNITS = 2048;           // 16-byte units per operand tile
+  constexpr int BUF_UNITS = 2 * TILE_UNITS;  // A + B
+  extern __shared__ u32x4 lds[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int li = lane & 31, lg = lane >> 5;
+
+  // ---- persistent tile walk: workgroup ids are dealt round-robin to the 8 XCDs, XCD x owns the tile
+  // range [x*chunk, (x+1)*chunk); with the 8 (m) x 4 (n) blocked numbering the 32 tiles an XCD works on
+  // at a time share 8 A panels and 4 B panels in its L2.
+  const int tiles_m = p.m / BM, tiles_n = p.n / BN;
+  const int total = tiles_m * tiles_n;
+  const int chunk_tiles = (total + 7) >> 3;
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, slots = gridDim.x >> 3;
+  const int range_end = min((xcd + 1) * chunk_tiles, total);
+  const bool blocked = (tiles_m & 7) == 0 && (tiles_n & 3) == 0;
+  auto tile_coords = [&](int t, int& m0, int& n0) {
+    int mt, nt;
+    if (blocked) {
+      const int sb = t >> 5, w = t & 31;
+      mt = (sb % (tiles_m >> 3)) * 8 + (w & 7);
+      nt = (sb / (tiles_m >> 3)) * 4 + (w >> 3);
+    } else {
+      mt = t % tiles_m;
+      nt = t / tiles_m;
+    }
+    m0 = mt * BM;
+    n0 = nt * BN;
+  };
+  const int first_tile = xcd * chunk_tiles + slot;
+  if (first_tile >= range_end) return;
+
+  const int kbytes = p.k >> 1;
+  const int nk = p.k >> 6;         // 64-deep steps; even
+  const int sf_padded = p.k >> 4;  // K % 128 == 0: no padding columns
+
+  // ---- operand stream: this thread's row of the tile the stream is in (lp) and of the tile it enters
+  // next (np); it advances by selects only
+  struct RowPtrs { const uint8_t *a, *b, *sa, *sb; };
+  auto tile_ptrs = [&](int t) {
+    int m0, n0;
+    tile_coords(t, m0, n0);
+    RowPtrs r;
+    r.a = p.a + (int64_t)(m0 + tid) * kbytes;
+    r.b = p.b + (int64_t)(n0 + tid) * kbytes;
+    r.sa = p.sfa + swizzle_128x4(m0 + tid, 0, sf_padded);
+    r.sb = p.sfb + swizzle_128x4(n0 + tid, 0, sf_padded);
+    return r;
+  };
+  RowPtrs lp = tile_ptrs(first_tile);
+  RowPtrs np = lp;
+  int l_ks = 0;
+  struct Raw { u32x4 a0, a1, b0, b1; uint32_t sa, sb; };
+  auto issue_loads = [&](Raw& r) {
+    const int64_t o = (int64_t)l_ks * 32;
+    r.a0 = *reinterpret_cast<const u32x4*>(lp.a + o);
+    r.a1 = *reinterpret_cast<const u32x4*>(lp.a + o + 16);
+    r.b0 = *reinterpret_cast<const u32x4*>(lp.b + o);
+    r.b1 = *reinterpret_cast<const u32x4*>(lp.b + o + 16);
+    r.sa = *reinterpret_cast<const uint32_t*>(lp.sa + (int64_t)l_ks * 512);
+    r.sb = *reinterpret_cast<const uint32_t*>(lp.sb + (int64_t)l_ks * 512);
+    const bool wrap = (l_ks + 1 == nk);
+    l_ks = wrap ? 0 : l_ks + 1;
+    lp.a = wrap ? np.a : lp.a;
+    lp.b = wrap ? np.b : lp.b;
+    lp.sa = wrap ? np.sa : lp.sa;
+    lp.sb = wrap ? np.sb : lp.sb;
+  };
+
+  // ---- conversion: unit u (0..15) = operand u>>3, 16-byte fp16 chunk u&7 of this thread's row
+  auto scale_pair = [&](uint32_t s4, int b) {
+    const uint32_t s = s4 >> (8 * b);
+    uint32_t h = ((s & 0x7fu) << 7) | ((s & 0x80u) << 8);  // e4m3 -> fp16 bits of s * 2^-8
+    h = ((s & 0x7fu) == 0x7fu) ? 0x7e00u : h;              // e4m3 NaN
+    return __builtin_bit_cast(f16x2, h | (h << 16));
+  };
+  auto convert_unit = [&](const Raw& r, const f16x2 (&sv)[2][4], int u, int wbuf) {
+    const int op = u >> 3, c = u & 7;
+    const uint32_t q = op ? (c < 4 ? r.b0[c & 3] : r.b1[c & 3]) : (c < 4 ? r.a0[c & 3] : r.a1[c & 3]);
+    const f16x2 s = sv[op][c >> 1];
+    const f16x2 h0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(q, 256.0f, 0) * s;
+    const f16x2 h1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(q, 256.0f, 1) * s;
+    const f16x2 h2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(q, 256.0f, 2) * s;
+    const f16x2 h3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(q, 256.0f, 3) * s;
+    lds[wbuf * BUF_UNITS + op * TILE_UNITS + lds_pos2(tid, c)] =
+        u32x4{__builtin_bit_cast(uint32_t, h0), __builtin_bit_cast(uint32_t, h1), __builtin_bit_cast(uint32_t, h2),
+              __builtin_bit_cast(uint32_t, h3)};
+  };
+  auto scale_vectors = [&](const Raw& r, f16x2 (&sv)[2][4]) {
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      sv[0][b] = scale_pair(r.sa, b);
+      sv[1][b] = scale_pair(r.sb, b);
+    }
+  };
+
+  // ---- MFMA fragments of one 16-deep sub-step: unit q (0..7) = operand q>>2, 32-row sub-tile q&3
+  struct Frag { u32x4 a[4], b[4]; };
+  auto load_frag_unit = [&](int buf, int kk, int q, Frag& f) {
+    const int op = q >> 2, t = q & 3;
+    const int row = (op ? wn : wm) * 128 + t * 32 + li;
+    const u32x4 v = lds[buf * BUF_UNITS + op * TILE_UNITS + lds_pos2(row, kk * 2 + lg)];
+    if (op) f.b[t] = v; else f.a[t] = v;
+  };
+
+  f32x16 acc[4][4];
+  auto zero_acc = [&]() {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+  };
+  zero_acc();
+
+  // Keeps the 16 accumulator tiles "used" at this point of the program, so that the MFMAs producing
+  // them cannot be moved past the statement that follows (they have no side effects of their own).
+#define NVF_PIN_ACC()                                                                                          \
+  do {                                                                                                         \
+    asm volatile("" : "+a"(acc[0][0]), "+a"(acc[0][1]), "+a"(acc[0][2]), "+a"(acc[0][3]), "+a"(acc[1][0]),     \
+                 "+a"(acc[1][1]), "+a"(acc[1][2]), "+a"(acc[1][3]));                                           \
+    asm volatile("" : "+a"(acc[2][0]), "+a"(acc[2][1]), "+a"(acc[2][2]), "+a"(acc[2][3]), "+a"(acc[3][0]),     \
+                 "+a"(acc[3][1]), "+a"(acc[3][2]), "+a"(acc[3][3]));                                           \
+  } while (0)
+
+  const float alpha = p.alpha[0];
+  Raw raw[2];
+  Frag fr[2];
+  f16x2 sv[2][4];
+
+  // ---- prologue: step 0 converted into buffer 0, step 1 in registers, fragments of sub-step 0 loaded
+  issue_loads(raw[0]);
+  issue_loads(raw[1]);
+  scale_vectors(raw[0], sv);
+#pragma unroll
+  for (int u = 0; u < 16; ++u) convert_unit(raw[0], sv, u, 0);
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+#pragma unroll
+  for (int q = 0; q < 8; ++q) load_frag_unit(0, 0, q, fr[0]);
+
+  for (int c_tile = first_tile; c_tile < range_end; c_tile += slots) {
+    np = (c_tile + slots < range_end) ? tile_ptrs(c_tile + slots) : lp;
+    for (int c_ks = 0; c_ks < nk; c_ks += 2) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {  // step g = c_ks + h computes from LDS buffer h
+        // loads of step g+2 go to raw[h] (converted one step ago); step g+1 = raw[h^1] is converted now
+        issue_loads(raw[h]);
+        scale_vectors(raw[h ^ 1], sv);
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+          if (kk == 3) {
+            // every wave has written its rows of step g+1 and read the last fragments of step g
+            NVF_PIN_ACC();
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+          }
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int q = 0; q < 16; ++q) {
+            const int i = q >> 2, j = q & 3;
+            const int slot_id = kk * 16 + q;
+            if ((q & 1) == 0) load_frag_unit(kk < 3 ? h : (h ^ 1), (kk + 1) & 3, q >> 1, fr[(kk + 1) & 1]);
+            if (kk < 3 && slot_id % 3 == 0) convert_unit(raw[h ^ 1], sv, slot_id / 3, h ^ 1);
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, fr[kk & 1].b[j]),
+                                                               __builtin_bit_cast(f16x8, fr[kk & 1].a[i]), acc[i][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        }
+      }
+    }
+    // ---- epilogue; the next tile's first step is already in LDS and its second in registers.
+    // acc[i][j][r] = C[m = li][n = (r/4)*8 + lg*4 + r%4] of its 32x32 sub-tile.
+    int m0, n0;
+    tile_coords(c_tile, m0, n0);
+    uint16_t* out = static_cast<uint16_t*>(p.out);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      uint16_t* orow = out + (int64_t)(m0 + wm * 128 + i * 32 + li) * p.n + n0 + wn * 128 + lg * 4;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq) {
+          u32x2 v;
+          v[0] = pack2(acc[i][j][rq * 4 + 0] * alpha, acc[i][j][rq * 4 + 1] * alpha, OUT_BF16);
+          v[1] = pack2(acc[i][j][rq * 4 + 2] * alpha, acc[i][j][rq * 4 + 3] * alpha, OUT_BF16);
+          *reinterpret_cast<u32x2*>(orow + j * 32 + rq * 8) = v;
+        }
+      }
+    }
+    zero_acc();
+  }
+#undef NVF_PIN_ACC
+}
+
+template <bool OUT_BF16>
+int launch_nvfp4_fast(const Params& p, int cus, hipStream_t stream) {
+  auto kern = nvfp4_gemm_256_kernel<OUT_BF16>;
+  constexpr int lds_bytes = 2 * 2 * 2048 * 16;  // 128 KiB
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    if (e != hipSuccess) return fail(NVF_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    configured = true;
+  }
+  const int64_t tiles = (int64_t)(p.m / 256) * (p.n / 256);
+  const unsigned grid = (unsigned)(tiles >= cus ? (cus & ~7) : ((tiles + 7) / 8) * 8);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_bytes, stream, p);
+  return check_launch("nvfp4_gemm_256_kernel");
+}
+
 template <int BM, int BN, bool NVFP4, bool BF16_MMA, bool OUT_BF16>
 int launch_cfg(const Params& p, int grid, hipStream_t stream) {
   auto kern = gemm16_kernel<BM, BN, NVFP4, BF16_MMA, OUT_BF16>;
@@ -311,6 +548,10 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, hipStream_t stream) {
   // Pick the largest tile that still yields about one work item per compute unit.
   auto tiles = [&](int bm, int bn) { return ceil_div(m_hint, bm) * ceil_div(p.n, bn); };
   const bool dense = p.problem_sizes == nullptr;
+  if constexpr (NVFP4) {
+    if (dense && tiles(256, 256) >= 128 && (p.m & 255) == 0 && (p.n & 255) == 0 && (p.k & 127) == 0 && p.k >= 256)
+      return launch_nvfp4_fast<OUT_BF16>(p, cus, stream);
+  }
   if (tiles(256, 256) >= cus || (!dense && m_hint >= 256 * (int64_t)p.groups)) {
     const int64_t upper = dense ? tiles(256, 256) : (ceil_div(p.m, 256) + p.groups) * ceil_div(p.n, 256);
     return launch_cfg<256, 256, NVFP4, BF16_MMA, OUT_BF16>(p, (int)(upper < cus ? upper : cus), stream);

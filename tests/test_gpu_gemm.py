@@ -174,6 +174,45 @@ def test_mxfp8_gemm_ragged_shapes_alpha_and_scale_spread(dev, shape):
 
 
 @pytest.mark.parametrize("shape", [(4096, 2048, 512), (2560, 3328, 384), (2048, 4096, 256), (8192, 1024, 1152)])
+def test_nvfp4_gemm_persistent_256_tile_kernel_full_compare(dev, shape):
+    """Dense shapes with M % 256 == N % 256 == K % 128 == 0 and at least 128 tiles take the persistent
+    kernel that converts the operands to fp16 between its MFMAs; every output element is compared with
+    the oracle.  Same tile-grid cases as the MXFP8 test below."""
+    m, n, k = shape
+    gen = torch.Generator().manual_seed(k + 1)
+    a, sa, ga = _nvfp4_operand(m, k, 1.0, gen)
+    b, sb, gb = _nvfp4_operand(n, k, 0.02, gen)
+    alpha = 1.0 / (ga * gb)
+    ref = O.ref_nvfp4_scaled_mm(a, b, sa, sb, alpha)
+    out = _run_nvfp4(a, b, sa, sb, alpha, torch.bfloat16, dev)
+    scale = ref.abs().amax(dim=1, keepdim=True).clamp(min=1e-30)
+    assert ((out.float().cpu() - ref).abs() / scale).max().item() <= GEMM_MAX_REL
+    assert torch.equal(out, _run_nvfp4(a, b, sa, sb, alpha, torch.bfloat16, dev))
+    out16 = _run_nvfp4(a, b, sa, sb, alpha, torch.float16, dev)
+    assert ((out16.float().cpu() - ref).abs() / scale).max().item() <= GEMM_MAX_REL
+
+
+@pytest.mark.parametrize("scale_range", [(0x01, 0x0F), (0x01, 0x7E), (0x70, 0x7E)])
+def test_nvfp4_gemm_persistent_kernel_every_scale_code_is_decoded_exactly(dev, scale_range):
+    """Random payload bytes and random e4m3 scale bytes, including the subnormal codes 0x01..0x07 and the
+    largest finite ones: each e2m1 x e4m3 product is exactly representable in fp16, so the only error
+    left is the fp32 summation order and the bf16 rounding of the output."""
+    m, n, k = 2048, 4096, 256
+    gen = torch.Generator().manual_seed(scale_range[0] * 131 + scale_range[1])
+    a = torch.randint(0, 256, (m, k // 2), dtype=torch.uint8, generator=gen)
+    b = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, generator=gen)
+    lo, hi = scale_range
+    sa = O.linear_to_swizzled_128_4(torch.randint(lo, hi + 1, (m, k // 16), dtype=torch.uint8, generator=gen))
+    sb = O.linear_to_swizzled_128_4(torch.randint(lo, hi + 1, (n, k // 16), dtype=torch.uint8, generator=gen))
+    alpha = 2.0 ** -12 if hi > 0x40 else 1.0
+    ref = O.ref_nvfp4_scaled_mm(a, b, sa, sb, alpha)
+    out = _run_nvfp4(a, b, sa, sb, alpha, torch.bfloat16, dev)
+    # row-wise: 2^-8 (half a bf16 ulp) of the largest magnitude plus fp32 summation noise
+    scale = ref.abs().amax(dim=1, keepdim=True).clamp(min=1e-38)
+    assert ((out.float().cpu() - ref).abs() / scale).max().item() <= 2.0 ** -7
+
+
+@pytest.mark.parametrize("shape", [(4096, 2048, 512), (2560, 3328, 384), (2048, 4096, 256), (8192, 1024, 1152)])
 def test_mxfp8_gemm_persistent_256_tile_kernel_full_compare(dev, shape):
     """Shapes with M % 256 == N % 256 == K % 128 == 0 and at least 128 tiles take the persistent
     LDS-direct kernel; every output element is compared with the oracle.  (2560, 3328) has a tile grid
