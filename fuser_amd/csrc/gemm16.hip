@@ -293,24 +293,33 @@ __global__ __launch_bounds__(256) void gemm16_kernel(const Params p) {
 }
 
 // -------------------------------------------------------------------------------------------------
-// NVFP4 fast path: dense, 256x256 tile, M % 256 == N % 256 == 0, K % 128 == 0.
+// NVFP4 fast path: dense, 256x256 tile, M % 256 == N % 256 == 0, K % 128 == 0, K >= 256.
+//   * 512 threads: 8 wavefronts as 2 (m) x 4 (n), each with a 128x64 accumulator tile, two per SIMD.
+//     A single wavefront issues at most one non-MFMA instruction per ~8 cycles, which is too little for
+//     the conversion work next to 32-cycle MFMAs; with two wavefronts per SIMD one converts while the
+//     other's MFMA runs.
 //   * Persistent workgroups walk the tiles in an XCD-aware order; the operand stream (global -> registers
-//     -> fp16 in LDS) runs continuously across tile borders, two 64-deep K steps ahead of the MFMAs.
-//   * Thread t owns row t of both operand tiles: per step it loads 32 payload bytes and one scale dword
-//     (the 128x4 layout keeps a row's four K-blocks of a step in one dword) per operand, two steps
-//     before use; the conversion to fp16 (one v_cvt_scalef32_pk_f16_fp4 and one v_pk_mul_f16 per two
-//     elements) and the LDS writes for step g+1 are spread between the MFMAs of step g.
-//   * e4m3 -> fp16 of a scale is a shift: (s & 0x7f) << 7 is s * 2^-8 as fp16 (also for subnormal s);
-//     the 2^8 is given back by the payload conversion's power-of-two scale operand.
+//     -> fp16 in LDS) runs continuously across tile borders, two 128-deep spans ahead of the MFMAs.
+//   * Loads cover two 64-deep steps (a span of 128 elements of K) at a time so that four neighbouring
+//     lanes read 64 contiguous bytes of a row: thread t loads 16 payload bytes (two scale blocks) and
+//     their 2 scale bytes for rows t/4 and t/4+128 of both operand tiles.  Of each such piece the first
+//     block belongs to the even step and the second to the odd step: inside a span the even step
+//     consumes blocks 0,2,4,6 and the odd step blocks 1,3,5,7 (the same permutation of K for A and B, so
+//     the dot products are unchanged), which keeps every lane busy in every step.
+//   * Conversion to fp16: one v_cvt_scalef32_pk_f16_fp4 and one v_pk_mul_f16 per two elements; the scale
+//     goes e4m3 -> fp32 -> packed fp16 pair in two instructions (every e4m3 value is an fp16 value).
+//   * Every piece of non-MFMA work is cut into MFMA-slot sized parts (3 conversion instructions, one LDS
+//     access, one global load) and pinned between two MFMAs, because the two wavefronts of a SIMD run
+//     in phase and a long run of other instructions in both would idle the matrix pipe.
 //   * One barrier per step, placed before the last quarter of its MFMAs: by then every wave has written
 //     its share of the next step and holds this step's last fragments in registers.
 // LDS: two buffers of (A tile + B tile), each tile 256 rows x 128 bytes with 16-byte chunk c of row r at
-// chunk position c ^ ((r >> 1) & 7): conflict-free for the row-per-lane writes and the fragment reads.
+// chunk position c ^ ((r >> 1) & 7): conflict-free for the fragment reads.
 // -------------------------------------------------------------------------------------------------
 __device__ __forceinline__ int lds_pos2(int row, int chunk) { return row * 8 + (chunk ^ ((row >> 1) & 7)); }
 
 template <bool OUT_BF16>
-__global__ __launch_bounds__(256, 1) void nvfp4_gemm_256_kernel(const Params p) {
+__global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   constexpr int BM = 256, BN = 256;
   constexpr int TILE_UNITS = 2048;           // 16-byte units per operand tile
   constexpr int BUF_UNITS = 2 * TILE_UNITS;  // A + B
@@ -319,8 +328,9 @@ __global__ __launch_bounds__(256, 1) void nvfp4_gemm_256_kernel(const Params p) 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave >> 2, wn = wave & 3;
   const int li = lane & 31, lg = lane >> 5;
+  const int srow = tid >> 2, spiece = tid & 3;  // staging: rows srow and srow+128, 16-byte piece of a 64-byte span
 
   // ---- persistent tile walk: workgroup ids are dealt round-robin to the 8 XCDs, XCD x owns the tile
   // range [x*chunk, (x+1)*chunk); with the 8 (m) x 4 (n) blocked numbering the 32 tiles an XCD works on
@@ -348,140 +358,163 @@ __global__ __launch_bounds__(256, 1) void nvfp4_gemm_256_kernel(const Params p) 
   if (first_tile >= range_end) return;
 
   const int kbytes = p.k >> 1;
-  const int nk = p.k >> 6;         // 64-deep steps; even
+  const int nmac = p.k >> 7;       // 128-deep load spans per tile (>= 2)
   const int sf_padded = p.k >> 4;  // K % 128 == 0: no padding columns
+  const int64_t row128 = (int64_t)128 * kbytes;       // payload distance of the thread's two rows
+  const int64_t sfrow128 = (int64_t)128 * sf_padded;  // same for the scales (next 128-row tile)
 
-  // ---- operand stream: this thread's row of the tile the stream is in (lp) and of the tile it enters
+  // ---- operand stream: this thread's piece in the tile the stream is in (lp) and in the tile it enters
   // next (np); it advances by selects only
   struct RowPtrs { const uint8_t *a, *b, *sa, *sb; };
   auto tile_ptrs = [&](int t) {
     int m0, n0;
     tile_coords(t, m0, n0);
     RowPtrs r;
-    r.a = p.a + (int64_t)(m0 + tid) * kbytes;
-    r.b = p.b + (int64_t)(n0 + tid) * kbytes;
-    r.sa = p.sfa + swizzle_128x4(m0 + tid, 0, sf_padded);
-    r.sb = p.sfb + swizzle_128x4(n0 + tid, 0, sf_padded);
+    r.a = p.a + (int64_t)(m0 + srow) * kbytes + spiece * 16;
+    r.b = p.b + (int64_t)(n0 + srow) * kbytes + spiece * 16;
+    // scale blocks 2*spiece, 2*spiece+1 of the span: 128x4 layout column tile spiece>>1, bytes 2*(spiece&1)..
+    r.sa = p.sfa + swizzle_128x4(m0 + srow, 0, sf_padded) + (spiece >> 1) * 512 + (spiece & 1) * 2;
+    r.sb = p.sfb + swizzle_128x4(n0 + srow, 0, sf_padded) + (spiece >> 1) * 512 + (spiece & 1) * 2;
     return r;
   };
   RowPtrs lp = tile_ptrs(first_tile);
   RowPtrs np = lp;
-  int l_ks = 0;
-  struct Raw { u32x4 a0, a1, b0, b1; uint32_t sa, sb; };
-  auto issue_loads = [&](Raw& r) {
-    const int64_t o = (int64_t)l_ks * 32;
-    r.a0 = *reinterpret_cast<const u32x4*>(lp.a + o);
-    r.a1 = *reinterpret_cast<const u32x4*>(lp.a + o + 16);
-    r.b0 = *reinterpret_cast<const u32x4*>(lp.b + o);
-    r.b1 = *reinterpret_cast<const u32x4*>(lp.b + o + 16);
-    r.sa = *reinterpret_cast<const uint32_t*>(lp.sa + (int64_t)l_ks * 512);
-    r.sb = *reinterpret_cast<const uint32_t*>(lp.sb + (int64_t)l_ks * 512);
-    const bool wrap = (l_ks + 1 == nk);
-    l_ks = wrap ? 0 : l_ks + 1;
+  int l_mac = 0;
+  struct Raw { u32x4 a[2], b[2]; uint32_t sa[2], sb[2]; };
+  // load unit q (0..7) of the span the stream is at; advance_stream() after the eighth
+  auto issue_load_unit = [&](Raw& r, int q) {
+    const int64_t o = (int64_t)l_mac * 64, so = (int64_t)l_mac * 1024;
+    if (q == 0) r.a[0] = *reinterpret_cast<const u32x4*>(lp.a + o);
+    if (q == 1) r.a[1] = *reinterpret_cast<const u32x4*>(lp.a + o + row128);
+    if (q == 2) r.b[0] = *reinterpret_cast<const u32x4*>(lp.b + o);
+    if (q == 3) r.b[1] = *reinterpret_cast<const u32x4*>(lp.b + o + row128);
+    if (q == 4) r.sa[0] = *reinterpret_cast<const uint16_t*>(lp.sa + so);
+    if (q == 5) r.sa[1] = *reinterpret_cast<const uint16_t*>(lp.sa + so + sfrow128);
+    if (q == 6) r.sb[0] = *reinterpret_cast<const uint16_t*>(lp.sb + so);
+    if (q == 7) r.sb[1] = *reinterpret_cast<const uint16_t*>(lp.sb + so + sfrow128);
+  };
+  auto advance_stream = [&]() {
+    const bool wrap = (l_mac + 1 == nmac);
+    l_mac = wrap ? 0 : l_mac + 1;
     lp.a = wrap ? np.a : lp.a;
     lp.b = wrap ? np.b : lp.b;
     lp.sa = wrap ? np.sa : lp.sa;
     lp.sb = wrap ? np.sb : lp.sb;
   };
 
-  // ---- conversion: unit u (0..15) = operand u>>3, 16-byte fp16 chunk u&7 of this thread's row
-  auto scale_pair = [&](uint32_t s4, int b) {
-    const uint32_t s = s4 >> (8 * b);
-    uint32_t h = ((s & 0x7fu) << 7) | ((s & 0x80u) << 8);  // e4m3 -> fp16 bits of s * 2^-8
-    h = ((s & 0x7fu) == 0x7fu) ? 0x7e00u : h;              // e4m3 NaN
-    return __builtin_bit_cast(f16x2, h | (h << 16));
+  // ---- conversion for a step of parity P: unit u (0..7) = operand u>>2, row (u>>1)&1, half block u&1.
+  // A unit is spread over three MFMA slots (about 3 VALU instructions each).
+  auto scale_pair = [&](uint32_t s2, int b) {
+    const float f = b ? __builtin_amdgcn_cvt_f32_fp8((int)s2, 1) : __builtin_amdgcn_cvt_f32_fp8((int)s2, 0);
+    return __builtin_bit_cast(f16x2, __builtin_amdgcn_cvt_pkrtz(f, f));  // exact: e4m3 fits fp16
   };
-  auto convert_unit = [&](const Raw& r, const f16x2 (&sv)[2][4], int u, int wbuf) {
-    const int op = u >> 3, c = u & 7;
-    const uint32_t q = op ? (c < 4 ? r.b0[c & 3] : r.b1[c & 3]) : (c < 4 ? r.a0[c & 3] : r.a1[c & 3]);
-    const f16x2 s = sv[op][c >> 1];
-    const f16x2 h0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(q, 256.0f, 0) * s;
-    const f16x2 h1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(q, 256.0f, 1) * s;
-    const f16x2 h2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(q, 256.0f, 2) * s;
-    const f16x2 h3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(q, 256.0f, 3) * s;
-    lds[wbuf * BUF_UNITS + op * TILE_UNITS + lds_pos2(tid, c)] =
-        u32x4{__builtin_bit_cast(uint32_t, h0), __builtin_bit_cast(uint32_t, h1), __builtin_bit_cast(uint32_t, h2),
-              __builtin_bit_cast(uint32_t, h3)};
-  };
-  auto scale_vectors = [&](const Raw& r, f16x2 (&sv)[2][4]) {
-#pragma unroll
-    for (int b = 0; b < 4; ++b) {
-      sv[0][b] = scale_pair(r.sa, b);
-      sv[1][b] = scale_pair(r.sb, b);
+  uint32_t cq;  // payload dword of the unit in progress
+  f16x2 ch[4];  // its four converted pairs
+  f16x2 sv[2][2];
+  auto convert_phase = [&](const Raw& r, int parity, int u, int phase, int wbuf) {
+    const int op = u >> 2, i = (u >> 1) & 1, cc = u & 1;
+    if (phase == 0) {
+      if (cc == 0) sv[op][i] = scale_pair(op ? r.sb[i] : r.sa[i], parity);
+      cq = op ? r.b[i][2 * parity + cc] : r.a[i][2 * parity + cc];
+      ch[0] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(cq, 1.0f, 0);
+      ch[1] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(cq, 1.0f, 1);
+      ch[2] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(cq, 1.0f, 2);
+    } else if (phase == 1) {
+      ch[3] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(cq, 1.0f, 3);
+      ch[0] = ch[0] * sv[op][i];
+      ch[1] = ch[1] * sv[op][i];
+    } else {
+      ch[2] = ch[2] * sv[op][i];
+      ch[3] = ch[3] * sv[op][i];
+      lds[wbuf * BUF_UNITS + op * TILE_UNITS + lds_pos2(srow + 128 * i, spiece * 2 + cc)] =
+          u32x4{__builtin_bit_cast(uint32_t, ch[0]), __builtin_bit_cast(uint32_t, ch[1]), __builtin_bit_cast(uint32_t, ch[2]),
+                __builtin_bit_cast(uint32_t, ch[3])};
     }
   };
 
-  // ---- MFMA fragments of one 16-deep sub-step: unit q (0..7) = operand q>>2, 32-row sub-tile q&3
-  struct Frag { u32x4 a[4], b[4]; };
+  // ---- MFMA fragments of one 16-deep sub-step, loaded in the order of their first use by the MFMA
+  // sequence (a0 b0) (a0 b1) (a1 b0) ...: units 0..5 = a0, b0, b1, a1, a2, a3
+  struct Frag { u32x4 a[4], b[2]; };
   auto load_frag_unit = [&](int buf, int kk, int q, Frag& f) {
-    const int op = q >> 2, t = q & 3;
-    const int row = (op ? wn : wm) * 128 + t * 32 + li;
+    const int op = (q == 1 || q == 2) ? 1 : 0;
+    const int t = op ? q - 1 : (q == 0 ? 0 : q - 2);
+    const int row = (op ? wn * 64 : wm * 128) + t * 32 + li;
     const u32x4 v = lds[buf * BUF_UNITS + op * TILE_UNITS + lds_pos2(row, kk * 2 + lg)];
     if (op) f.b[t] = v; else f.a[t] = v;
   };
 
-  f32x16 acc[4][4];
+  f32x16 acc[4][2];
   auto zero_acc = [&]() {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
+      for (int j = 0; j < 2; ++j)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
   };
   zero_acc();
 
-  // Keeps the 16 accumulator tiles "used" at this point of the program, so that the MFMAs producing
-  // them cannot be moved past the statement that follows (they have no side effects of their own).
-#define NVF_PIN_ACC()                                                                                          \
-  do {                                                                                                         \
-    asm volatile("" : "+a"(acc[0][0]), "+a"(acc[0][1]), "+a"(acc[0][2]), "+a"(acc[0][3]), "+a"(acc[1][0]),     \
-                 "+a"(acc[1][1]), "+a"(acc[1][2]), "+a"(acc[1][3]));                                           \
-    asm volatile("" : "+a"(acc[2][0]), "+a"(acc[2][1]), "+a"(acc[2][2]), "+a"(acc[2][3]), "+a"(acc[3][0]),     \
-                 "+a"(acc[3][1]), "+a"(acc[3][2]), "+a"(acc[3][3]));                                           \
-  } while (0)
+  // Keeps the accumulator tiles "used" at this point of the program, so that the MFMAs producing them
+  // cannot be moved past the statement that follows (they have no side effects of their own).
+#define NVF_PIN_ACC()                                                                                        \
+  asm volatile("" : "+a"(acc[0][0]), "+a"(acc[0][1]), "+a"(acc[1][0]), "+a"(acc[1][1]), "+a"(acc[2][0]),     \
+               "+a"(acc[2][1]), "+a"(acc[3][0]), "+a"(acc[3][1]))
 
   const float alpha = p.alpha[0];
-  Raw raw[2];
+  Raw cur, nxt;  // span whose odd step is converted next / span whose even step is converted next
   Frag fr[2];
-  f16x2 sv[2][4];
 
-  // ---- prologue: step 0 converted into buffer 0, step 1 in registers, fragments of sub-step 0 loaded
-  issue_loads(raw[0]);
-  issue_loads(raw[1]);
-  scale_vectors(raw[0], sv);
+  // The stream runs two spans ahead of the MFMAs; with two spans per tile it is a whole tile ahead.
+  const int tiles_ahead = nmac == 2 ? 2 : 1;
+  auto ptrs_or_current = [&](int t) { return t < range_end ? tile_ptrs(t) : lp; };
+
+  // ---- prologue: spans 0 and 1 requested, even step of span 0 converted into buffer 0
+  np = ptrs_or_current(first_tile + slots);
 #pragma unroll
-  for (int u = 0; u < 16; ++u) convert_unit(raw[0], sv, u, 0);
+  for (int q = 0; q < 8; ++q) issue_load_unit(cur, q);
+  advance_stream();
+#pragma unroll
+  for (int q = 0; q < 8; ++q) issue_load_unit(nxt, q);
+  advance_stream();
+#pragma unroll
+  for (int u = 0; u < 8; ++u)
+#pragma unroll
+    for (int ph = 0; ph < 3; ++ph) convert_phase(cur, 0, u, ph, 0);
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
 #pragma unroll
-  for (int q = 0; q < 8; ++q) load_frag_unit(0, 0, q, fr[0]);
+  for (int q = 0; q < 6; ++q) load_frag_unit(0, 0, q, fr[0]);
 
   for (int c_tile = first_tile; c_tile < range_end; c_tile += slots) {
-    np = (c_tile + slots < range_end) ? tile_ptrs(c_tile + slots) : lp;
-    for (int c_ks = 0; c_ks < nk; c_ks += 2) {
+    np = ptrs_or_current(c_tile + tiles_ahead * slots);
+    for (int c_mac = 0; c_mac < nmac; ++c_mac) {
 #pragma unroll
-      for (int h = 0; h < 2; ++h) {  // step g = c_ks + h computes from LDS buffer h
-        // loads of step g+2 go to raw[h] (converted one step ago); step g+1 = raw[h^1] is converted now
-        issue_loads(raw[h]);
-        scale_vectors(raw[h ^ 1], sv);
+      for (int h = 0; h < 2; ++h) {  // step g = 2*c_mac + h computes from LDS buffer h
+        // h == 0: the odd step of the current span is converted into buffer 1
+        // h == 1: the even step of the next span is converted into buffer 0; then that span becomes the
+        //         current one and the span after it is requested
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk) {
           if (kk == 3) {
-            // every wave has written its rows of step g+1 and read the last fragments of step g
+            // every wave has written its share of step g+1 and read the last fragments of step g
             NVF_PIN_ACC();
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
+            if (h == 1) cur = nxt;
           }
           __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-          for (int q = 0; q < 16; ++q) {
-            const int i = q >> 2, j = q & 3;
-            const int slot_id = kk * 16 + q;
-            if ((q & 1) == 0) load_frag_unit(kk < 3 ? h : (h ^ 1), (kk + 1) & 3, q >> 1, fr[(kk + 1) & 1]);
-            if (kk < 3 && slot_id % 3 == 0) convert_unit(raw[h ^ 1], sv, slot_id / 3, h ^ 1);
+          for (int q = 0; q < 8; ++q) {
+            const int i = q >> 1, j = q & 1;
+            const int slot_id = kk * 8 + q;
+            if (q < 6) load_frag_unit(kk < 3 ? h : (h ^ 1), (kk + 1) & 3, q, fr[(kk + 1) & 1]);
+            if (kk < 3) convert_phase(h ? nxt : cur, h ^ 1, slot_id / 3, slot_id % 3, h ^ 1);
+            if (kk == 3 && h == 1) {
+              issue_load_unit(nxt, q);
+              if (q == 7) advance_stream();
+            }
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, fr[kk & 1].b[j]),
                                                                __builtin_bit_cast(f16x8, fr[kk & 1].a[i]), acc[i][j], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
@@ -489,16 +522,16 @@ __global__ __launch_bounds__(256, 1) void nvfp4_gemm_256_kernel(const Params p) 
         }
       }
     }
-    // ---- epilogue; the next tile's first step is already in LDS and its second in registers.
+    // ---- epilogue; the next tile's first step is already in LDS.
     // acc[i][j][r] = C[m = li][n = (r/4)*8 + lg*4 + r%4] of its 32x32 sub-tile.
     int m0, n0;
     tile_coords(c_tile, m0, n0);
     uint16_t* out = static_cast<uint16_t*>(p.out);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      uint16_t* orow = out + (int64_t)(m0 + wm * 128 + i * 32 + li) * p.n + n0 + wn * 128 + lg * 4;
+      uint16_t* orow = out + (int64_t)(m0 + wm * 128 + i * 32 + li) * p.n + n0 + wn * 64 + lg * 4;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+      for (int j = 0; j < 2; ++j) {
 #pragma unroll
         for (int rq = 0; rq < 4; ++rq) {
           u32x2 v;
@@ -525,7 +558,7 @@ int launch_nvfp4_fast(const Params& p, int cus, hipStream_t stream) {
   }
   const int64_t tiles = (int64_t)(p.m / 256) * (p.n / 256);
   const unsigned grid = (unsigned)(tiles >= cus ? (cus & ~7) : ((tiles + 7) / 8) * 8);
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_bytes, stream, p);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds_bytes, stream, p);
   return check_launch("nvfp4_gemm_256_kernel");
 }
 
