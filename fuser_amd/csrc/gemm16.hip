@@ -562,6 +562,165 @@ int launch_nvfp4_fast(const Params& p, int cus, hipStream_t stream) {
   return check_launch("nvfp4_gemm_256_kernel");
 }
 
+// -------------------------------------------------------------------------------------------------
+// NVFP4 skinny path: dense, M <= 128 (decode-sized activations), K % 128 == 0, N % (16*RT) == 0.
+// The weight matrix is streamed exactly once, so the op is bound by HBM and by the conversion work,
+// not by the MFMAs:
+//   * A workgroup owns 16*RT weight rows for the whole of K and all M activation rows; its 8
+//     wavefronts split K in interleaved 128-element chunks and their partial sums are added in a fixed
+//     order through LDS (no atomics, no workspace, deterministic).
+//   * Nothing is staged through LDS: in v_mfma_f32_16x16x32_f16 lane (i, g) supplies 8 elements of row i,
+//     and both operands use the same (lane group, element) -> k assignment, so a lane loads the 16
+//     payload bytes [32g, 32g+32) of its row's chunk, converts them to fp16 in registers and feeds MFMA
+//     t = 0..3 with elements 8t..8t+7.  Weight rows are the first operand (output rows), activation rows
+//     the second, so a lane ends up with 4 consecutive N-elements of one output row.
+// -------------------------------------------------------------------------------------------------
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// 32 packed e2m1 values and their two e4m3 block scales -> four MFMA operands of 8 fp16 values
+__device__ __forceinline__ void dequant_frags(const u32x4 q, uint32_t s2, u32x4 out[4]) {
+  const float f0 = __builtin_amdgcn_cvt_f32_fp8((int)s2, 0), f1 = __builtin_amdgcn_cvt_f32_fp8((int)s2, 1);
+  const f16x2 sv[2] = {__builtin_bit_cast(f16x2, __builtin_amdgcn_cvt_pkrtz(f0, f0)),
+                       __builtin_bit_cast(f16x2, __builtin_amdgcn_cvt_pkrtz(f1, f1))};
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {  // dword w = elements 8w..8w+7, scale block w/2
+    const f16x2 h0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(q[w], 1.0f, 0) * sv[w >> 1];
+    const f16x2 h1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(q[w], 1.0f, 1) * sv[w >> 1];
+    const f16x2 h2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(q[w], 1.0f, 2) * sv[w >> 1];
+    const f16x2 h3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(q[w], 1.0f, 3) * sv[w >> 1];
+    out[w] = u32x4{__builtin_bit_cast(uint32_t, h0), __builtin_bit_cast(uint32_t, h1), __builtin_bit_cast(uint32_t, h2),
+                   __builtin_bit_cast(uint32_t, h3)};
+  }
+}
+
+template <int RT, int TT, bool OUT_BF16>
+__global__ __launch_bounds__(512) void nvfp4_skinny_kernel(const Params p) {
+  constexpr int W = 8;  // wavefronts
+  extern __shared__ f32x4 red[];  // [W][tt_count][64 lanes], reused for each of the RT row tiles
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * (16 * RT);
+  const int tt_count = (p.m + 15) >> 4;  // 16-row activation tiles, at most TT
+  const int kbytes = p.k >> 1;
+  const int chunks = p.k >> 7;
+  const int sf_padded = p.k >> 4;  // K % 128 == 0: no padding columns
+  // chunk c, lane group g: payload bytes [64c + 16g, +16), scale blocks 8c + 2g, 8c + 2g + 1
+  const int sf_lane_off = (g >> 1) * 512 + (g & 1) * 2;
+
+  const uint8_t* b_row[RT];
+  const uint8_t* b_sf[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    b_row[rt] = p.b + (int64_t)(n0 + rt * 16 + r) * kbytes + g * 16;
+    b_sf[rt] = p.sfb + swizzle_128x4(n0 + rt * 16 + r, 0, sf_padded) + sf_lane_off;
+  }
+  f32x4 acc[RT][TT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) acc[rt][tt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+  for (int c = wave; c < chunks; c += W) {
+    u32x4 bq[RT];
+    uint32_t bs[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      bq[rt] = *reinterpret_cast<const u32x4*>(b_row[rt] + (int64_t)c * 64);
+      bs[rt] = *reinterpret_cast<const uint16_t*>(b_sf[rt] + (int64_t)c * 1024);
+    }
+    // activation tiles: the loads of tile tt+1 are in flight while tile tt is converted and multiplied
+    auto load_a = [&](int tt, u32x4& q, uint32_t& sc) {
+      const int tok = min(tt * 16 + r, p.m - 1);  // rows past M repeat the last one; they are not stored
+      q = *reinterpret_cast<const u32x4*>(p.a + (int64_t)tok * kbytes + g * 16 + (int64_t)c * 64);
+      sc = *reinterpret_cast<const uint16_t*>(p.sfa + swizzle_128x4(tok, 0, sf_padded) + sf_lane_off + (int64_t)c * 1024);
+    };
+    u32x4 aq_next;
+    uint32_t as_next;
+    load_a(0, aq_next, as_next);
+    u32x4 fb[RT][4];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) dequant_frags(bq[rt], bs[rt], fb[rt]);
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) {
+      if (tt < tt_count) {
+        const u32x4 aq = aq_next;
+        const uint32_t as = as_next;
+        if (tt + 1 < TT && tt + 1 < tt_count) load_a(tt + 1, aq_next, as_next);
+        u32x4 fa[4];
+        dequant_frags(aq, as, fa);
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt)
+            acc[rt][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, fb[rt][t]),
+                                                                 __builtin_bit_cast(f16x8, fa[t]), acc[rt][tt], 0, 0, 0);
+      }
+    }
+  }
+
+  // ---- per row tile: sum the wavefronts' partial tiles in wave order and store
+  const float alpha = p.alpha[0];
+  uint16_t* out = static_cast<uint16_t*>(p.out);
+  const int units = tt_count * 64;
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    if (rt > 0) __syncthreads();
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt)
+      if (tt < tt_count) red[(wave * tt_count + tt) * 64 + lane] = acc[rt][tt];
+    __syncthreads();
+    for (int u = tid; u < units; u += 512) {
+      const int l = u & 63, tt = u >> 6;
+      f32x4 s = red[u];
+#pragma unroll
+      for (int w = 1; w < W; ++w) s += red[w * units + u];
+      // element e of lane l: weight row 4*(l/16) + e (output column), activation row l%16 (output row)
+      const int tok = tt * 16 + (l & 15);
+      if (tok < p.m) {
+        u32x2 v;
+        v[0] = pack2(s[0] * alpha, s[1] * alpha, OUT_BF16);
+        v[1] = pack2(s[2] * alpha, s[3] * alpha, OUT_BF16);
+        *reinterpret_cast<u32x2*>(out + (int64_t)tok * p.n + n0 + rt * 16 + 4 * (l >> 4)) = v;
+      }
+    }
+  }
+}
+
+template <int RT, int TT, bool OUT_BF16>
+int launch_nvfp4_skinny_cfg(const Params& p, hipStream_t stream) {
+  auto kern = nvfp4_skinny_kernel<RT, TT, OUT_BF16>;
+  const int tt_count = (p.m + 15) >> 4;
+  const int lds_bytes = 8 * tt_count * 64 * 16;  // one set of partial tiles per wavefront: at most 64 KiB
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 8 * TT * 64 * 16);
+    if (e != hipSuccess) return fail(NVF_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    configured = true;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)(p.n / (16 * RT))), dim3(512), lds_bytes, stream, p);
+  return check_launch("nvfp4_skinny_kernel");
+}
+
+template <int TT, bool OUT_BF16>
+int launch_nvfp4_skinny_tt(const Params& p, int cus, hipStream_t stream) {
+  // More weight rows per workgroup convert the activations less often; keep enough workgroups to fill
+  // the chip (small activation tiles leave room for several workgroups per compute unit).
+  const int64_t want = (int64_t)cus * (TT >= 8 ? 3 : TT >= 4 ? 4 : 8) / 4;
+  if ((p.n & 63) == 0 && p.n / 64 >= want) return launch_nvfp4_skinny_cfg<4, TT, OUT_BF16>(p, stream);
+  if ((p.n & 31) == 0 && p.n / 32 >= want) return launch_nvfp4_skinny_cfg<2, TT, OUT_BF16>(p, stream);
+  return launch_nvfp4_skinny_cfg<1, TT, OUT_BF16>(p, stream);
+}
+
+template <bool OUT_BF16>
+int launch_nvfp4_skinny(const Params& p, int cus, hipStream_t stream) {
+  if (p.m <= 16) return launch_nvfp4_skinny_tt<1, OUT_BF16>(p, cus, stream);
+  if (p.m <= 32) return launch_nvfp4_skinny_tt<2, OUT_BF16>(p, cus, stream);
+  if (p.m <= 64) return launch_nvfp4_skinny_tt<4, OUT_BF16>(p, cus, stream);
+  return launch_nvfp4_skinny_tt<8, OUT_BF16>(p, cus, stream);
+}
+
 template <int BM, int BN, bool NVFP4, bool BF16_MMA, bool OUT_BF16>
 int launch_cfg(const Params& p, int grid, hipStream_t stream) {
   auto kern = gemm16_kernel<BM, BN, NVFP4, BF16_MMA, OUT_BF16>;
@@ -582,6 +741,7 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, hipStream_t stream) {
   auto tiles = [&](int bm, int bn) { return ceil_div(m_hint, bm) * ceil_div(p.n, bn); };
   const bool dense = p.problem_sizes == nullptr;
   if constexpr (NVFP4) {
+    if (dense && p.m <= 128 && (p.k & 127) == 0 && (p.n & 15) == 0) return launch_nvfp4_skinny<OUT_BF16>(p, cus, stream);
     if (dense && tiles(256, 256) >= 128 && (p.m & 255) == 0 && (p.n & 255) == 0 && (p.k & 127) == 0 && p.k >= 256)
       return launch_nvfp4_fast<OUT_BF16>(p, cus, stream);
   }

@@ -91,6 +91,27 @@ def test_nvfp4_gemm_llm_and_ragged_shapes(dev, shape):
         assert max_rel(out, ref) <= GEMM_MAX_REL, (shape, dtype)
 
 
+@pytest.mark.parametrize("shape", [(1, 32, 128), (7, 96, 256), (16, 32, 128), (17, 64, 384), (33, 160, 1152),
+                                   (64, 4096, 512), (65, 2048, 256), (127, 224, 640), (128, 16384, 128)])
+def test_nvfp4_gemm_decode_sized_activations(dev, shape):
+    """M <= 128 with K % 128 == 0 and N % 16 == 0 takes the kernel that streams the weights once and
+    splits K over the wavefronts of a workgroup: every count of 16-row activation tiles, activation rows
+    that do not fill a tile, 1 / 2 / 4 weight-row tiles per workgroup, poisoned scale padding, both
+    output types, run-to-run determinism of the in-workgroup reduction."""
+    m, n, k = shape
+    gen = torch.Generator().manual_seed(m * 31 + n)
+    a, sa, ga = _nvfp4_operand(m, k, 1.0, gen)
+    b, sb, gb = _nvfp4_operand(n, k, 0.02, gen)
+    alpha = 1.0 / (ga * gb)
+    ref = O.ref_nvfp4_scaled_mm(a, b, sa, sb, alpha)
+    sa_p = sa.clone()  # NaN code in every scale byte of the padding rows
+    sa_p[O.linear_to_swizzled_128_4(torch.ones(m, k // 16, dtype=torch.uint8)) == 0] = 0x7F
+    for dtype in (torch.bfloat16, torch.float16):
+        out = _run_nvfp4(a, b, sa_p, sb, alpha, dtype, dev)
+        assert out.shape == (m, n) and max_rel(out, ref) <= GEMM_MAX_REL, (shape, dtype)
+        assert torch.equal(out, _run_nvfp4(a, b, sa_p, sb, alpha, dtype, dev))
+
+
 def test_nvfp4_gemm_ignores_scale_padding_and_is_deterministic(dev):
     gen = torch.Generator().manual_seed(9)
     m, n, k = 100, 160, 96  # k/16 = 6 -> padded to 8 ; rows padded to 128 / 256
