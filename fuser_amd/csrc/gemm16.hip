@@ -721,6 +721,262 @@ int launch_nvfp4_skinny(const Params& p, int cus, hipStream_t stream) {
   return launch_nvfp4_skinny_tt<8, OUT_BF16>(p, cus, stream);
 }
 
+// -------------------------------------------------------------------------------------------------
+// grouped_mm fast path (16-bit operands): 256x256 tiles, N % 256 == 0, K % 64 == 0, K >= 128.
+//   * Persistent workgroups walk the (group, m-tile, n-tile) list derived on the device from
+//     problem_sizes; each XCD owns a contiguous part of the list, whose neighbouring tiles share the
+//     group's weight panel in that XCD's L2.
+//   * Tiles travel global -> LDS with 16-byte LDS-direct loads issued from inline assembly into a double
+//     buffer (256 rows x 128 bytes per operand and 64-deep K step); the load stream runs two steps ahead
+//     of the MFMAs and continues across tile and group borders.  Rows past the end of a group load the
+//     group's last row again (never another group's memory past the tensor) and are not stored.
+//   * MFMA fragments are double-buffered in registers: the LDS reads of the next half step are in flight
+//     under the 32 MFMAs of the current one; one barrier per K step.
+// LDS layout as in the NVFP4 fast path: chunk c of row r at chunk position c ^ ((r >> 1) & 7).
+// -------------------------------------------------------------------------------------------------
+__device__ __forceinline__ void lds_dma16(uint32_t lds_byte_addr, const uint8_t* base, uint32_t voff) {
+  // lds_byte_addr and base are wave-uniform; lane L's 16 bytes land at lds_byte_addr + 16 * L
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_byte_addr), "v"(voff), "s"(base) : "memory");
+}
+
+template <bool BF16_MMA, bool OUT_BF16>
+__global__ __launch_bounds__(256, 1) void grouped16_gemm_256_kernel(const Params p) {
+  constexpr int BM = 256, BN = 256;
+  constexpr int TILE_UNITS = 2048;           // 16-byte units per operand tile (256 rows x 8 chunks)
+  constexpr int BUF_UNITS = 2 * TILE_UNITS;  // A + B
+  extern __shared__ u32x4 lds[];
+  __shared__ int tile_prefix[kMaxGroups + 1];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int li = lane & 31, lg = lane >> 5;
+  const int tiles_n = p.n / BN;
+
+  // ---- work list: prefix sums of tiles per group (one wavefront, 64 groups per round)
+  if (wave == 0) {
+    int running = 0;
+    for (int base = 0; base < p.groups; base += 64) {
+      const int g = base + lane;
+      int cnt = 0;
+      if (g < p.groups) {
+        const int mg = p.problem_sizes[g * 3];
+        cnt = mg > 0 ? ((mg + BM - 1) / BM) * tiles_n : 0;
+      }
+      int incl = cnt;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const int o = __shfl_up(incl, d, 64);
+        if (lane >= d) incl += o;
+      }
+      if (g < p.groups) tile_prefix[g + 1] = running + incl;
+      running += __shfl(incl, 63, 64);
+    }
+    if (lane == 0) tile_prefix[0] = 0;
+  }
+  __syncthreads();
+  const int total = __builtin_amdgcn_readfirstlane(tile_prefix[p.groups]);
+  const int chunk_tiles = (total + 7) >> 3;
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, slots = gridDim.x >> 3;
+  const int range_end = min((xcd + 1) * chunk_tiles, total);
+  const int first_tile = xcd * chunk_tiles + slot;
+  if (first_tile >= range_end) return;
+
+  const int kb = p.k * 2;   // bytes per operand row
+  const int nk = p.k >> 6;  // 64-deep steps
+
+  struct Tile { const uint8_t *a, *b; int valid; int64_t out_row; int n0; };
+  auto tile_info = [&](int t) {
+    int lo = 0, hi = p.groups;
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (t < tile_prefix[mid]) hi = mid; else lo = mid;
+    }
+    const int g = __builtin_amdgcn_readfirstlane(lo);
+    // (loaded through the vector path, which is coherent with this kernel's own stores; made scalar here)
+    const int m_g = __builtin_amdgcn_readfirstlane(p.problem_sizes[g * 3]);
+    const int64_t row_off = __builtin_amdgcn_readfirstlane(p.expert_offsets[g]);
+    const int tiles_m = (m_g + BM - 1) / BM;
+    const int local = __builtin_amdgcn_readfirstlane(t - tile_prefix[g]);
+    const int nt = local / tiles_m, mt = local - nt * tiles_m;
+    Tile r;
+    r.a = p.a + (row_off + (int64_t)mt * BM) * kb;
+    r.b = p.b + ((int64_t)g * p.n + (int64_t)nt * BN) * kb;
+    r.valid = min(BM, m_g - mt * BM);
+    r.out_row = row_off + (int64_t)mt * BM;
+    r.n0 = nt * BN;
+    return r;
+  };
+
+  // ---- LDS-direct load addressing.  Wave w issues 8 loads per operand per K step; load j covers LDS
+  // units [(w*8+j)*64, +64) = rows (w*8+j)*8 .. +7; lane L lands at unit +L, i.e. row +(L>>3), chunk
+  // position L&7, which must hold global chunk (L&7) ^ ((row>>1)&7) = (L&7) ^ ((L>>4) | ((j&1)<<2)).
+  const uint32_t lrow = (uint32_t)(wave * 64 + (lane >> 3));  // row of this lane in load 0
+  const uint32_t coff_even = (uint32_t)(((lane & 7) ^ (lane >> 4)) << 4);
+  const uint32_t coff_odd = (uint32_t)(((lane & 7) ^ ((lane >> 4) | 4)) << 4);
+  const uint32_t lds_base = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)lds);
+
+  // ---- load stream: the tile the next loads are issued for (lp) and the one after it (np); it
+  // advances without branches so that the hot loop stays one basic block
+  Tile lp = tile_info(first_tile);
+  Tile np = lp;
+  int l_ks = 0, l_count = 0;
+  // Unit q (0..15) of a step: operand q&1, rows (wave*8 + q/2)*8 .. +7
+  auto issue_step_unit = [&](int q) {
+    const int buf = l_count & 1;
+    const int j = q >> 1;
+    const uint32_t l = lds_base + (uint32_t)(buf * BUF_UNITS + (q & 1) * TILE_UNITS + wave * 512) * 16u + j * 1024u;
+    const uint32_t row = lrow + 8u * j;
+    const uint32_t coff = (j & 1) ? coff_odd : coff_even;
+    if (q & 1) {
+      lds_dma16(l, lp.b + ((int64_t)l_ks << 7), row * (uint32_t)kb + coff);
+    } else {
+      lds_dma16(l, lp.a + ((int64_t)l_ks << 7), min(row, (uint32_t)(lp.valid - 1)) * (uint32_t)kb + coff);
+    }
+  };
+  auto issue_step_tail = [&]() {
+    ++l_count;
+    const bool wrap = (l_ks + 1 == nk);
+    l_ks = wrap ? 0 : l_ks + 1;
+    lp.a = wrap ? np.a : lp.a;
+    lp.b = wrap ? np.b : lp.b;
+    lp.valid = wrap ? np.valid : lp.valid;
+  };
+  // Fragment storage: [operand: 0 = A, 1 = B][sub-tile][MFMA of the half step].  Unit q (0..15) of a
+  // half step is one ds_read_b128: operand q>>3, sub-tile (q>>1)&3, MFMA q&1.
+  struct Frags { u32x4 h[2][4][2]; };
+  auto load_unit = [&](int buf, int sub, int q, Frags& f) {
+    const int op = q >> 3, t = (q >> 1) & 3, half = q & 1;
+    const u32x4* base = lds + buf * BUF_UNITS + op * TILE_UNITS;
+    const int row = (op ? wn : wm) * 128 + t * 32 + li;
+    f.h[op][t][half] = base[lds_pos2(row, sub * 4 + lg + 2 * half)];
+  };
+
+  f32x16 acc[4][4];
+  auto zero_acc = [&]() {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+  };
+  zero_acc();
+  auto mfma2 = [&](const Frags& f, int i, int j) {
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+      if constexpr (BF16_MMA) {
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, f.h[1][j][kk]),
+                                                            __builtin_bit_cast(bf16x8, f.h[0][i][kk]), acc[i][j], 0, 0, 0);
+      } else {
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, f.h[1][j][kk]),
+                                                           __builtin_bit_cast(f16x8, f.h[0][i][kk]), acc[i][j], 0, 0, 0);
+      }
+    }
+  };
+
+  // Keeps the 16 accumulator tiles "used" at this point of the program, so that the MFMAs producing
+  // them cannot be moved past the statement that follows (they have no side effects of their own).
+#define NVF_PIN_ACC()                                                                                          \
+  do {                                                                                                         \
+    asm volatile("" : "+a"(acc[0][0]), "+a"(acc[0][1]), "+a"(acc[0][2]), "+a"(acc[0][3]), "+a"(acc[1][0]),     \
+                 "+a"(acc[1][1]), "+a"(acc[1][2]), "+a"(acc[1][3]));                                           \
+    asm volatile("" : "+a"(acc[2][0]), "+a"(acc[2][1]), "+a"(acc[2][2]), "+a"(acc[2][3]), "+a"(acc[3][0]),     \
+                 "+a"(acc[3][1]), "+a"(acc[3][2]), "+a"(acc[3][3]));                                           \
+  } while (0)
+
+  Frags f0, f1;  // fragments of the first / second half (K 0..31 / 32..63) of a step
+
+  np = (first_tile + slots < range_end && nk == 1) ? tile_info(first_tile + slots) : lp;
+#pragma unroll
+  for (int q = 0; q < 16; ++q) issue_step_unit(q);  // step 0
+  issue_step_tail();
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+  for (int q = 0; q < 16; ++q) issue_step_unit(q);  // step 1
+  issue_step_tail();
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+#pragma unroll
+  for (int q = 0; q < 16; ++q) load_unit(0, 0, q, f0);
+
+  int g = 0;
+  Tile ct = tile_info(first_tile);
+  for (int c_tile = first_tile; c_tile < range_end; c_tile += slots) {
+    // the stream is inside this tile by now; prepare the tile it will enter two steps before the end
+    const Tile nt_info = (c_tile + slots < range_end) ? tile_info(c_tile + slots) : ct;
+    np = nt_info;
+    for (int c_ks = 0; c_ks < nk; ++c_ks, ++g) {
+      const int buf = g & 1;
+      // ---- first half: MFMAs on f0, interleaved with the LDS reads that fill f1
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int q = 0; q < 16; ++q) {
+        load_unit(buf, 1, q, f1);
+        mfma2(f0, q >> 2, q & 3);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      NVF_PIN_ACC();
+      // Everything this wave loaded for step g+1 has landed and its reads of buf are complete; after
+      // the barrier that holds for every wave, so buf^1 may be read and buf may be overwritten.
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      // ---- second half: MFMAs on f1, interleaved with the LDS reads of the next step's f0 (from buf^1;
+      // after the last step they read stale data that is never used) and the loads of step g+2 into buf
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int q = 0; q < 16; ++q) {
+        load_unit(buf ^ 1, 0, q, f0);
+        issue_step_unit(q);
+        if (q == 15) issue_step_tail();
+        mfma2(f1, q >> 2, q & 3);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      NVF_PIN_ACC();
+    }
+    // ---- epilogue of this tile; the loads of the next tile's first two steps are already in flight.
+    // acc[i][j][r] = C[m = li][n = (r/4)*8 + lg*4 + r%4] of its 32x32 sub-tile.
+    uint16_t* out = static_cast<uint16_t*>(p.out);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int mrow = wm * 128 + i * 32 + li;
+      if (mrow < ct.valid) {
+        uint16_t* orow = out + (ct.out_row + mrow) * (int64_t)p.n + ct.n0 + wn * 128 + lg * 4;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+          for (int rq = 0; rq < 4; ++rq) {
+            u32x2 v;
+            v[0] = pack2(acc[i][j][rq * 4 + 0], acc[i][j][rq * 4 + 1], OUT_BF16);
+            v[1] = pack2(acc[i][j][rq * 4 + 2], acc[i][j][rq * 4 + 3], OUT_BF16);
+            *reinterpret_cast<u32x2*>(orow + j * 32 + rq * 8) = v;
+          }
+        }
+      }
+    }
+    zero_acc();
+    ct = nt_info;
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no LDS-direct load may outlive the workgroup
+#undef NVF_PIN_ACC
+}
+
+template <bool BF16_MMA, bool OUT_BF16>
+int launch_grouped16_fast(const Params& p, int cus, hipStream_t stream) {
+  auto kern = grouped16_gemm_256_kernel<BF16_MMA, OUT_BF16>;
+  constexpr int lds_bytes = 2 * 2 * 2048 * 16;  // 128 KiB
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    if (e != hipSuccess) return fail(NVF_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    configured = true;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)(cus & ~7)), dim3(256), lds_bytes, stream, p);
+  return check_launch("grouped16_gemm_256_kernel");
+}
+
 template <int BM, int BN, bool NVFP4, bool BF16_MMA, bool OUT_BF16>
 int launch_cfg(const Params& p, int grid, hipStream_t stream) {
   auto kern = gemm16_kernel<BM, BN, NVFP4, BF16_MMA, OUT_BF16>;
@@ -744,6 +1000,12 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, hipStream_t stream) {
     if (dense && p.m <= 128 && (p.k & 127) == 0 && (p.n & 15) == 0) return launch_nvfp4_skinny<OUT_BF16>(p, cus, stream);
     if (dense && tiles(256, 256) >= 128 && (p.m & 255) == 0 && (p.n & 255) == 0 && (p.k & 127) == 0 && p.k >= 256)
       return launch_nvfp4_fast<OUT_BF16>(p, cus, stream);
+  }
+  if constexpr (!NVFP4) {
+    // grouped_mm with groups of a few hundred rows on average: persistent LDS-direct kernel
+    if (!dense && m_hint >= 256 * (int64_t)p.groups && tiles(256, 256) >= cus / 2 && (p.n & 255) == 0 && (p.k & 63) == 0 &&
+        p.k >= 128 && (int64_t)p.k * 2 * 256 < (1ll << 31))
+      return launch_grouped16_fast<BF16_MMA, OUT_BF16>(p, cus, stream);
   }
   if (tiles(256, 256) >= cus || (!dense && m_hint >= 256 * (int64_t)p.groups)) {
     const int64_t upper = dense ? tiles(256, 256) : (ceil_div(p.m, 256) + p.groups) * ceil_div(p.n, 256);

@@ -61,6 +61,33 @@ def test_grouped_mm_empty_groups_and_untouched_rows(dev):
     assert max_rel(out[:200], ref[:200]) <= GEMM_MAX_REL
 
 
+@pytest.mark.parametrize("tensor_dtype,k", [(torch.bfloat16, 192), (torch.float16, 128), (torch.bfloat16, 1088)])
+def test_grouped_mm_persistent_256_tile_kernel_full_compare(dev, tensor_dtype, k):
+    """Large enough for the persistent LDS-direct kernel (N % 256 == 0, K % 64 == 0, >= 256 rows per
+    group on average): groups that end inside a tile, an empty group, a one-row group and a group of
+    257 rows; every output element compared, rows past the last group untouched."""
+    from fuser_amd import capi
+
+    sizes = [1000, 0, 1791, 257, 1, 1000]
+    m, n = sum(sizes) + 47, 2048
+    gen = torch.Generator().manual_seed(k)
+    a = torch.randn(m, k, generator=gen).to(tensor_dtype)
+    b = (torch.randn(len(sizes), n, k, generator=gen) * 0.05).to(tensor_dtype)
+    ps, eo, _, _ = _grouped_args(sizes, n, k, dev)
+    ad, bd, psd, eod = a.to(dev), b.to(dev), ps.to(dev), eo.to(dev)
+    out = torch.full((m, n), 7.0, dtype=tensor_dtype, device=dev)
+    dt = capi.BF16 if tensor_dtype == torch.bfloat16 else capi.F16
+    for _ in range(2):
+        capi.check(capi.lib().nvf_grouped_mm(ad.data_ptr(), bd.data_ptr(), out.data_ptr(), psd.data_ptr(), eod.data_ptr(), len(sizes),
+                                             m, n, k, dt, None))
+    torch.cuda.synchronize()
+    ref = O.ref_grouped_mm(a, b, ps, eo)
+    rows = sum(sizes)
+    assert (out[rows:] == 7.0).all()
+    scale = ref[:rows].abs().amax(dim=1, keepdim=True).clamp(min=1e-30)
+    assert ((out[:rows].float().cpu() - ref[:rows]).abs() / scale).max().item() <= GEMM_MAX_REL
+
+
 def _moe_sizes_top2(tokens, experts, seed):
     gen = torch.Generator().manual_seed(seed)
     logits = torch.randn(tokens, experts, generator=gen) + torch.linspace(-1.5, 1.5, experts)
