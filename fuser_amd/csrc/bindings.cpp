@@ -24,6 +24,14 @@ PYBIND11_MODULE(_C, m) {
       [](const torch::Tensor& a, const torch::Tensor& b, const torch::Tensor& scales_a, const torch::Tensor& scales_b,
          const torch::Tensor& alpha, at::ScalarType out_dtype) { return ck::nvfp4_scaled_mm(a, b, scales_a, scales_b, alpha, out_dtype); },
       "nvfp4_scaled_mm(a, b, scales_a, scales_b, alpha, out_dtype) -> Tensor");
+  cutlass.def(
+      "nvfp4_scaled_mm_blockscale",
+      [](const torch::Tensor& a, const torch::Tensor& b, const torch::Tensor& scales_a, const torch::Tensor& scales_b,
+         const torch::Tensor& alpha, const torch::Tensor& global_normconst) -> py::tuple {
+        auto r = ck::nvfp4_scaled_mm_blockscale(a, b, scales_a, scales_b, alpha, global_normconst);
+        return py::make_tuple(r.first, r.second);
+      },
+      "nvfp4_scaled_mm_blockscale(a, b, scales_a, scales_b, alpha, global_normconst) -> (out_nvfp4, blockscale)");
   cutlass.def("grouped_mm", &ck::grouped_mm,
               "grouped_mm(a, b, ab_strides, c_strides, problem_sizes, expert_offsets) -> Tensor");
   cutlass.def("nvfp4_scaled_grouped_mm", &ck::nvfp4_scaled_grouped_mm,

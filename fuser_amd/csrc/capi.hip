@@ -136,6 +136,22 @@ int nvf_nvfp4_scaled_mm(const void* a, const void* b, const void* scales_a, cons
   return launch_gemm16(0, g, static_cast<hipStream_t>(stream));
 }
 
+int nvf_nvfp4_scaled_mm_blockscale(const void* a, const void* b, const void* scales_a, const void* scales_b,
+                                   const float* alpha, const float* global_normconst, void* out_fp4, void* out_scales,
+                                   float* workspace, int64_t m, int64_t n, int64_t k, void* stream) {
+  NVF_REQUIRE(m >= 0 && n >= 0 && k >= 0, NVF_ERR_INVALID_ARGUMENT, "negative size");
+  NVF_REQUIRE(k % 32 == 0, NVF_ERR_UNSUPPORTED_SHAPE, "The K dimension %lld is not divisible by 32", (long long)k);
+  NVF_REQUIRE(n % 32 == 0, NVF_ERR_UNSUPPORTED_SHAPE, "The N dimension %lld is not divisible by 32", (long long)n);
+  if (m == 0 || n == 0) return NVF_OK;
+  NVF_REQUIRE(a && b && scales_a && scales_b && alpha && global_normconst && out_fp4 && out_scales && workspace,
+              NVF_ERR_INVALID_ARGUMENT, "NULL buffer");
+  Gemm16Args g{a, b, scales_a, scales_b, alpha, workspace, nullptr, nullptr, nullptr, 1, m, n, k, NVF_F32};
+  const int rc = launch_gemm16(0, g, static_cast<hipStream_t>(stream));
+  if (rc != NVF_OK) return rc;
+  return launch_nvfp4_quantize(workspace, NVF_F32, m, n, global_normconst, /*layout: 128x4*/ 1, nullptr, nullptr, 1, out_fp4,
+                               out_scales, static_cast<hipStream_t>(stream));
+}
+
 int nvf_mxfp8_scaled_mm(const void* a, const void* b, const void* scales_a, const void* scales_b, const float* alpha,
                         void* out, int64_t m, int64_t n, int64_t k, int out_dtype, void* stream) {
   NVF_REQUIRE(dtype16(out_dtype), NVF_ERR_INVALID_ARGUMENT, "output dtype must be bf16 or f16, got %d", out_dtype);

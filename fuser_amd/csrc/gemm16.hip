@@ -75,7 +75,7 @@ __device__ __forceinline__ void dequant32(const u32x4 q, uint32_t sf2, u32x4 out
 // 8 consecutive lanes fall into distinct banks.
 __device__ __forceinline__ int lds_pos(int row, int chunk) { return row * 8 + (chunk ^ (row & 7)); }
 
-template <int BM, int BN, bool NVFP4, bool BF16_MMA, bool OUT_BF16>
+template <int BM, int BN, bool NVFP4, bool BF16_MMA, bool OUT_BF16, bool OUT_F32 = false>
 __global__ __launch_bounds__(256) void gemm16_kernel(const Params p) {
   constexpr int BK = 64;
   constexpr int WTM = BM / 2, WTN = BN / 2;  // wave tile
@@ -280,7 +280,14 @@ __global__ __launch_bounds__(256) void gemm16_kernel(const Params p) {
 #pragma unroll
         for (int rq = 0; rq < 4; ++rq) {
           const int ncol = n0 + wn * WTN + j * 32 + rq * 8 + (lane >> 5) * 4;
-          if (ncol < p.n) {
+          if constexpr (OUT_F32) {
+            if (ncol < p.n) {
+              typedef float f32x4_t __attribute__((ext_vector_type(4)));
+              float* frow = static_cast<float*>(p.out) + (row_off + mrow) * (int64_t)p.n;
+              *reinterpret_cast<f32x4_t*>(frow + ncol) = f32x4_t{acc[i][j][rq * 4 + 0] * alpha, acc[i][j][rq * 4 + 1] * alpha,
+                                                                 acc[i][j][rq * 4 + 2] * alpha, acc[i][j][rq * 4 + 3] * alpha};
+            }
+          } else if (ncol < p.n) {
             u32x2 v;
             v[0] = pack2(acc[i][j][rq * 4 + 0] * alpha, acc[i][j][rq * 4 + 1] * alpha, OUT_BF16);
             v[1] = pack2(acc[i][j][rq * 4 + 2] * alpha, acc[i][j][rq * 4 + 3] * alpha, OUT_BF16);
@@ -977,9 +984,9 @@ int launch_grouped16_fast(const Params& p, int cus, hipStream_t stream) {
   return check_launch("grouped16_gemm_256_kernel");
 }
 
-template <int BM, int BN, bool NVFP4, bool BF16_MMA, bool OUT_BF16>
+template <int BM, int BN, bool NVFP4, bool BF16_MMA, bool OUT_BF16, bool OUT_F32 = false>
 int launch_cfg(const Params& p, int grid, hipStream_t stream) {
-  auto kern = gemm16_kernel<BM, BN, NVFP4, BF16_MMA, OUT_BF16>;
+  auto kern = gemm16_kernel<BM, BN, NVFP4, BF16_MMA, OUT_BF16, OUT_F32>;
   constexpr int lds_bytes = (BM + BN) * 128;
   static bool configured = false;  // benign race: the attribute call is idempotent
   if (!configured) {
@@ -1021,6 +1028,18 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, hipStream_t stream) {
   return launch_cfg<64, 64, NVFP4, BF16_MMA, OUT_BF16>(p, (int)(upper < cap ? upper : cap), stream);
 }
 
+// dense NVFP4 with an fp32 result (the product that the block-scaled epilogue op re-quantizes)
+int launch_nvfp4_f32(const Params& p, int cus, hipStream_t stream) {
+  auto tiles = [&](int bm, int bn) { return ceil_div(p.m, bm) * ceil_div(p.n, bn); };
+  if (tiles(256, 256) >= cus) return launch_cfg<256, 256, true, false, false, true>(p, cus, stream);
+  if (tiles(128, 128) >= cus) {
+    const int64_t t = tiles(128, 128);
+    return launch_cfg<128, 128, true, false, false, true>(p, (int)(t < 2 * cus ? t : 2 * cus), stream);
+  }
+  const int64_t t = tiles(64, 64);
+  return launch_cfg<64, 64, true, false, false, true>(p, (int)(t < 4 * cus ? t : 4 * cus), stream);
+}
+
 int cu_count() {
   static int cached = 0;
   if (cached == 0) {
@@ -1054,6 +1073,7 @@ int launch_gemm16(int op, const Gemm16Args& a, hipStream_t stream) {
   p.k = (int)a.k;
   const int cus = cu_count();
   const bool bf16 = a.dtype == NVF_BF16;
+  if (op == 0 && a.dtype == NVF_F32) return launch_nvfp4_f32(p, cus, stream);
   if (op == 0 || op == 1) {
     return bf16 ? launch_sized<true, false, true>(p, a.m, cus, stream) : launch_sized<true, false, false>(p, a.m, cus, stream);
   }

@@ -150,6 +150,30 @@ torch::Tensor nvfp4_scaled_mm(const torch::Tensor& a, const torch::Tensor& b, co
   return output;
 }
 
+// cutlass/nvfp4_scaled_mm_blockscale.cu:332-373
+std::pair<torch::Tensor, torch::Tensor> nvfp4_scaled_mm_blockscale(const torch::Tensor& a, const torch::Tensor& b,
+                                                                   const torch::Tensor& scales_a, const torch::Tensor& scales_b,
+                                                                   const torch::Tensor& alpha,
+                                                                   const torch::Tensor& global_normconst, bool skip_checks) {
+  auto [m, n, k] = validateInputsNvfp4ScaledMm(a, b, scales_a, scales_b, alpha, skip_checks);
+  NVF_CHECK(global_normconst.is_cuda() && global_normconst.scalar_type() == at::ScalarType::Float && global_normconst.numel() == 1,
+            "global_normconst must be a single fp32 value on the device.");
+  c10::DeviceGuard guard(a.device());
+  void* stream = current_stream(a);
+  torch::Tensor output = at::empty({m, ceilDiv(n, 2)}, at::TensorOptions().dtype(at::ScalarType::Float4_e2m1fn_x2).device(a.device()));
+  // The 128x4 layout needs whole 128-row tiles; for m % 128 == 0 this is the reference's [m, roundUp(n/16, 4)].
+  torch::Tensor output_blockscale =
+      at::empty({roundUp(m, 128), roundUp(n / 16, 4)}, at::TensorOptions().dtype(at::ScalarType::Float8_e4m3fn).device(a.device()));
+  torch::Tensor product = at::empty({m, n}, at::TensorOptions().dtype(at::ScalarType::Float).device(a.device()));
+  check_status(nvf_nvfp4_scaled_mm_blockscale(a.data_ptr(), b.data_ptr(), scales_a.data_ptr(), scales_b.data_ptr(),
+                                              static_cast<const float*>(alpha.data_ptr()),
+                                              static_cast<const float*>(global_normconst.data_ptr()), output.data_ptr(),
+                                              output_blockscale.data_ptr(), static_cast<float*>(product.data_ptr()), m, n, k,
+                                              stream),
+               "nvfp4_scaled_mm_blockscale");
+  return {output, output_blockscale};
+}
+
 // cutlass/mxfp8_scaled_mm.cu:290-319
 torch::Tensor mxfp8_scaled_mm(const torch::Tensor& a, const torch::Tensor& b, const torch::Tensor& scales_a,
                               const torch::Tensor& scales_b, const torch::Tensor& alpha, at::ScalarType out_dtype,

@@ -45,6 +45,13 @@ NVF_HOST_API torch::Tensor nvfp4_scaled_mm(const torch::Tensor& a, const torch::
                                            const torch::Tensor& scales_b, const torch::Tensor& alpha,
                                            at::ScalarType out_dtype, bool skip_checks = false);
 
+// cutlass/nvf_cutlass.h:147-154.  The product alpha * dequant(a) @ dequant(b)^T (fp32) quantized again to
+// NVFP4 along N: returns (fp4 [m, n/2], e4m3 block scales in the 128x4 layout of [roundUp(m,128), roundUp(n/16,4)]);
+// global_normconst is the fp32 global (encode) scale of the output.
+NVF_HOST_API std::pair<torch::Tensor, torch::Tensor> nvfp4_scaled_mm_blockscale(
+    const torch::Tensor& a, const torch::Tensor& b, const torch::Tensor& scales_a, const torch::Tensor& scales_b,
+    const torch::Tensor& alpha, const torch::Tensor& global_normconst, bool skip_checks = false);
+
 // cutlass/nvf_cutlass.h:95-101.  Returns (m, n, k) with k = a.size(1).
 NVF_HOST_API std::tuple<int64_t, int64_t, int64_t> validateInputsMxFp8ScaledMm(
     const torch::Tensor& a, const torch::Tensor& b, const torch::Tensor& scales_a, const torch::Tensor& scales_b,

@@ -113,6 +113,16 @@ NVF_API int nvf_nvfp4_scaled_mm(const void* a, const void* b, const void* scales
                                 const float* alpha, void* out, int64_t m, int64_t n, int64_t k,
                                 int out_dtype, void* stream);
 
+/* cutlass/nvfp4_scaled_mm_blockscale.cu:332-373 nvfp4_scaled_mm_blockscale (decl cutlass/nvf_cutlass.h:147-154).
+ *   Operands as nvf_nvfp4_scaled_mm.  The fp32 product alpha * A * B^T is quantized again along n with
+ *   the NVFP4 block quantizer (block 16, global scale *global_normconst): out_fp4 [m, n/2], out_scales
+ *   e4m3 in the 128x4 layout of [roundUp(m,128), roundUp(n/16,4)].  workspace: m * n floats of device
+ *   memory owned by the caller (the product lives there between the two launches). */
+NVF_API int nvf_nvfp4_scaled_mm_blockscale(const void* a, const void* b, const void* scales_a, const void* scales_b,
+                                           const float* alpha, const float* global_normconst, void* out_fp4,
+                                           void* out_scales, float* workspace, int64_t m, int64_t n, int64_t k,
+                                           void* stream);
+
 /* cutlass/mxfp8_scaled_mm.cu:290-319 mxfp8_scaled_mm (shape rules: cutlass/nvf_cutlass.cpp:124-234).
  *   a [m, k], b [n, k] e4m3; scales e8m0 in the 128x4 layout of [roundUp(m|n,128), roundUp(k/32,4)].
  *   k % 16 == 0, n % 16 == 0 (as in the reference); this implementation also needs k % 32 == 0. */

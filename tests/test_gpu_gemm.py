@@ -45,6 +45,70 @@ def test_nvfp4_gemm_reference_shapes(dev, dtype, shape):
     assert max_rel(out, ref) <= GEMM_MAX_REL
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(128, 128, 64), (128, 128, 128), (256, 128, 64), (128, 256, 128)])
+def test_nvfp4_gemm_epilogue_reference_shapes(dev, dtype, shape):
+    """tests/python/direct/test_cutlass_nvfp4_gemm.py:103-175 with its own tolerances: operands quantized
+    from `dtype` data, the expectation is the NVFP4 quantization (global scale 2) of the product rounded to
+    `dtype`; then the tighter statement against the fp32 product."""
+    from fuser_amd import nvf_cutlass
+
+    m, n, packed_k = shape
+    k = packed_k * 2
+    gen = torch.Generator().manual_seed(0)
+    a, sa, ga = _nvfp4_operand(m, k, 1.0, gen)
+    b, sb, gb = _nvfp4_operand(n, k, 1.0, gen)
+    alpha = 1.0 / (ga * gb)
+    norm = 2.0
+    q, sf = nvf_cutlass.nvfp4_scaled_mm_blockscale(fp4(a.to(dev)), fp4(b.to(dev)), e4m3(sa.to(dev)), e4m3(sb.to(dev)),
+                                                   torch.tensor(alpha, dtype=torch.float32, device=dev),
+                                                   torch.tensor(norm, dtype=torch.float32, device=dev))
+    torch.cuda.synchronize()
+    assert q.dtype == torch.float4_e2m1fn_x2 and q.shape == (m, n // 2)
+    assert sf.dtype == torch.float8_e4m3fn and sf.shape == (m, O.round_up(n // 16, 4))
+    q, sf = q.view(torch.uint8).cpu(), sf.view(torch.uint8).cpu()
+    lut, e4 = torch.from_numpy(O.e2m1_table()), torch.from_numpy(O.e4m3_table())
+
+    def unpack(p):
+        return torch.stack([lut[(p & 15).long()], lut[(p >> 4).long()]], dim=-1).reshape(p.shape[0], -1)
+
+    prod = O.ref_nvfp4_scaled_mm(a, b, sa, sb, alpha)
+    eq, esf = O.block_quantize_nvfp4(prod.to(dtype), norm, True)  # the reference test's expectation
+    diff = (unpack(q) - unpack(eq)).abs()
+    assert diff.max() <= 2.0 and (diff != 0).float().mean() < 0.1
+    torch.testing.assert_close(e4[sf.long()], e4[esf.long()], atol=2e-3, rtol=0.125)
+    # against the fp32 product: only a summation-order ulp can flip a code or a scale
+    eq, esf = O.ref_nvfp4_scaled_mm_blockscale(a, b, sa, sb, alpha, norm)
+    assert (unpack(q) != unpack(eq)).float().mean() < 2e-3 and (sf != esf).float().mean() < 2e-3
+
+
+def test_nvfp4_gemm_epilogue_quantizes_its_own_fp32_product_bit_exactly(dev):
+    """Through the C ABI, where the caller owns the workspace: the fp32 product left there agrees with the
+    oracle product to fp32 summation noise, and payload and scales are bit-identical to the oracle
+    quantizer applied to exactly that product (rows not a multiple of 128, scale columns padded)."""
+    from fuser_amd import capi
+
+    m, n, k = 200, 160, 192
+    gen = torch.Generator().manual_seed(11)
+    a, sa, ga = _nvfp4_operand(m, k, 1.0, gen)
+    b, sb, gb = _nvfp4_operand(n, k, 1.0, gen)
+    alpha, norm = 1.0 / (ga * gb), 2688.0 / 40.0
+    d = [t.to(dev) for t in (a, b, sa, sb)]
+    al, nc = torch.tensor(alpha, dtype=torch.float32, device=dev), torch.tensor(norm, dtype=torch.float32, device=dev)
+    q = torch.zeros(m, n // 2, dtype=torch.uint8, device=dev)
+    sf = torch.full((O.round_up(m, 128), O.round_up(n // 16, 4)), 0x55, dtype=torch.uint8, device=dev)
+    ws = torch.zeros(m, n, dtype=torch.float32, device=dev)
+    capi.check(capi.lib().nvf_nvfp4_scaled_mm_blockscale(d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), d[3].data_ptr(), al.data_ptr(),
+                                                         nc.data_ptr(), q.data_ptr(), sf.data_ptr(), ws.data_ptr(), m, n, k, None))
+    torch.cuda.synchronize()
+    prod = O.ref_nvfp4_scaled_mm(a, b, sa, sb, alpha)
+    assert max_rel(ws, prod) <= 1e-5
+    eq, esf = O.block_quantize_nvfp4(ws.cpu(), norm, True)
+    assert torch.equal(q.cpu(), eq)
+    valid = O.linear_to_swizzled_128_4(torch.ones(m, n // 16, dtype=torch.uint8)) != 0
+    assert torch.equal(sf.cpu()[valid], esf[valid])
+
+
 def test_config1_quantize_then_gemm(dev):
     """BASELINE config 1: A [256,1024], B [1024,1024] N(0,1) bf16, quantized on the GPU, C = A B^T bf16."""
     from fuser_amd import nvf_cutlass, ops
