@@ -28,6 +28,8 @@ def test_dense_validators_reject_cpu_tensors_and_bad_ranks():
     a, b, sa, sb, alpha = _nvfp4_args()
     with pytest.raises(RuntimeError, match="must be a CUDA tensor and contiguous"):
         nvf_cutlass.nvfp4_scaled_mm(a, b, sa, sb, alpha, torch.bfloat16)
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor and contiguous"):
+        nvf_cutlass.nvfp4_scaled_mm_blockscale(a, b, sa, sb, alpha, torch.tensor(2.0))
     with pytest.raises(RuntimeError, match="Operand A must be a matrix"):
         nvf_cutlass.validate_inputs_nvfp4_scaled_mm(a[0], b, sa, sb, alpha)
     with pytest.raises(RuntimeError, match="cannot be multiplied"):
