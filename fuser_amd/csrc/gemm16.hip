@@ -70,19 +70,19 @@ __device__ __forceinline__ void dequant32(const u32x4 q, uint32_t sf2, u32x4 out
   }
 }
 
-// LDS tile: rows x 64 16-bit elements (128 bytes per row); 16-byte chunk c of row r sits at
-// chunk position c ^ (r & 7) so that both the staging writes and the MFMA fragment reads of
-// 8 consecutive lanes fall into distinct banks.
-__device__ __forceinline__ int lds_pos(int row, int chunk) { return row * 8 + (chunk ^ (row & 7)); }
+// LDS tile: rows x 64 16-bit elements (128 bytes per row); 16-byte chunk c of row r sits at chunk
+// position c ^ ((r >> 1) & 7): two rows fill the 64 banks once, so the MFMA fragment reads (16
+// consecutive lanes = 16 consecutive rows, one chunk) are conflict-free.
+__device__ __forceinline__ int lds_pos2(int row, int chunk) { return row * 8 + (chunk ^ ((row >> 1) & 7)); }
+__device__ __forceinline__ int lds_pos(int row, int chunk) { return lds_pos2(row, chunk); }
 
 template <int BM, int BN, bool NVFP4, bool BF16_MMA, bool OUT_BF16, bool OUT_F32 = false>
 __global__ __launch_bounds__(256) void gemm16_kernel(const Params p) {
   constexpr int BK = 64;
   constexpr int WTM = BM / 2, WTN = BN / 2;  // wave tile
   constexpr int TM = WTM / 32, TN = WTN / 32;
-  extern __shared__ u32x4 lds[];
-  u32x4* lds_a = lds;
-  u32x4* lds_b = lds + BM * 8;
+  extern __shared__ u32x4 lds[];  // two buffers of (A tile, B tile)
+  constexpr int BUF_UNITS = (BM + BN) * 8;
   __shared__ int tile_prefix[kMaxGroups + 1];
 
   const int tid = threadIdx.x;
@@ -205,7 +205,9 @@ __global__ __launch_bounds__(256) void gemm16_kernel(const Params p) {
       }
     };
 
-    auto store_lds = [&]() {
+    auto store_lds = [&](int buf) {
+      u32x4* lds_a = lds + buf * BUF_UNITS;
+      u32x4* lds_b = lds_a + BM * 8;
 #pragma unroll
       for (int i = 0; i < A_CH; ++i) {
         const int c = tid + 256 * i;
@@ -236,11 +238,14 @@ __global__ __launch_bounds__(256) void gemm16_kernel(const Params p) {
       }
     };
 
+    // K loop: the loads of step ks+1 are in flight under the MFMAs of step ks, then converted into the
+    // other LDS buffer; one barrier per step
     issue_loads(0);
+    store_lds(0);  // every wave is past the barrier that ended the previous tile's last step
+    __syncthreads();
     for (int ks = 0; ks < nk; ++ks) {
-      __syncthreads();  // previous step's fragment reads are done
-      store_lds();
-      __syncthreads();
+      const u32x4* lds_a = lds + (ks & 1) * BUF_UNITS;
+      const u32x4* lds_b = lds_a + BM * 8;
       if (ks + 1 < nk) issue_loads(ks + 1);
 
 #pragma unroll
@@ -264,6 +269,8 @@ __global__ __launch_bounds__(256) void gemm16_kernel(const Params p) {
             }
           }
       }
+      if (ks + 1 < nk) store_lds((ks + 1) & 1);
+      __syncthreads();
     }
 
     // ---- epilogue: acc[i][j][r] = C[m = lane%32][n = (r/4)*8 + (lane/32)*4 + r%4] of its 32x32 tile ----
@@ -323,8 +330,6 @@ __global__ __launch_bounds__(256) void gemm16_kernel(const Params p) {
 // LDS: two buffers of (A tile + B tile), each tile 256 rows x 128 bytes with 16-byte chunk c of row r at
 // chunk position c ^ ((r >> 1) & 7): conflict-free for the fragment reads.
 // -------------------------------------------------------------------------------------------------
-__device__ __forceinline__ int lds_pos2(int row, int chunk) { return row * 8 + (chunk ^ ((row >> 1) & 7)); }
-
 template <bool OUT_BF16>
 __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   constexpr int BM = 256, BN = 256;
@@ -987,7 +992,7 @@ int launch_grouped16_fast(const Params& p, int cus, hipStream_t stream) {
 template <int BM, int BN, bool NVFP4, bool BF16_MMA, bool OUT_BF16, bool OUT_F32 = false>
 int launch_cfg(const Params& p, int grid, hipStream_t stream) {
   auto kern = gemm16_kernel<BM, BN, NVFP4, BF16_MMA, OUT_BF16, OUT_F32>;
-  constexpr int lds_bytes = (BM + BN) * 128;
+  constexpr int lds_bytes = 2 * (BM + BN) * 128;
   static bool configured = false;  // benign race: the attribute call is idempotent
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
@@ -1014,7 +1019,8 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, hipStream_t stream) {
         p.k >= 128 && (int64_t)p.k * 2 * 256 < (1ll << 31))
       return launch_grouped16_fast<BF16_MMA, OUT_BF16>(p, cus, stream);
   }
-  if (tiles(256, 256) >= cus || (!dense && m_hint >= 256 * (int64_t)p.groups)) {
+  // grouped: the tile height follows the average group (a 256-row tile on a 77-row group is mostly padding)
+  if (dense ? tiles(256, 256) >= cus : m_hint >= 512 * (int64_t)p.groups) {
     const int64_t upper = dense ? tiles(256, 256) : (ceil_div(p.m, 256) + p.groups) * ceil_div(p.n, 256);
     return launch_cfg<256, 256, NVFP4, BF16_MMA, OUT_BF16>(p, (int)(upper < cus ? upper : cus), stream);
   }
