@@ -717,9 +717,9 @@ int launch_nvfp4_skinny_cfg(const Params& p, hipStream_t stream) {
 
 template <int TT, bool OUT_BF16>
 int launch_nvfp4_skinny_tt(const Params& p, int cus, hipStream_t stream) {
-  // More weight rows per workgroup convert the activations less often; keep enough workgroups to fill
-  // the chip (small activation tiles leave room for several workgroups per compute unit).
-  const int64_t want = (int64_t)cus * (TT >= 8 ? 3 : TT >= 4 ? 4 : 8) / 4;
+  // The conversion work bounds this kernel, and every workgroup converts all activation rows it uses:
+  // take as many weight rows per workgroup as still leaves about one workgroup per compute unit.
+  const int64_t want = (int64_t)cus * 4 / 5;
   if ((p.n & 63) == 0 && p.n / 64 >= want) return launch_nvfp4_skinny_cfg<4, TT, OUT_BF16>(p, stream);
   if ((p.n & 31) == 0 && p.n / 32 >= want) return launch_nvfp4_skinny_cfg<2, TT, OUT_BF16>(p, stream);
   return launch_nvfp4_skinny_cfg<1, TT, OUT_BF16>(p, stream);
