@@ -900,7 +900,10 @@ __global__ __launch_bounds__(256, 1) void grouped16_gemm_256_kernel(const Params
 
   Frags f0, f1;  // fragments of the first / second half (K 0..31 / 32..63) of a step
 
-  np = (first_tile + slots < range_end && nk == 1) ? tile_info(first_tile + slots) : lp;
+  // The stream runs two steps ahead of the MFMAs; with two steps per tile it is a whole tile ahead and
+  // already leaves the first tile during this prologue.
+  const int tiles_ahead = nk == 2 ? 2 : 1;
+  np = (first_tile + slots < range_end) ? tile_info(first_tile + slots) : lp;
 #pragma unroll
   for (int q = 0; q < 16; ++q) issue_step_unit(q);  // step 0
   issue_step_tail();
@@ -916,9 +919,9 @@ __global__ __launch_bounds__(256, 1) void grouped16_gemm_256_kernel(const Params
   int g = 0;
   Tile ct = tile_info(first_tile);
   for (int c_tile = first_tile; c_tile < range_end; c_tile += slots) {
-    // the stream is inside this tile by now; prepare the tile it will enter two steps before the end
+    // prepare the tile the stream enters next (past the end of the list: any valid tile, loaded and ignored)
     const Tile nt_info = (c_tile + slots < range_end) ? tile_info(c_tile + slots) : ct;
-    np = nt_info;
+    np = (c_tile + tiles_ahead * slots < range_end) ? tile_info(c_tile + tiles_ahead * slots) : ct;
     for (int c_ks = 0; c_ks < nk; ++c_ks, ++g) {
       const int buf = g & 1;
       // ---- first half: MFMAs on f0, interleaved with the LDS reads that fill f1

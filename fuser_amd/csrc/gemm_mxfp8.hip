@@ -354,6 +354,10 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
   u32x4 wa, wb;      // scales of the step being computed, shifted for this lane group
   u32x4 na, nb;      // scales of the next step
 
+  // The stream runs two steps ahead of the MFMAs; with two steps per tile it is a whole tile ahead and
+  // already leaves the first tile during this prologue.
+  const int tiles_ahead = nk == 2 ? 2 : 1;
+  np = (first_tile + slots < range_end) ? tile_ptrs(first_tile + slots) : lp;
 #pragma unroll
   for (int q = 0; q < 16; ++q) issue_step_unit(q);  // step 0
   issue_step_tail();
@@ -372,7 +376,7 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
   int g = 0;
   for (int c_tile = first_tile; c_tile < range_end; c_tile += slots) {
     // the stream is inside this tile by now; prepare the tile it will enter two steps before the end
-    np = (c_tile + slots < range_end) ? tile_ptrs(c_tile + slots) : lp;
+    np = (c_tile + tiles_ahead * slots < range_end) ? tile_ptrs(c_tile + tiles_ahead * slots) : lp;
     for (int c_ks = 0; c_ks < nk; ++c_ks, ++g) {
       const int buf = g & 1;
       // ---- first half: MFMAs on f0, interleaved one-to-one with the LDS reads that fill f1

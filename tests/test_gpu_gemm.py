@@ -258,11 +258,13 @@ def test_mxfp8_gemm_ragged_shapes_alpha_and_scale_spread(dev, shape):
         assert err <= GEMM_MAX_REL, (shape, dtype, err)
 
 
-@pytest.mark.parametrize("shape", [(4096, 2048, 512), (2560, 3328, 384), (2048, 4096, 256), (8192, 1024, 1152)])
+@pytest.mark.parametrize("shape", [(4096, 2048, 512), (2560, 3328, 384), (2048, 4096, 256), (8192, 1024, 1152),
+                                   (4096, 8192, 256), (8192, 4096, 384), (4352, 4096, 128 * 5)])
 def test_nvfp4_gemm_persistent_256_tile_kernel_full_compare(dev, shape):
     """Dense shapes with M % 256 == N % 256 == K % 128 == 0 and at least 128 tiles take the persistent
     kernel that converts the operands to fp16 between its MFMAs; every output element is compared with
-    the oracle.  Same tile-grid cases as the MXFP8 test below."""
+    the oracle.  Same tile-grid cases as the MXFP8 test below (incl. several tiles per workgroup with two,
+    three and five 128-deep spans per tile)."""
     m, n, k = shape
     gen = torch.Generator().manual_seed(k + 1)
     a, sa, ga = _nvfp4_operand(m, k, 1.0, gen)
@@ -297,12 +299,14 @@ def test_nvfp4_gemm_persistent_kernel_every_scale_code_is_decoded_exactly(dev, s
     assert ((out.float().cpu() - ref).abs() / scale).max().item() <= 2.0 ** -7
 
 
-@pytest.mark.parametrize("shape", [(4096, 2048, 512), (2560, 3328, 384), (2048, 4096, 256), (8192, 1024, 1152)])
+@pytest.mark.parametrize("shape", [(4096, 2048, 512), (2560, 3328, 384), (2048, 4096, 256), (8192, 1024, 1152),
+                                   (4096, 8192, 256), (8192, 4096, 384), (4352, 4096, 640)])
 def test_mxfp8_gemm_persistent_256_tile_kernel_full_compare(dev, shape):
     """Shapes with M % 256 == N % 256 == K % 128 == 0 and at least 128 tiles take the persistent
     LDS-direct kernel; every output element is compared with the oracle.  (2560, 3328) has a tile grid
-    that is not a multiple of the 8 x 4 blocking, (8192, 1024) gives some workgroups two tiles and K
-    steps that wrap the load stream across tiles."""
+    that is not a multiple of the 8 x 4 blocking; the 512- and 272-tile shapes give every workgroup two
+    (or one and two) tiles, so that the load stream wraps across tiles, with two, three and five K steps
+    or spans per tile."""
     m, n, k = shape
     gen = torch.Generator().manual_seed(k)
     a, sa = _mxfp8_operand(m, k, gen, 1.0)

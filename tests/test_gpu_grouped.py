@@ -61,15 +61,17 @@ def test_grouped_mm_empty_groups_and_untouched_rows(dev):
     assert max_rel(out[:200], ref[:200]) <= GEMM_MAX_REL
 
 
-@pytest.mark.parametrize("tensor_dtype,k", [(torch.bfloat16, 192), (torch.float16, 128), (torch.bfloat16, 1088)])
-def test_grouped_mm_persistent_256_tile_kernel_full_compare(dev, tensor_dtype, k):
+@pytest.mark.parametrize("tensor_dtype,k,n", [(torch.bfloat16, 192, 2048), (torch.float16, 128, 2048), (torch.bfloat16, 1088, 2048),
+                                              (torch.bfloat16, 128, 4096), (torch.float16, 192, 4096)])
+def test_grouped_mm_persistent_256_tile_kernel_full_compare(dev, tensor_dtype, k, n):
     """Large enough for the persistent LDS-direct kernel (N % 256 == 0, K % 64 == 0, >= 256 rows per
     group on average): groups that end inside a tile, an empty group, a one-row group and a group of
-    257 rows; every output element compared, rows past the last group untouched."""
+    257 rows; every output element compared, rows past the last group untouched.  N = 4096 gives 288
+    tiles, i.e. two tiles for some workgroups, with two and three K steps per tile."""
     from fuser_amd import capi
 
     sizes = [1000, 0, 1791, 257, 1, 1000]
-    m, n = sum(sizes) + 47, 2048
+    m = sum(sizes) + 47
     gen = torch.Generator().manual_seed(k)
     a = torch.randn(m, k, generator=gen).to(tensor_dtype)
     b = (torch.randn(len(sizes), n, k, generator=gen) * 0.05).to(tensor_dtype)
