@@ -589,6 +589,13 @@ int launch_nvfp4_fast(const Params& p, int cus, hipStream_t stream) {
 // -------------------------------------------------------------------------------------------------
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
+// LDS-direct load.  lds_byte_addr and base are wave-uniform; lane L's 16 bytes land at lds_byte_addr + 16 * L.
+// Issued from inline assembly: the compiler neither waits for it nor orders LDS reads against it, the
+// kernels do that with explicit s_waitcnt vmcnt(n).
+__device__ __forceinline__ void lds_dma16(uint32_t lds_byte_addr, const uint8_t* base, uint32_t voff) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_byte_addr), "v"(voff), "s"(base) : "memory");
+}
+
 // 32 packed e2m1 values and their two e4m3 block scales -> four MFMA operands of 8 fp16 values
 __device__ __forceinline__ void dequant_frags(const u32x4 q, uint32_t s2, u32x4 out[4]) {
   const float f0 = __builtin_amdgcn_cvt_f32_fp8((int)s2, 0), f1 = __builtin_amdgcn_cvt_f32_fp8((int)s2, 1);
@@ -700,6 +707,174 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_kernel(const Params p) {
   }
 }
 
+// Variant for few activation rows (M <= 32).  A load in MFMA lane order (lane = row % 16 + 16 * piece)
+// touches 64 unrelated 16-byte pieces and occupies the address unit for 64 cycles, which - not HBM, not
+// latency - bounds the plain kernel above.  Here the tiles are fetched with LDS-direct loads in memory
+// order (4 neighbouring lanes = 64 contiguous bytes of a row; scales as the 256 contiguous bytes that
+// hold a 16-row tile's scale words) into a private LDS ring of each wavefront and read back in MFMA
+// order; no barrier is involved because a wavefront only reads what it loaded itself.
+//   LDS per slot: NT payload tiles of 16 rows x 64 B, piece p of row r at piece position p ^ ((r >> 2) & 3)
+//   (conflict-free reads), then per operand one 1 KiB scale block per pair of tiles: [tile][col tile][row][16 B].
+template <int RT, int TT, bool OUT_BF16>
+__global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) {
+  constexpr int W = 8;
+  constexpr int NT = RT + TT;
+  constexpr int B_SC = (RT + 1) / 2, A_SC = (TT + 1) / 2;     // scale blocks (1 KiB) per operand
+  constexpr int SLOT_BYTES = (NT + B_SC + A_SC) * 1024;
+  constexpr int NDMA = NT + B_SC + A_SC;                      // loads per chunk and wavefront
+  constexpr int DEPTH = 2;
+  static_assert(DEPTH == 2 && W * DEPTH * SLOT_BYTES <= 128 * 1024 && DEPTH * NDMA <= 63, "ring does not fit");
+  extern __shared__ f32x4 red[];  // ring during the K loop, then [W][tiles][64 lanes] partial sums
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * (16 * RT);
+  const int tt_count = (p.m + 15) >> 4;
+  const int kbytes = p.k >> 1;
+  const int chunks = p.k >> 7;
+  const int sf_padded = p.k >> 4;  // K % 128 == 0: no padding columns
+
+  // ---- load side (memory order): lane L fetches row L/4, piece (L%4) ^ ((L/16)&3) of a payload tile
+  const int lrow = lane >> 2, lpiece = (lane & 3) ^ ((lane >> 4) & 3);
+  const uint8_t* b_base = p.b + (int64_t)n0 * kbytes;
+  const uint8_t* bsf_base = p.sfb + swizzle_128x4(n0 & ~127, 0, sf_padded);
+  uint32_t b_off[RT], a_off[TT], bsf_off[B_SC], asf_off[A_SC];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) b_off[rt] = (uint32_t)(rt * 16 + lrow) * (uint32_t)kbytes + lpiece * 16;
+#pragma unroll
+  for (int tt = 0; tt < TT; ++tt) a_off[tt] = (uint32_t)min(tt * 16 + lrow, p.m - 1) * (uint32_t)kbytes + lpiece * 16;
+  // scale block j of an operand: lane L = tile 2j + (L>>5), col tile (L>>4)&1, row L&15: the 16 bytes that
+  // hold the scale words of rows {row, row+32, row+64, row+96} (mod 128) for that col tile
+#pragma unroll
+  for (int j = 0; j < B_SC; ++j) {
+    const int t = min(2 * j + (lane >> 5), RT - 1);
+    const int row = (n0 & 127) + t * 16 + (lane & 15);
+    bsf_off[j] = (uint32_t)((row & 31) * 16 + ((lane >> 4) & 1) * 512);
+  }
+#pragma unroll
+  for (int j = 0; j < A_SC; ++j) {
+    const int t = min(2 * j + (lane >> 5), TT - 1);
+    const int row = t * 16 + (lane & 15);  // < 128: inside the first 128-row tile of the activations' scales
+    asf_off[j] = (uint32_t)((row & 31) * 16 + ((lane >> 4) & 1) * 512);
+  }
+  const uint32_t lds_base = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)red);
+  const uint32_t ring_base = lds_base + (uint32_t)wave * (DEPTH * SLOT_BYTES);
+  auto issue_chunk = [&](int c_in, int slot) {  // c_in is wave-uniform
+    if (c_in >= chunks) return;
+    const uint32_t c = (uint32_t)c_in;
+    const uint32_t sb = ring_base + (uint32_t)slot * SLOT_BYTES;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) lds_dma16(sb + rt * 1024, b_base, b_off[rt] + c * 64u);
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) lds_dma16(sb + (RT + tt) * 1024, p.a, a_off[tt] + c * 64u);
+#pragma unroll
+    for (int j = 0; j < B_SC; ++j) lds_dma16(sb + (NT + j) * 1024, bsf_base, bsf_off[j] + c * 1024u);
+#pragma unroll
+    for (int j = 0; j < A_SC; ++j) lds_dma16(sb + (NT + B_SC + j) * 1024, p.sfa, asf_off[j] + c * 1024u);
+  };
+
+  // ---- read side (MFMA order): lane (r, g) = row r, payload piece g, scale blocks 2g, 2g+1 of the chunk
+  const int rd_payload = r * 64 + ((g ^ ((r >> 2) & 3)) * 16);
+  int rd_bsc[RT], rd_asc[TT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const int rowgroup = (((n0 & 127) + rt * 16) >> 5) & 3;  // which of the 4 words of the 16 bytes
+    rd_bsc[rt] = (NT + (rt >> 1)) * 1024 + ((rt & 1) * 2 + (g >> 1)) * 256 + r * 16 + rowgroup * 4;
+  }
+#pragma unroll
+  for (int tt = 0; tt < TT; ++tt)
+    rd_asc[tt] = (NT + B_SC + (tt >> 1)) * 1024 + ((tt & 1) * 2 + (g >> 1)) * 256 + r * 16 + ((tt * 16) >> 5) * 4;
+  const int sc_shift = (g & 1) * 16;
+
+  f32x4 acc[RT][TT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) acc[rt][tt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d) issue_chunk(wave + d * W, d);
+  int slot = 0;
+  for (int c = wave; c < chunks; c += W) {
+    // the oldest chunk in flight has landed when only the loads of the next one (if there is one) are pending
+    if (c + W < chunks)
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NDMA) : "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    const char* sp = reinterpret_cast<const char*>(red) + (wave * DEPTH + slot) * SLOT_BYTES;
+    u32x4 q[NT];
+    uint32_t sc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) q[t] = *reinterpret_cast<const u32x4*>(sp + t * 1024 + rd_payload);
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) sc[rt] = *reinterpret_cast<const uint32_t*>(sp + rd_bsc[rt]) >> sc_shift;
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) sc[RT + tt] = *reinterpret_cast<const uint32_t*>(sp + rd_asc[tt]) >> sc_shift;
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // read out: the slot may be refilled
+    issue_chunk(c + DEPTH * W, slot);
+    slot ^= 1;
+    u32x4 fb[RT][4];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) dequant_frags(q[rt], sc[rt], fb[rt]);
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) {
+      if (tt < tt_count) {
+        u32x4 fa[4];
+        dequant_frags(q[RT + tt], sc[RT + tt], fa);
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt)
+            acc[rt][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, fb[rt][t]),
+                                                                 __builtin_bit_cast(f16x8, fa[t]), acc[rt][tt], 0, 0, 0);
+      }
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no LDS-direct load may be pending when the ring is reused
+  __syncthreads();
+
+  // ---- all partial tiles in one round (RT * TT <= 8): sum in wave order and store
+  const float alpha = p.alpha[0];
+  uint16_t* out = static_cast<uint16_t*>(p.out);
+  const int tiles = RT * tt_count;  // tile index: rt * tt_count + tt
+  const int units = tiles * 64;
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt)
+      if (tt < tt_count) red[(wave * tiles + rt * tt_count + tt) * 64 + lane] = acc[rt][tt];
+  __syncthreads();
+  for (int u = tid; u < units; u += 512) {
+    const int l = u & 63, tile = u >> 6;
+    const int rt = tile / tt_count, tt = tile - rt * tt_count;
+    f32x4 s = red[u];
+#pragma unroll
+    for (int w = 1; w < W; ++w) s += red[w * units + u];
+    const int tok = tt * 16 + (l & 15);
+    if (tok < p.m) {
+      u32x2 v;
+      v[0] = pack2(s[0] * alpha, s[1] * alpha, OUT_BF16);
+      v[1] = pack2(s[2] * alpha, s[3] * alpha, OUT_BF16);
+      *reinterpret_cast<u32x2*>(out + (int64_t)tok * p.n + n0 + rt * 16 + 4 * (l >> 4)) = v;
+    }
+  }
+}
+
+template <int RT, int TT, bool OUT_BF16>
+int launch_nvfp4_skinny_ring_cfg(const Params& p, hipStream_t stream) {
+  auto kern = nvfp4_skinny_ring_kernel<RT, TT, OUT_BF16>;
+  constexpr int lds_bytes = 8 * 2 * (RT + TT + (RT + 1) / 2 + (TT + 1) / 2) * 1024;  // >= the 8 * RT * TT KiB of the reduction
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    if (e != hipSuccess) return fail(NVF_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    configured = true;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)(p.n / (16 * RT))), dim3(512), lds_bytes, stream, p);
+  return check_launch("nvfp4_skinny_ring_kernel");
+}
+
 template <int RT, int TT, bool OUT_BF16>
 int launch_nvfp4_skinny_cfg(const Params& p, hipStream_t stream) {
   auto kern = nvfp4_skinny_kernel<RT, TT, OUT_BF16>;
@@ -720,6 +895,15 @@ int launch_nvfp4_skinny_tt(const Params& p, int cus, hipStream_t stream) {
   // The conversion work bounds this kernel, and every workgroup converts all activation rows it uses:
   // take as many weight rows per workgroup as still leaves about one workgroup per compute unit.
   const int64_t want = (int64_t)cus * 4 / 5;
+  if constexpr (TT <= 2) {
+    if ((int64_t)p.k * 64 < (1ll << 31)) {  // 32-bit lane offsets
+      if constexpr (TT == 1) {
+        if ((p.n & 63) == 0 && p.n / 64 >= want) return launch_nvfp4_skinny_ring_cfg<4, TT, OUT_BF16>(p, stream);
+      }
+      if ((p.n & 31) == 0 && p.n / 32 >= want) return launch_nvfp4_skinny_ring_cfg<2, TT, OUT_BF16>(p, stream);
+      return launch_nvfp4_skinny_ring_cfg<1, TT, OUT_BF16>(p, stream);
+    }
+  }
   if ((p.n & 63) == 0 && p.n / 64 >= want) return launch_nvfp4_skinny_cfg<4, TT, OUT_BF16>(p, stream);
   if ((p.n & 31) == 0 && p.n / 32 >= want) return launch_nvfp4_skinny_cfg<2, TT, OUT_BF16>(p, stream);
   return launch_nvfp4_skinny_cfg<1, TT, OUT_BF16>(p, stream);
@@ -746,11 +930,6 @@ int launch_nvfp4_skinny(const Params& p, int cus, hipStream_t stream) {
 //     under the 32 MFMAs of the current one; one barrier per K step.
 // LDS layout as in the NVFP4 fast path: chunk c of row r at chunk position c ^ ((r >> 1) & 7).
 // -------------------------------------------------------------------------------------------------
-__device__ __forceinline__ void lds_dma16(uint32_t lds_byte_addr, const uint8_t* base, uint32_t voff) {
-  // lds_byte_addr and base are wave-uniform; lane L's 16 bytes land at lds_byte_addr + 16 * L
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_byte_addr), "v"(voff), "s"(base) : "memory");
-}
-
 template <bool BF16_MMA, bool OUT_BF16>
 __global__ __launch_bounds__(256, 1) void grouped16_gemm_256_kernel(const Params p) {
   constexpr int BM = 256, BN = 256;
