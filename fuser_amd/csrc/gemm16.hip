@@ -581,7 +581,7 @@ int launch_nvfp4_fast(const Params& p, int cus, hipStream_t stream) {
 //   * A workgroup owns 16*RT weight rows for the whole of K and all M activation rows; its 8
 //     wavefronts split K in interleaved 128-element chunks and their partial sums are added in a fixed
 //     order through LDS (no atomics, no workspace, deterministic).
-//   * Nothing is staged through LDS: in v_mfma_f32_16x16x32_f16 lane (i, g) supplies 8 elements of row i,
+//   * In v_mfma_f32_16x16x32_f16 lane (i, g) supplies 8 elements of row i,
 //     and both operands use the same (lane group, element) -> k assignment, so a lane loads the 16
 //     payload bytes [32g, 32g+32) of its row's chunk, converts them to fp16 in registers and feeds MFMA
 //     t = 0..3 with elements 8t..8t+7.  Weight rows are the first operand (output rows), activation rows
@@ -707,7 +707,7 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_kernel(const Params p) {
   }
 }
 
-// Variant for few activation rows (M <= 32).  A load in MFMA lane order (lane = row % 16 + 16 * piece)
+// Variant for few activation rows (M <= 64).  A load in MFMA lane order (lane = row % 16 + 16 * piece)
 // touches 64 unrelated 16-byte pieces and occupies the address unit for 64 cycles, which - not HBM, not
 // latency - bounds the plain kernel above.  Here the tiles are fetched with LDS-direct loads in memory
 // order (4 neighbouring lanes = 64 contiguous bytes of a row; scales as the 256 contiguous bytes that
@@ -723,7 +723,7 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
   constexpr int SLOT_BYTES = (NT + B_SC + A_SC) * 1024;
   constexpr int NDMA = NT + B_SC + A_SC;                      // loads per chunk and wavefront
   constexpr int DEPTH = 2;
-  static_assert(DEPTH == 2 && W * DEPTH * SLOT_BYTES <= 128 * 1024 && DEPTH * NDMA <= 63, "ring does not fit");
+  static_assert(DEPTH == 2 && W * DEPTH * SLOT_BYTES <= 160 * 1024 && DEPTH * NDMA <= 63, "ring does not fit");
   extern __shared__ f32x4 red[];  // ring during the K loop, then [W][tiles][64 lanes] partial sums
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -895,17 +895,21 @@ int launch_nvfp4_skinny_tt(const Params& p, int cus, hipStream_t stream) {
   // The conversion work bounds this kernel, and every workgroup converts all activation rows it uses:
   // take as many weight rows per workgroup as still leaves about one workgroup per compute unit.
   const int64_t want = (int64_t)cus * 4 / 5;
+  const bool rt4 = (p.n & 63) == 0 && p.n / 64 >= want, rt2 = (p.n & 31) == 0 && p.n / 32 >= want;
+  // The ring variant wins wherever its LDS ring fits the tile counts, except that with four activation
+  // tiles it cannot take four weight-row tiles, which matter more (measured).
+  const bool ring_ok = (int64_t)p.k * 64 < (1ll << 31);  // 32-bit lane offsets
   if constexpr (TT <= 2) {
-    if ((int64_t)p.k * 64 < (1ll << 31)) {  // 32-bit lane offsets
-      if constexpr (TT == 1) {
-        if ((p.n & 63) == 0 && p.n / 64 >= want) return launch_nvfp4_skinny_ring_cfg<4, TT, OUT_BF16>(p, stream);
-      }
-      if ((p.n & 31) == 0 && p.n / 32 >= want) return launch_nvfp4_skinny_ring_cfg<2, TT, OUT_BF16>(p, stream);
+    if (ring_ok && rt4) return launch_nvfp4_skinny_ring_cfg<4, TT, OUT_BF16>(p, stream);
+  }
+  if constexpr (TT <= 4) {
+    if (ring_ok && !(TT == 4 && rt4)) {
+      if (rt2) return launch_nvfp4_skinny_ring_cfg<2, TT, OUT_BF16>(p, stream);
       return launch_nvfp4_skinny_ring_cfg<1, TT, OUT_BF16>(p, stream);
     }
   }
-  if ((p.n & 63) == 0 && p.n / 64 >= want) return launch_nvfp4_skinny_cfg<4, TT, OUT_BF16>(p, stream);
-  if ((p.n & 31) == 0 && p.n / 32 >= want) return launch_nvfp4_skinny_cfg<2, TT, OUT_BF16>(p, stream);
+  if (rt4) return launch_nvfp4_skinny_cfg<4, TT, OUT_BF16>(p, stream);
+  if (rt2) return launch_nvfp4_skinny_cfg<2, TT, OUT_BF16>(p, stream);
   return launch_nvfp4_skinny_cfg<1, TT, OUT_BF16>(p, stream);
 }
 
