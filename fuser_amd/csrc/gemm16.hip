@@ -9,9 +9,11 @@
 // they are staged into LDS and fed to v_mfma_f32_32x32x16_f16 with fp32 accumulation.  Every
 // product is exact; only the fp32 accumulation order differs from any other correct implementation.
 //
-// All three ops share one kernel: a persistent workgroup walks (group, m-tile, n-tile) work items
-// whose list is derived on the device from problem_sizes, so no host synchronisation is needed and
-// empty groups cost nothing.  The dense op is the one-group case.
+// The tile kernels (one for 16-bit operands, one for NVFP4) are persistent: a workgroup walks (group,
+// m-tile, n-tile) work items whose list is derived on the device from problem_sizes, so no host
+// synchronisation is needed and empty groups cost nothing.  The dense op is the one-group case.
+// Specialised kernels take the shapes they fit: 256x256 persistent NVFP4 and grouped 16-bit kernels,
+// and a weight-streaming NVFP4 kernel for up to 128 activation rows.
 //
 // Output layout trick: the MFMA is issued with the B fragment as first operand, so that a lane's
 // accumulator registers hold 4 consecutive N-elements of one output row and are stored as 8 bytes.
@@ -26,6 +28,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kMaxGroups = 1024;  // same bound as the reference's <<<1, num_experts>>> set-up kernel
 
@@ -53,30 +56,13 @@ __device__ __forceinline__ uint32_t pack2(float a, float b, bool out_bf16) {
   return __builtin_bit_cast(uint32_t, v);
 }
 
-// 32 packed e2m1 values (16 bytes) times two e4m3 block scales -> 32 fp16 values (4 x 16 bytes)
-__device__ __forceinline__ void dequant32(const u32x4 q, uint32_t sf2, u32x4 out[4]) {
-  const _Float16 s0 = (_Float16)e4m3_to_f32(sf2 & 0xffu);
-  const _Float16 s1 = (_Float16)e4m3_to_f32((sf2 >> 8) & 0xffu);
-#pragma unroll
-  for (int w = 0; w < 4; ++w) {  // dword w holds elements 8w .. 8w+7 ; block = w / 2
-    const _Float16 s = (w < 2) ? s0 : s1;
-    const f16x2 sv = {s, s};
-    f16x2 h0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(q[w], 1.0f, 0) * sv;
-    f16x2 h1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(q[w], 1.0f, 1) * sv;
-    f16x2 h2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(q[w], 1.0f, 2) * sv;
-    f16x2 h3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(q[w], 1.0f, 3) * sv;
-    out[w] = u32x4{__builtin_bit_cast(uint32_t, h0), __builtin_bit_cast(uint32_t, h1), __builtin_bit_cast(uint32_t, h2),
-                   __builtin_bit_cast(uint32_t, h3)};
-  }
-}
-
 // LDS tile: rows x 64 16-bit elements (128 bytes per row); 16-byte chunk c of row r sits at chunk
 // position c ^ ((r >> 1) & 7): two rows fill the 64 banks once, so the MFMA fragment reads (16
 // consecutive lanes = 16 consecutive rows, one chunk) are conflict-free.
 __device__ __forceinline__ int lds_pos2(int row, int chunk) { return row * 8 + (chunk ^ ((row >> 1) & 7)); }
 __device__ __forceinline__ int lds_pos(int row, int chunk) { return lds_pos2(row, chunk); }
 
-template <int BM, int BN, bool NVFP4, bool BF16_MMA, bool OUT_BF16, bool OUT_F32 = false>
+template <int BM, int BN, bool BF16_MMA, bool OUT_BF16>
 __global__ __launch_bounds__(256) void gemm16_kernel(const Params p) {
   constexpr int BK = 64;
   constexpr int WTM = BM / 2, WTN = BN / 2;  // wave tile
@@ -124,9 +110,7 @@ __global__ __launch_bounds__(256) void gemm16_kernel(const Params p) {
   __syncthreads();
   const int total_tiles = tile_prefix[p.groups];
 
-  const int kbytes = NVFP4 ? p.k / 2 : p.k * 2;     // bytes per operand row
-  const int sf_cols = p.k / 16;
-  const int sf_padded = (sf_cols + 3) & ~3;
+  const int kbytes = p.k * 2;  // bytes per operand row
   const int nk = (p.k + BK - 1) / BK;
 
   for (int tile = blockIdx.x; tile < total_tiles; tile += gridDim.x) {
@@ -149,13 +133,6 @@ __global__ __launch_bounds__(256) void gemm16_kernel(const Params p) {
 
     const uint8_t* a_base = p.a + (row_off + m0) * (int64_t)kbytes;
     const uint8_t* b_base = p.b + ((int64_t)g * p.n + n0) * (int64_t)kbytes;
-    const uint8_t* sfa_base = nullptr;
-    const uint8_t* sfb_base = nullptr;
-    if constexpr (NVFP4) {
-      const int64_t sf_row_off = dense ? 0 : p.sf_offsets[g];
-      sfa_base = p.sfa + sf_row_off * sf_cols;           // group slab, swizzled on its own
-      sfb_base = p.sfb + (int64_t)g * p.n * sf_cols;
-    }
 
     f32x16 acc[TM][TN];
 #pragma unroll
@@ -166,42 +143,29 @@ __global__ __launch_bounds__(256) void gemm16_kernel(const Params p) {
         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
     // ---- staging registers ----
-    constexpr int A_TOTAL = NVFP4 ? BM * 2 : BM * 8;  // 16-byte global chunks per tile
-    constexpr int B_TOTAL = NVFP4 ? BN * 2 : BN * 8;
+    constexpr int A_TOTAL = BM * 8;  // 16-byte global chunks per tile
+    constexpr int B_TOTAL = BN * 8;
     constexpr int A_CH = (A_TOTAL + 255) / 256;       // ... per thread
     constexpr int B_CH = (B_TOTAL + 255) / 256;
     u32x4 sa[A_CH], sb[B_CH];
-    uint32_t ssa[NVFP4 ? A_CH : 1], ssb[NVFP4 ? B_CH : 1];
 
     auto issue_loads = [&](int ks) {
-      const int kbyte0 = NVFP4 ? ks * (BK / 2) : ks * (BK * 2);
+      const int kbyte0 = ks * (BK * 2);
 #pragma unroll
       for (int i = 0; i < A_CH; ++i) {
         const int c = tid + 256 * i;
-        const int row = NVFP4 ? (c >> 1) : (c >> 3);
-        const int chunk = NVFP4 ? (c & 1) : (c & 7);
+        const int row = c >> 3, chunk = c & 7;
         const bool ok = (c < A_TOTAL) && (m0 + row < m_g) && (kbyte0 + chunk * 16 < kbytes);
         sa[i] = u32x4{0, 0, 0, 0};
         if (ok) sa[i] = *reinterpret_cast<const u32x4*>(a_base + (int64_t)row * kbytes + kbyte0 + chunk * 16);
-        if constexpr (NVFP4) {
-          ssa[i] = 0;
-          if (ok)
-            ssa[i] = *reinterpret_cast<const uint16_t*>(sfa_base + swizzle_128x4(m0 + row, ks * 4, sf_padded) + chunk * 2);
-        }
       }
 #pragma unroll
       for (int i = 0; i < B_CH; ++i) {
         const int c = tid + 256 * i;
-        const int row = NVFP4 ? (c >> 1) : (c >> 3);
-        const int chunk = NVFP4 ? (c & 1) : (c & 7);
+        const int row = c >> 3, chunk = c & 7;
         const bool ok = (c < B_TOTAL) && (n0 + row < p.n) && (kbyte0 + chunk * 16 < kbytes);
         sb[i] = u32x4{0, 0, 0, 0};
         if (ok) sb[i] = *reinterpret_cast<const u32x4*>(b_base + (int64_t)row * kbytes + kbyte0 + chunk * 16);
-        if constexpr (NVFP4) {
-          ssb[i] = 0;
-          if (ok)
-            ssb[i] = *reinterpret_cast<const uint16_t*>(sfb_base + swizzle_128x4(n0 + row, ks * 4, sf_padded) + chunk * 2);
-        }
       }
     };
 
@@ -212,29 +176,13 @@ __global__ __launch_bounds__(256) void gemm16_kernel(const Params p) {
       for (int i = 0; i < A_CH; ++i) {
         const int c = tid + 256 * i;
         if (c >= A_TOTAL) break;
-        if constexpr (NVFP4) {
-          const int row = c >> 1, half = c & 1;
-          u32x4 d[4];
-          dequant32(sa[i], ssa[i], d);
-#pragma unroll
-          for (int q = 0; q < 4; ++q) lds_a[lds_pos(row, half * 4 + q)] = d[q];
-        } else {
-          lds_a[lds_pos(c >> 3, c & 7)] = sa[i];
-        }
+        lds_a[lds_pos(c >> 3, c & 7)] = sa[i];
       }
 #pragma unroll
       for (int i = 0; i < B_CH; ++i) {
         const int c = tid + 256 * i;
         if (c >= B_TOTAL) break;
-        if constexpr (NVFP4) {
-          const int row = c >> 1, half = c & 1;
-          u32x4 d[4];
-          dequant32(sb[i], ssb[i], d);
-#pragma unroll
-          for (int q = 0; q < 4; ++q) lds_b[lds_pos(row, half * 4 + q)] = d[q];
-        } else {
-          lds_b[lds_pos(c >> 3, c & 7)] = sb[i];
-        }
+        lds_b[lds_pos(c >> 3, c & 7)] = sb[i];
       }
     };
 
@@ -274,8 +222,6 @@ __global__ __launch_bounds__(256) void gemm16_kernel(const Params p) {
     }
 
     // ---- epilogue: acc[i][j][r] = C[m = lane%32][n = (r/4)*8 + (lane/32)*4 + r%4] of its 32x32 tile ----
-    float alpha = 1.0f;
-    if constexpr (NVFP4) alpha = dense ? p.alpha[0] : p.alpha[g];
     uint16_t* out = static_cast<uint16_t*>(p.out);
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
@@ -287,14 +233,222 @@ __global__ __launch_bounds__(256) void gemm16_kernel(const Params p) {
 #pragma unroll
         for (int rq = 0; rq < 4; ++rq) {
           const int ncol = n0 + wn * WTN + j * 32 + rq * 8 + (lane >> 5) * 4;
+          if (ncol < p.n) {
+            u32x2 v;
+            v[0] = pack2(acc[i][j][rq * 4 + 0], acc[i][j][rq * 4 + 1], OUT_BF16);
+            v[1] = pack2(acc[i][j][rq * 4 + 2], acc[i][j][rq * 4 + 3], OUT_BF16);
+            *reinterpret_cast<u32x2*>(orow + ncol) = v;
+          }
+        }
+      }
+    }
+  }
+}
+
+// -------------------------------------------------------------------------------------------------
+// NVFP4 tile kernel for every shape the specialised NVFP4 kernels below do not take (ragged sizes, groups,
+// fp32 result).  Same persistent walk over (group, m-tile, n-tile) items, LDS layout and MFMA loop as the
+// kernel above; what differs is how operands get from global memory into LDS:
+//   * Loads cover a span of 128 elements of K (two 64-deep steps): thread unit c = row c/4, 16-byte piece
+//     c%4, so four neighbouring lanes read 64 contiguous bytes of a row, and one dword load fetches the
+//     scales of a row's four blocks (the two lanes that share a dword pick their half).  A load whose
+//     lanes each touch a different cache line keeps the address unit busy for 64 cycles; with 32 bytes
+//     per row and two-byte scale loads per step that, not the MFMAs, bounded this kernel.
+//   * Of each 16-byte piece (two scale blocks) the first block is consumed by the even step of the span and
+//     the second by the odd step: the same permutation of K for both operands, so the dot products are
+//     unchanged and every lane converts in every step.
+//   * The span after the current one is requested at the start of the even step and first needed when the
+//     odd step converts its even half: a full step of MFMAs hides the latency.
+// Requires K % 32 == 0 (a piece never straddles the end of a row).
+// -------------------------------------------------------------------------------------------------
+template <int BM, int BN, bool OUT_BF16, bool OUT_F32>
+__global__ __launch_bounds__(256) void nvfp4_tile_kernel(const Params p) {
+  constexpr int WTM = BM / 2, WTN = BN / 2;  // wave tile
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  extern __shared__ u32x4 lds[];  // two buffers of (A tile, B tile), 64 fp16 of K per row
+  constexpr int BUF_UNITS = (BM + BN) * 8;
+  __shared__ int tile_prefix[kMaxGroups + 1];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int tiles_n = (p.n + BN - 1) / BN;
+  const bool dense = p.problem_sizes == nullptr;
+
+  if (dense) {
+    if (tid == 0) {
+      tile_prefix[0] = 0;
+      tile_prefix[1] = ((p.m + BM - 1) / BM) * tiles_n;
+    }
+  } else if (wave == 0) {  // serial scan in chunks of 64 groups
+    int running = 0;
+    for (int base = 0; base < p.groups; base += 64) {
+      const int g = base + lane;
+      int cnt = 0;
+      if (g < p.groups) {
+        const int mg = p.problem_sizes[g * 3];
+        cnt = mg > 0 ? ((mg + BM - 1) / BM) * tiles_n : 0;
+      }
+      int incl = cnt;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const int o = __shfl_up(incl, d, 64);
+        if (lane >= d) incl += o;
+      }
+      if (g < p.groups) tile_prefix[g + 1] = running + incl;
+      running += __shfl(incl, 63, 64);
+    }
+    if (lane == 0) tile_prefix[0] = 0;
+  }
+  __syncthreads();
+  const int total_tiles = tile_prefix[p.groups];
+
+  const int kbytes = p.k >> 1;
+  const int sf_cols = p.k >> 4;
+  const int sf_padded = (sf_cols + 3) & ~3;
+  const int nspans = (p.k + 127) >> 7;
+
+  constexpr int A_CH = BM / 64, B_CH = BN / 64;  // 16-byte pieces per thread and span
+  struct Raw { u32x4 a[A_CH], b[B_CH]; uint32_t sa[A_CH], sb[B_CH]; };
+  const int urow = tid >> 2, upiece = tid & 3;  // unit i of a thread: row urow + 64 * i
+
+  for (int tile = blockIdx.x; tile < total_tiles; tile += gridDim.x) {
+    int g = 0;
+    {
+      int lo = 0, hi = p.groups;
+      while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (tile < tile_prefix[mid]) hi = mid; else lo = mid;
+      }
+      g = lo;
+    }
+    const int m_g = dense ? p.m : p.problem_sizes[g * 3];
+    const int64_t row_off = dense ? 0 : p.expert_offsets[g];
+    const int tiles_m = (m_g + BM - 1) / BM;
+    const int local = tile - tile_prefix[g];
+    const int mt = local % tiles_m, nt = local / tiles_m;
+    const int m0 = mt * BM, n0 = nt * BN;
+
+    const uint8_t* a_base = p.a + (row_off + m0) * (int64_t)kbytes;
+    const uint8_t* b_base = p.b + ((int64_t)g * p.n + n0) * (int64_t)kbytes;
+    const uint8_t* sfa_base = p.sfa + (dense ? 0 : (int64_t)p.sf_offsets[g]) * sf_cols;  // group slab, swizzled on its own
+    const uint8_t* sfb_base = p.sfb + (int64_t)g * p.n * sf_cols;
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    auto issue_span = [&](Raw& r, int sp) {
+      const int kb = sp * 64 + upiece * 16;            // byte in the row
+      const int sf_col = sp * 8 + (upiece >> 1) * 4;   // first of the 4 blocks the dword covers
+      const bool k_ok = kb < kbytes;
+#pragma unroll
+      for (int i = 0; i < A_CH; ++i) {
+        const int row = urow + 64 * i;
+        const bool ok = k_ok && (m0 + row < m_g);
+        r.a[i] = u32x4{0, 0, 0, 0};
+        r.sa[i] = 0;
+        if (ok) {
+          r.a[i] = *reinterpret_cast<const u32x4*>(a_base + (int64_t)row * kbytes + kb);
+          r.sa[i] = *reinterpret_cast<const uint32_t*>(sfa_base + swizzle_128x4(m0 + row, sf_col, sf_padded));
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < B_CH; ++i) {
+        const int row = urow + 64 * i;
+        const bool ok = k_ok && (n0 + row < p.n);
+        r.b[i] = u32x4{0, 0, 0, 0};
+        r.sb[i] = 0;
+        if (ok) {
+          r.b[i] = *reinterpret_cast<const u32x4*>(b_base + (int64_t)row * kbytes + kb);
+          r.sb[i] = *reinterpret_cast<const uint32_t*>(sfb_base + swizzle_128x4(n0 + row, sf_col, sf_padded));
+        }
+      }
+    };
+
+    // block `parity` of every piece -> fp16 -> LDS buffer buf (chunks 2*piece, 2*piece+1 of the row)
+    auto convert_one = [&](u32x4 q, uint32_t s4, int parity, u32x4* dst_tile, int row) {
+      const uint32_t s2 = s4 >> ((upiece & 1) * 16);  // this piece's two scale bytes
+      const float f = parity ? __builtin_amdgcn_cvt_f32_fp8((int)s2, 1) : __builtin_amdgcn_cvt_f32_fp8((int)s2, 0);
+      const f16x2 sv = __builtin_bit_cast(f16x2, __builtin_amdgcn_cvt_pkrtz(f, f));  // exact: e4m3 fits fp16
+#pragma unroll
+      for (int cc = 0; cc < 2; ++cc) {
+        const uint32_t w = q[2 * parity + cc];
+        const f16x2 h0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 1.0f, 0) * sv;
+        const f16x2 h1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 1.0f, 1) * sv;
+        const f16x2 h2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 1.0f, 2) * sv;
+        const f16x2 h3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 1.0f, 3) * sv;
+        dst_tile[lds_pos2(row, upiece * 2 + cc)] = u32x4{__builtin_bit_cast(uint32_t, h0), __builtin_bit_cast(uint32_t, h1),
+                                                         __builtin_bit_cast(uint32_t, h2), __builtin_bit_cast(uint32_t, h3)};
+      }
+    };
+    auto convert = [&](const Raw& r, int parity, int buf) {
+      u32x4* lds_a = lds + buf * BUF_UNITS;
+      u32x4* lds_b = lds_a + BM * 8;
+#pragma unroll
+      for (int i = 0; i < A_CH; ++i) convert_one(r.a[i], r.sa[i], parity, lds_a, urow + 64 * i);
+#pragma unroll
+      for (int i = 0; i < B_CH; ++i) convert_one(r.b[i], r.sb[i], parity, lds_b, urow + 64 * i);
+    };
+    auto mfma_step = [&](int buf) {
+      const u32x4* lds_a = lds + buf * BUF_UNITS;
+      const u32x4* lds_b = lds_a + BM * 8;
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        u32x4 fa[TM], fb[TN];
+        const int chunk = kk * 2 + (lane >> 5);
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fa[i] = lds_a[lds_pos2(wm * WTM + i * 32 + (lane & 31), chunk)];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fb[j] = lds_b[lds_pos2(wn * WTN + j * 32 + (lane & 31), chunk)];
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, fb[j]), __builtin_bit_cast(f16x8, fa[i]),
+                                                               acc[i][j], 0, 0, 0);
+      }
+    };
+
+    Raw cur, nxt;
+    issue_span(cur, 0);
+    convert(cur, 0, 0);  // every wave is past the barrier that ended the previous tile's last step
+    __syncthreads();
+    for (int sp = 0; sp < nspans; ++sp) {
+      const bool more = sp + 1 < nspans;
+      if (more) issue_span(nxt, sp + 1);
+      mfma_step(0);
+      convert(cur, 1, 1);
+      __syncthreads();
+      mfma_step(1);
+      if (more) convert(nxt, 0, 0);
+      __syncthreads();
+      cur = nxt;
+    }
+
+    // ---- epilogue: acc[i][j][r] = C[m = lane%32][n = (r/4)*8 + (lane/32)*4 + r%4] of its 32x32 tile ----
+    const float alpha = dense ? p.alpha[0] : p.alpha[g];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int mrow = m0 + wm * WTM + i * 32 + (lane & 31);
+      if (mrow >= m_g) continue;
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq) {
+          const int ncol = n0 + wn * WTN + j * 32 + rq * 8 + (lane >> 5) * 4;
+          if (ncol >= p.n) continue;
           if constexpr (OUT_F32) {
-            if (ncol < p.n) {
-              typedef float f32x4_t __attribute__((ext_vector_type(4)));
-              float* frow = static_cast<float*>(p.out) + (row_off + mrow) * (int64_t)p.n;
-              *reinterpret_cast<f32x4_t*>(frow + ncol) = f32x4_t{acc[i][j][rq * 4 + 0] * alpha, acc[i][j][rq * 4 + 1] * alpha,
-                                                                 acc[i][j][rq * 4 + 2] * alpha, acc[i][j][rq * 4 + 3] * alpha};
-            }
-          } else if (ncol < p.n) {
+            float* frow = static_cast<float*>(p.out) + (row_off + mrow) * (int64_t)p.n;
+            *reinterpret_cast<f32x4*>(frow + ncol) = f32x4{acc[i][j][rq * 4 + 0] * alpha, acc[i][j][rq * 4 + 1] * alpha,
+                                                           acc[i][j][rq * 4 + 2] * alpha, acc[i][j][rq * 4 + 3] * alpha};
+          } else {
+            uint16_t* orow = static_cast<uint16_t*>(p.out) + (row_off + mrow) * (int64_t)p.n;
             u32x2 v;
             v[0] = pack2(acc[i][j][rq * 4 + 0] * alpha, acc[i][j][rq * 4 + 1] * alpha, OUT_BF16);
             v[1] = pack2(acc[i][j][rq * 4 + 2] * alpha, acc[i][j][rq * 4 + 3] * alpha, OUT_BF16);
@@ -587,7 +741,6 @@ int launch_nvfp4_fast(const Params& p, int cus, hipStream_t stream) {
 //     t = 0..3 with elements 8t..8t+7.  Weight rows are the first operand (output rows), activation rows
 //     the second, so a lane ends up with 4 consecutive N-elements of one output row.
 // -------------------------------------------------------------------------------------------------
-typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 // LDS-direct load.  lds_byte_addr and base are wave-uniform; lane L's 16 bytes land at lds_byte_addr + 16 * L.
 // Issued from inline assembly: the compiler neither waits for it nor orders LDS reads against it, the
@@ -1175,9 +1328,9 @@ int launch_grouped16_fast(const Params& p, int cus, hipStream_t stream) {
   return check_launch("grouped16_gemm_256_kernel");
 }
 
-template <int BM, int BN, bool NVFP4, bool BF16_MMA, bool OUT_BF16, bool OUT_F32 = false>
+template <int BM, int BN, bool BF16_MMA, bool OUT_BF16>
 int launch_cfg(const Params& p, int grid, hipStream_t stream) {
-  auto kern = gemm16_kernel<BM, BN, NVFP4, BF16_MMA, OUT_BF16, OUT_F32>;
+  auto kern = gemm16_kernel<BM, BN, BF16_MMA, OUT_BF16>;
   constexpr int lds_bytes = 2 * (BM + BN) * 128;
   static bool configured = false;  // benign race: the attribute call is idempotent
   if (!configured) {
@@ -1187,6 +1340,27 @@ int launch_cfg(const Params& p, int grid, hipStream_t stream) {
   }
   hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_bytes, stream, p);
   return check_launch("gemm16_kernel");
+}
+
+template <int BM, int BN, bool OUT_BF16, bool OUT_F32 = false>
+int launch_nvfp4_tile(const Params& p, int grid, hipStream_t stream) {
+  auto kern = nvfp4_tile_kernel<BM, BN, OUT_BF16, OUT_F32>;
+  constexpr int lds_bytes = 2 * (BM + BN) * 128;
+  static bool configured = false;  // benign race: the attribute call is idempotent
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    if (e != hipSuccess) return fail(NVF_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    configured = true;
+  }
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_bytes, stream, p);
+  return check_launch("nvfp4_tile_kernel");
+}
+
+// tile kernel of the operand type: NVFP4 or 16-bit
+template <int BM, int BN, bool NVFP4, bool BF16_MMA, bool OUT_BF16>
+int launch_tile(const Params& p, int grid, hipStream_t stream) {
+  if constexpr (NVFP4) return launch_nvfp4_tile<BM, BN, OUT_BF16>(p, grid, stream);
+  else return launch_cfg<BM, BN, BF16_MMA, OUT_BF16>(p, grid, stream);
 }
 
 template <bool NVFP4, bool BF16_MMA, bool OUT_BF16>
@@ -1208,28 +1382,28 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, hipStream_t stream) {
   // grouped: the tile height follows the average group (a 256-row tile on a 77-row group is mostly padding)
   if (dense ? tiles(256, 256) >= cus : m_hint >= 512 * (int64_t)p.groups) {
     const int64_t upper = dense ? tiles(256, 256) : (ceil_div(p.m, 256) + p.groups) * ceil_div(p.n, 256);
-    return launch_cfg<256, 256, NVFP4, BF16_MMA, OUT_BF16>(p, (int)(upper < cus ? upper : cus), stream);
+    return launch_tile<256, 256, NVFP4, BF16_MMA, OUT_BF16>(p, (int)(upper < cus ? upper : cus), stream);
   }
   if (tiles(128, 128) >= cus || !dense) {
     const int64_t upper = dense ? tiles(128, 128) : (ceil_div(p.m, 128) + p.groups) * ceil_div(p.n, 128);
     const int64_t cap = 2 * (int64_t)cus;
-    return launch_cfg<128, 128, NVFP4, BF16_MMA, OUT_BF16>(p, (int)(upper < cap ? upper : cap), stream);
+    return launch_tile<128, 128, NVFP4, BF16_MMA, OUT_BF16>(p, (int)(upper < cap ? upper : cap), stream);
   }
   const int64_t upper = tiles(64, 64);
   const int64_t cap = 4 * (int64_t)cus;
-  return launch_cfg<64, 64, NVFP4, BF16_MMA, OUT_BF16>(p, (int)(upper < cap ? upper : cap), stream);
+  return launch_tile<64, 64, NVFP4, BF16_MMA, OUT_BF16>(p, (int)(upper < cap ? upper : cap), stream);
 }
 
 // dense NVFP4 with an fp32 result (the product that the block-scaled epilogue op re-quantizes)
 int launch_nvfp4_f32(const Params& p, int cus, hipStream_t stream) {
   auto tiles = [&](int bm, int bn) { return ceil_div(p.m, bm) * ceil_div(p.n, bn); };
-  if (tiles(256, 256) >= cus) return launch_cfg<256, 256, true, false, false, true>(p, cus, stream);
+  if (tiles(256, 256) >= cus) return launch_nvfp4_tile<256, 256, false, true>(p, cus, stream);
   if (tiles(128, 128) >= cus) {
     const int64_t t = tiles(128, 128);
-    return launch_cfg<128, 128, true, false, false, true>(p, (int)(t < 2 * cus ? t : 2 * cus), stream);
+    return launch_nvfp4_tile<128, 128, false, true>(p, (int)(t < 2 * cus ? t : 2 * cus), stream);
   }
   const int64_t t = tiles(64, 64);
-  return launch_cfg<64, 64, true, false, false, true>(p, (int)(t < 4 * cus ? t : 4 * cus), stream);
+  return launch_nvfp4_tile<64, 64, false, true>(p, (int)(t < 4 * cus ? t : 4 * cus), stream);
 }
 
 int cu_count() {
