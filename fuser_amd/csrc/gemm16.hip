@@ -1370,8 +1370,12 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, hipStream_t stream) {
   const bool dense = p.problem_sizes == nullptr;
   if constexpr (NVFP4) {
     if (dense && p.m <= 128 && (p.k & 127) == 0 && (p.n & 15) == 0) return launch_nvfp4_skinny<OUT_BF16>(p, cus, stream);
-    if (dense && tiles(256, 256) >= 128 && (p.m & 255) == 0 && (p.n & 255) == 0 && (p.k & 127) == 0 && p.k >= 256)
-      return launch_nvfp4_fast<OUT_BF16>(p, cus, stream);
+    if (dense && (p.m & 255) == 0 && (p.n & 255) == 0 && (p.k & 127) == 0 && p.k >= 256) {
+      // The 256x256 kernel is about 1.4 times as fast per tile-flop as the tile kernel below, so it wins
+      // unless its last round of tiles leaves more than about 30 % of the compute units' slots empty.
+      const int64_t t = tiles(256, 256), rounds = ceil_div(t, cus);
+      if (10 * t >= 7 * rounds * cus) return launch_nvfp4_fast<OUT_BF16>(p, cus, stream);
+    }
   }
   if constexpr (!NVFP4) {
     // grouped_mm with groups of a few hundred rows on average: persistent LDS-direct kernel

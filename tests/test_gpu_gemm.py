@@ -263,13 +263,16 @@ def test_mxfp8_gemm_ragged_shapes_alpha_and_scale_spread(dev, shape):
         assert err <= GEMM_MAX_REL, (shape, dtype, err)
 
 
-@pytest.mark.parametrize("shape", [(4096, 2048, 512), (2560, 3328, 384), (2048, 4096, 256), (8192, 1024, 1152),
-                                   (4096, 8192, 256), (8192, 4096, 384), (4352, 4096, 128 * 5)])
+@pytest.mark.parametrize("shape", [(4096, 3072, 512), (3328, 3840, 384), (2048, 6144, 256), (8192, 1536, 1152),
+                                   (4096, 8192, 256), (8192, 4096, 384), (4608, 5120, 128 * 5),
+                                   (4096, 2048, 512), (4352, 4096, 384)])
 def test_nvfp4_gemm_persistent_256_tile_kernel_full_compare(dev, shape):
-    """Dense shapes with M % 256 == N % 256 == K % 128 == 0 and at least 128 tiles take the persistent
-    kernel that converts the operands to fp16 between its MFMAs; every output element is compared with
-    the oracle.  Same tile-grid cases as the MXFP8 test below (incl. several tiles per workgroup with two,
-    three and five 128-deep spans per tile)."""
+    """Dense shapes with M % 256 == N % 256 == K % 128 == 0 take the persistent 256x256 kernel that converts
+    the operands to fp16 between its MFMAs when their tiles fill at least 70 % of the compute units' slots
+    (192, 195, 192, 192, 512, 512 and 360 tiles on 256 units here: blocked and unblocked tile grids, one
+    and several tiles per workgroup with two, three, five and nine 128-deep spans per tile); the last two
+    shapes (128 and 272 tiles) fall to the 128x128 tile kernel.  Every output element is compared with the
+    oracle."""
     m, n, k = shape
     gen = torch.Generator().manual_seed(k + 1)
     a, sa, ga = _nvfp4_operand(m, k, 1.0, gen)
@@ -284,12 +287,13 @@ def test_nvfp4_gemm_persistent_256_tile_kernel_full_compare(dev, shape):
     assert ((out16.float().cpu() - ref).abs() / scale).max().item() <= GEMM_MAX_REL
 
 
+@pytest.mark.parametrize("n_cols", [6144, 4096])  # 256x256 persistent kernel, 128x128 tile kernel
 @pytest.mark.parametrize("scale_range", [(0x01, 0x0F), (0x01, 0x7E), (0x70, 0x7E)])
-def test_nvfp4_gemm_persistent_kernel_every_scale_code_is_decoded_exactly(dev, scale_range):
+def test_nvfp4_gemm_persistent_kernel_every_scale_code_is_decoded_exactly(dev, scale_range, n_cols):
     """Random payload bytes and random e4m3 scale bytes, including the subnormal codes 0x01..0x07 and the
     largest finite ones: each e2m1 x e4m3 product is exactly representable in fp16, so the only error
     left is the fp32 summation order and the bf16 rounding of the output."""
-    m, n, k = 2048, 4096, 256
+    m, n, k = 2048, n_cols, 256
     gen = torch.Generator().manual_seed(scale_range[0] * 131 + scale_range[1])
     a = torch.randint(0, 256, (m, k // 2), dtype=torch.uint8, generator=gen)
     b = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, generator=gen)
