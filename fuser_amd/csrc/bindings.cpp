@@ -3,11 +3,13 @@
 // plus eager entry points for the block quantizers.
 #include <torch/extension.h>
 
+#include "callers.h"
 #include "nvf_cutlass.h"
 
 namespace py = pybind11;
 namespace ck = nvfuser::cutlass_kernels;
 namespace bq = nvfuser::block_quantization;
+namespace cl = nvfuser::callers;
 
 PYBIND11_MODULE(_C, m) {
   m.doc() = "MI355X implementation of nvFuser's quantized-GEMM path";
@@ -70,4 +72,34 @@ PYBIND11_MODULE(_C, m) {
       py::arg("block_size") = 16, py::arg("dtype") = at::ScalarType::Float4_e2m1fn_x2);
   m.def("preprocess_grouped_matmul_input_sf", &bq::preprocess_grouped_matmul_input_sf, py::arg("input"),
         py::arg("input_offsets"), py::arg("output_offsets"));
+
+  // Conventions of the reference's expression nodes around the kernels (csrc/ir/composite_nodes.cpp).
+  // A kernel branch that does not apply returns None: the caller falls back.
+  py::module_ callers = m.def_submodule("callers", "ScaledMmaOp / GroupedMmaOp / CutlassNvfp4GroupedMmaOp conventions.");
+  auto or_none = [](const torch::Tensor& t) -> py::object { return t.defined() ? py::cast(t) : py::none(); };
+  callers.def(
+      "scaled_mma",
+      [or_none](const torch::Tensor& mat1, const torch::Tensor& mat2, const torch::Tensor& scale1, const torch::Tensor& scale2,
+                const c10::optional<torch::Tensor>& alpha, const c10::optional<torch::Tensor>& bias,
+                const c10::optional<torch::Tensor>& beta, at::ScalarType out_dtype) {
+        return or_none(cl::scaled_mma(mat1, mat2, scale1, scale2, alpha, bias, beta, out_dtype));
+      },
+      py::arg("mat1"), py::arg("mat2"), py::arg("scale1"), py::arg("scale2"), py::arg("alpha") = py::none(),
+      py::arg("bias") = py::none(), py::arg("beta") = py::none(), py::arg("out_dtype") = at::ScalarType::BFloat16);
+  callers.def(
+      "grouped_mma_arguments",
+      [](const torch::Tensor& offsets, int64_t n, int64_t k) {
+        auto r = cl::grouped_mma_arguments(offsets, n, k);
+        return py::make_tuple(r.problem_sizes, r.expert_offsets, r.ab_strides, r.c_strides);
+      },
+      py::arg("offsets"), py::arg("n"), py::arg("k"));
+  callers.def(
+      "grouped_mma",
+      [or_none](const torch::Tensor& mat1, const torch::Tensor& mat2, const torch::Tensor& offsets) {
+        return or_none(cl::grouped_mma(mat1, mat2, offsets));
+      },
+      py::arg("mat1"), py::arg("mat2"), py::arg("offsets"));
+  callers.def("cutlass_nvfp4_grouped_mma", &cl::cutlass_nvfp4_grouped_mma, py::arg("mat1"), py::arg("mat2"),
+              py::arg("scale1"), py::arg("scale2"), py::arg("alpha"), py::arg("problem_sizes"), py::arg("expert_offsets"),
+              py::arg("sf_offsets"), py::arg("out_dtype") = at::ScalarType::BFloat16);
 }
