@@ -35,7 +35,7 @@ def parse():
     ap.add_argument("--calib", action="store_true", help="profiling aid: also run a plain 1 GiB device copy a few times, "
                     "so that a counter run shows what FETCH_SIZE / WRITE_SIZE read for a kernel of known traffic")
     ap.add_argument("--only", default="", help="profiling aid: run just this extra workload "
-                    "(quant | nvfp4 | llm | grouped | gnvfp4) and print its line")
+                    "(quant | fused | nvfp4 | llm | grouped | gnvfp4) and print its line")
     return ap.parse_args()
 
 
@@ -117,6 +117,28 @@ def main():
             xs = torch.randn(mm, kk, device=dev, generator=gen).bfloat16()
             ms, _ = timed(lambda: ops.nv_block_quantize(xs, gs, True, 16), 50, 5)
             extra[f"nvfp4_quantize_{mm}x{kk}"] = {"us": round(ms * 1e3, 2), "GB/s": round(mm * kk * 2.5625 / ms / 1e6, 1)}
+
+    def run_fused():
+        # the steps either side of the quantizer in the NVFP4 MoE layer at config 5's intermediate size
+        m, k = 65536, 2048
+        gate = torch.randn(m, k, device=dev, generator=gen).bfloat16()
+        up = torch.randn(m, k, device=dev, generator=gen).bfloat16()
+        sizes = moe_zipf(8192, 8, 256, 1.1, 0).int()
+        padded = (sizes + 127) // 128 * 128
+        eo = (torch.cumsum(sizes, 0) - sizes).int().to(dev)
+        so = (torch.cumsum(padded, 0) - padded).int().to(dev)
+        ms_f, _ = timed(lambda: ops.silu_mul_nv_grouped_block_quantize(gate, up, eo, so, None), 30, 5)
+        ms_c, _ = timed(lambda: ops.nv_grouped_block_quantize(torch.nn.functional.silu(gate) * up, eo, so, None, 16), 30, 5)
+        extra["silu_mul_grouped_quantize"] = {
+            "workload": "silu(gate) * up -> NVFP4, gate/up bf16 [65536,2048], 256 Zipf(1.1) groups",
+            "fused_ms": round(ms_f, 4), "fused_GB/s": round(m * k * 4.5625 / ms_f / 1e6, 1),
+            "unfused_chain_ms": round(ms_c, 4), "note": "fused bytes/element: 4 read + 0.5625 written; the chain moves 12.56"}
+        x = torch.randn(65536, 7168, device=dev, generator=gen).bfloat16()
+        ms_g, _ = timed(lambda: ops.compute_nvfp4_global_scale(x), 30, 5)
+        ms_t, _ = timed(lambda: (2688.0 / x.abs().max().float()), 10, 2)
+        extra["nvfp4_global_scale"] = {"workload": "bf16 [65536,7168] -> fp32 scalar on the device",
+                                       "ms": round(ms_g, 4), "GB/s": round(x.numel() * 2 / ms_g / 1e6, 1),
+                                       "torch_abs_max_ms": round(ms_t, 4)}
 
     def quantized_nvfp4(rows, k, std):
         x = (torch.randn(rows, k, device=dev, generator=gen) * std).bfloat16()
@@ -209,7 +231,8 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    runners = {"quant": run_quant, "nvfp4": run_nvfp4, "llm": run_llm, "grouped": run_grouped, "gnvfp4": run_gnvfp4}
+    runners = {"quant": run_quant, "fused": run_fused, "nvfp4": run_nvfp4, "llm": run_llm, "grouped": run_grouped,
+               "gnvfp4": run_gnvfp4}
     if args.only:
         runners[args.only]()
         print(json.dumps({"only": args.only, "extra": extra}))
@@ -261,7 +284,7 @@ def main():
         del da, db, ref, got
 
     if not args.no_extra:
-        for name in ("quant", "nvfp4", "llm", "grouped", "gnvfp4"):
+        for name in ("quant", "fused", "nvfp4", "llm", "grouped", "gnvfp4"):
             runners[name]()
 
     line = {

@@ -16,6 +16,8 @@ SIGNATURES = {
     "nvf_get_multiprocessor_count": (_int, [_p]),
     "nvf_nvfp4_block_quantize": (_int, [_p, _int, _i64, _i64, _p, _int, _p, _p, _p]),
     "nvf_nvfp4_grouped_block_quantize": (_int, [_p, _int, _i64, _i64, _p, _p, _int, _p, _p, _p, _p]),
+    "nvf_nvfp4_silu_mul_block_quantize": (_int, [_p, _p, _int, _i64, _i64, _p, _p, _int, _p, _p, _p, _p]),
+    "nvf_nvfp4_global_scale": (_int, [_p, _int, _i64, _p, _p]),
     "nvf_preprocess_grouped_matmul_input_sf": (_int, [_p, _int, _i64, _i64, _p, _p, _int, _p, _p]),
     "nvf_mxfp8_block_quantize": (_int, [_p, _int, _i64, _i64, _int, _p, _p, _p]),
     "nvf_cast_f32_to_e2m1": (_int, [_p, _i64, _p, _p]),

@@ -72,6 +72,15 @@ PYBIND11_MODULE(_C, m) {
       py::arg("block_size") = 16, py::arg("dtype") = at::ScalarType::Float4_e2m1fn_x2);
   m.def("preprocess_grouped_matmul_input_sf", &bq::preprocess_grouped_matmul_input_sf, py::arg("input"),
         py::arg("input_offsets"), py::arg("output_offsets"));
+  m.def(
+      "silu_mul_nv_grouped_block_quantize",
+      [](const torch::Tensor& gate, const torch::Tensor& up, const torch::Tensor& input_offsets,
+         const torch::Tensor& output_offsets, const c10::optional<torch::Tensor>& global_scale) {
+        auto r = bq::silu_mul_nv_grouped_block_quantize(gate, up, input_offsets, output_offsets, global_scale);
+        return py::make_tuple(r.first, r.second);
+      },
+      py::arg("gate"), py::arg("up"), py::arg("input_offsets"), py::arg("output_offsets"), py::arg("global_scale") = py::none());
+  m.def("compute_nvfp4_global_scale", &bq::compute_nvfp4_global_scale, py::arg("tensor"));
 
   // Conventions of the reference's expression nodes around the kernels (csrc/ir/composite_nodes.cpp).
   // A kernel branch that does not apply returns None: the caller falls back.

@@ -91,6 +91,27 @@ int nvf_nvfp4_grouped_block_quantize(const void* in, int in_dtype, int64_t rows,
                                out_scales, static_cast<hipStream_t>(stream));
 }
 
+int nvf_nvfp4_silu_mul_block_quantize(const void* gate, const void* up, int in_dtype, int64_t rows, int64_t cols,
+                                      const int32_t* input_offsets, const int32_t* output_offsets, int groups,
+                                      const float* global_scale, void* out_fp4, void* out_scales, void* stream) {
+  NVF_REQUIRE(in_dtype == NVF_BF16 || in_dtype == NVF_F16, NVF_ERR_INVALID_ARGUMENT, "inputs must be bf16 or f16, got dtype %d", in_dtype);
+  NVF_REQUIRE(rows >= 0 && cols >= 0, NVF_ERR_INVALID_ARGUMENT, "negative size (%lld, %lld)", (long long)rows, (long long)cols);
+  NVF_REQUIRE(cols % 16 == 0, NVF_ERR_UNSUPPORTED_SHAPE, "the inner dimension %lld is not divisible by the block size 16", (long long)cols);
+  const bool grouped = input_offsets != nullptr;
+  if (grouped) NVF_REQUIRE(groups >= 1, NVF_ERR_INVALID_ARGUMENT, "groups must be >= 1, got %d", groups);
+  if (rows == 0 || cols == 0) return NVF_OK;
+  NVF_REQUIRE(gate && up && out_fp4 && out_scales && (!grouped || output_offsets), NVF_ERR_INVALID_ARGUMENT, "NULL buffer");
+  return launch_nvfp4_silu_mul_quantize(gate, up, in_dtype, rows, cols, global_scale, grouped ? 2 : 1, input_offsets, output_offsets,
+                                        grouped ? groups : 1, out_fp4, out_scales, static_cast<hipStream_t>(stream));
+}
+
+int nvf_nvfp4_global_scale(const void* in, int in_dtype, int64_t numel, float* out_scale, void* stream) {
+  NVF_REQUIRE(dtype_in(in_dtype), NVF_ERR_INVALID_ARGUMENT, "unknown input dtype %d", in_dtype);
+  NVF_REQUIRE(numel >= 0, NVF_ERR_INVALID_ARGUMENT, "negative size %lld", (long long)numel);
+  NVF_REQUIRE(out_scale && (in || numel == 0), NVF_ERR_INVALID_ARGUMENT, "NULL buffer");
+  return launch_nvfp4_global_scale(in, in_dtype, numel, out_scale, static_cast<hipStream_t>(stream));
+}
+
 int nvf_preprocess_grouped_matmul_input_sf(const void* in, int elem_size, int64_t rows, int64_t cols,
                                            const int32_t* input_offsets, const int32_t* output_offsets, int groups,
                                            void* out, void* stream) {

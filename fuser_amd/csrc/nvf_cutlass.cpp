@@ -411,6 +411,53 @@ std::pair<torch::Tensor, torch::Tensor> nv_grouped_block_quantize(const torch::T
   return {quantized, scales};
 }
 
+std::pair<torch::Tensor, torch::Tensor> silu_mul_nv_grouped_block_quantize(const torch::Tensor& gate, const torch::Tensor& up,
+                                                                           const torch::Tensor& input_offsets,
+                                                                           const torch::Tensor& output_offsets,
+                                                                           const c10::optional<torch::Tensor>& global_scale) {
+  check_quant_input(gate, 16);
+  check_quant_input(up, 16);
+  NVF_CHECK(gate.dim() == 2, "Grouped block quantization only supports 2D input tensors");
+  NVF_CHECK(gate.scalar_type() == at::ScalarType::BFloat16 || gate.scalar_type() == at::ScalarType::Half,
+            "Expected BFloat16 or Half inputs.");
+  NVF_CHECK(up.scalar_type() == gate.scalar_type() && up.sizes() == gate.sizes() && up.device() == gate.device(),
+            "gate and up must have the same dtype, shape and device.");
+  const float* gs = check_global_scale(global_scale, gate);
+  for (const torch::Tensor& t : {input_offsets, output_offsets}) {
+    NVF_CHECK(t.is_cuda() && t.is_contiguous() && t.dim() == 1 && t.scalar_type() == at::ScalarType::Int,
+              "Offsets must be contiguous 1-D int32 CUDA tensors.");
+  }
+  NVF_CHECK_EQ(input_offsets.size(0), output_offsets.size(0), "input_offsets and output_offsets differ in length.");
+  const int64_t rows = gate.size(0), cols = gate.size(1), groups = input_offsets.size(0);
+  NVF_CHECK(groups >= 1, "At least one group is required.");
+
+  c10::DeviceGuard guard(gate.device());
+  void* stream = current_stream(gate);
+  torch::Tensor quantized = at::empty({rows, cols / 2}, gate.options().dtype(at::ScalarType::Float4_e2m1fn_x2));
+  torch::Tensor scales = at::empty({rows + groups * 127, cutlass_kernels::roundUp(cols / 16, 4)},
+                                   gate.options().dtype(at::ScalarType::Float8_e4m3fn));
+  check_status(nvf_nvfp4_silu_mul_block_quantize(gate.data_ptr(), up.data_ptr(), to_nvf_dtype(gate.scalar_type()), rows, cols,
+                                                 static_cast<const int32_t*>(input_offsets.data_ptr()),
+                                                 static_cast<const int32_t*>(output_offsets.data_ptr()),
+                                                 static_cast<int>(groups), gs, quantized.data_ptr(), scales.data_ptr(), stream),
+               "silu_mul_nv_grouped_block_quantize");
+  return {quantized, scales};
+}
+
+torch::Tensor compute_nvfp4_global_scale(const torch::Tensor& tensor) {
+  NVF_CHECK(tensor.is_cuda(), "Expected a CUDA tensor.");
+  NVF_CHECK(tensor.is_contiguous(), "Expected a contiguous tensor.");
+  const at::ScalarType t = tensor.scalar_type();
+  NVF_CHECK(t == at::ScalarType::Float || t == at::ScalarType::BFloat16 || t == at::ScalarType::Half,
+            "Expected a Float, BFloat16 or Half tensor.");
+  c10::DeviceGuard guard(tensor.device());
+  torch::Tensor scale = at::empty({}, tensor.options().dtype(at::ScalarType::Float));
+  check_status(nvf_nvfp4_global_scale(tensor.data_ptr(), to_nvf_dtype(t), tensor.numel(), static_cast<float*>(scale.data_ptr()),
+                                      current_stream(tensor)),
+               "compute_nvfp4_global_scale");
+  return scale;
+}
+
 torch::Tensor preprocess_grouped_matmul_input_sf(const torch::Tensor& input, const torch::Tensor& input_offsets,
                                                  const torch::Tensor& output_offsets) {
   NVF_CHECK(input.is_cuda() && input.is_contiguous() && input.dim() == 2, "Expected a contiguous 2-D CUDA tensor.");

@@ -94,6 +94,17 @@ NVF_HOST_API std::pair<torch::Tensor, torch::Tensor> nv_grouped_block_quantize(
     const torch::Tensor& input, const torch::Tensor& input_offsets, const torch::Tensor& output_offsets,
     const c10::optional<torch::Tensor>& global_scale, int64_t block_size, at::ScalarType dtype);
 
+// nv_grouped_block_quantize of silu(gate) * up (evaluated in the inputs' 16-bit type as the eager chain of
+// benchmarks/python/layers_for_inference_benchmark.py:504 does), without materialising the product.
+NVF_HOST_API std::pair<torch::Tensor, torch::Tensor> silu_mul_nv_grouped_block_quantize(
+    const torch::Tensor& gate, const torch::Tensor& up, const torch::Tensor& input_offsets,
+    const torch::Tensor& output_offsets, const c10::optional<torch::Tensor>& global_scale);
+
+// 0-dim fp32 device tensor 448 * 6 / max|tensor| (1.0 if all zero), the global_scale argument of the
+// quantizers; compute_nvfp4_global_scale of tests/python/direct/test_narrow_precision.py:138-156 without the
+// host round trip.
+NVF_HOST_API torch::Tensor compute_nvfp4_global_scale(const torch::Tensor& tensor);
+
 NVF_HOST_API torch::Tensor preprocess_grouped_matmul_input_sf(const torch::Tensor& input,
                                                               const torch::Tensor& input_offsets,
                                                               const torch::Tensor& output_offsets);

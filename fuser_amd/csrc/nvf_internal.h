@@ -27,6 +27,12 @@ inline int64_t round_up(int64_t x, int64_t y) { return ceil_div(x, y) * y; }
 int launch_nvfp4_quantize(const void* in, int in_dtype, int64_t rows, int64_t cols, const float* gs, int layout,
                           const int32_t* in_off, const int32_t* out_off, int groups, void* out_fp4, void* out_sf,
                           hipStream_t stream);
+// input = silu(gate) * up evaluated in the inputs' 16-bit type (bf16 / f16 only)
+int launch_nvfp4_silu_mul_quantize(const void* gate, const void* up, int in_dtype, int64_t rows, int64_t cols, const float* gs,
+                                   int layout, const int32_t* in_off, const int32_t* out_off, int groups, void* out_fp4,
+                                   void* out_sf, hipStream_t stream);
+// out[0] = 448 * 6 / max|in| (1 if the tensor is all zero)
+int launch_nvfp4_global_scale(const void* in, int in_dtype, int64_t n, float* out, hipStream_t stream);
 int launch_preprocess_sf(const void* in, int elem_size, int64_t rows, int64_t cols, const int32_t* in_off,
                          const int32_t* out_off, int groups, void* out, hipStream_t stream);
 int launch_mxfp8_quantize(const void* in, int in_dtype, int64_t rows, int64_t cols, int swizzle, void* out_fp8,

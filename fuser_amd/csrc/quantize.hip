@@ -129,8 +129,24 @@ __device__ __forceinline__ float fast_rcp(float v) {
 
 constexpr int kSegCols = 1024;  // elements per wavefront row segment
 
-template <typename T, int LAYOUT>
-__global__ __launch_bounds__(256) void nvfp4_quantize_kernel(const T* __restrict__ in, int64_t rows, int64_t cols,
+// value -> nearest value of the 16-bit type T (round to nearest even), as fp32
+template <typename T>
+__device__ __forceinline__ float round_to(float v);
+template <>
+__device__ __forceinline__ float round_to<bf16_t>(float v) { return (float)(__bf16)v; }
+template <>
+__device__ __forceinline__ float round_to<f16_t>(float v) { return (float)(_Float16)v; }
+template <>
+__device__ __forceinline__ float round_to<float>(float v) { return v; }
+
+// SILU_MUL: the quantizer's input is silu(in) * in_up, evaluated the way the eager chain
+// `torch.nn.functional.silu(gate) * up` evaluates it on tensors of type T - silu as x / (1 + exp(-x)) in fp32,
+// rounded to T, the product in fp32, rounded to T - so the fused kernel returns the bytes of the chain
+// (benchmarks/python/layers_for_inference_benchmark.py:504 followed by the grouped quantizer) without the
+// chain's write and re-read of the intermediate.
+template <typename T, int LAYOUT, bool SILU_MUL = false>
+__global__ __launch_bounds__(256) void nvfp4_quantize_kernel(const T* __restrict__ in, const T* __restrict__ in_up,
+                                                             int64_t rows, int64_t cols,
                                                              const float* __restrict__ gs_ptr,
                                                              const int32_t* __restrict__ in_off,
                                                              const int32_t* __restrict__ out_off, int groups,
@@ -152,6 +168,8 @@ __global__ __launch_bounds__(256) void nvfp4_quantize_kernel(const T* __restrict
   const bool word_scales = !(LAYOUT == LAYOUT_LINEAR && (sf_cols & 3) != 0);
 
   const Raw16<T> raw = issue16(active ? in + row * cols + col : in);
+  Raw16<T> raw_up;
+  if constexpr (SILU_MUL) raw_up = issue16(active ? in_up + row * cols + col : in_up);
 
   const bool use_gs = gs_ptr != nullptr;
   const float gs = use_gs ? *gs_ptr : 1.0f;
@@ -173,6 +191,18 @@ __global__ __launch_bounds__(256) void nvfp4_quantize_kernel(const T* __restrict
   float x[16];
   bool nonfinite;
   decode16(raw, active, x, nonfinite);
+  if constexpr (SILU_MUL) {
+    float u[16];
+    bool up_nonfinite;
+    decode16(raw_up, active, u, up_nonfinite);
+    nonfinite = false;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const float act = round_to<T>(x[j] / (1.0f + expf(-x[j])));
+      x[j] = round_to<T>(act * u[j]);
+      nonfinite |= !(fabsf(x[j]) < INFINITY);
+    }
+  }
   const bool wave_nonfinite = __builtin_amdgcn_ballot_w64(nonfinite) != 0;
 
   // amax, NaN ignored (fmaxf), start -inf: block_quantization_kernels.cu:124-128
@@ -234,8 +264,8 @@ __global__ __launch_bounds__(256) void nvfp4_quantize_kernel(const T* __restrict
   }
 }
 
-template <typename T, int LAYOUT>
-int launch_nvfp4_layout(const T* in, int64_t rows, int64_t cols, const float* gs, const int32_t* in_off,
+template <typename T, int LAYOUT, bool SILU_MUL>
+int launch_nvfp4_layout(const T* in, const T* in_up, int64_t rows, int64_t cols, const float* gs, const int32_t* in_off,
                         const int32_t* out_off, int groups, uint8_t* out_fp4, uint8_t* out_sf, hipStream_t stream) {
   const int64_t segs = ceil_div(cols, kSegCols);
   // rows the grid must cover: the swizzled layout also zero-fills the padding rows of the last tile
@@ -243,19 +273,103 @@ int launch_nvfp4_layout(const T* in, int64_t rows, int64_t cols, const float* gs
   const int64_t wgs = ceil_div(cover, 4) * segs;
   if (wgs >= ((int64_t)1 << 31)) return fail(NVF_ERR_UNSUPPORTED_SHAPE, "tensor of %lld x %lld is too large for one launch",
                                              (long long)rows, (long long)cols);
-  hipLaunchKernelGGL((nvfp4_quantize_kernel<T, LAYOUT>), dim3((unsigned)wgs), dim3(256), 0, stream, in, rows, cols, gs,
-                     in_off, out_off, groups, (uint32_t)segs, out_fp4, out_sf);
+  hipLaunchKernelGGL((nvfp4_quantize_kernel<T, LAYOUT, SILU_MUL>), dim3((unsigned)wgs), dim3(256), 0, stream, in, in_up, rows,
+                     cols, gs, in_off, out_off, groups, (uint32_t)segs, out_fp4, out_sf);
   return check_launch("nvfp4_quantize_kernel");
 }
 
-template <typename T>
-int launch_nvfp4_typed(const T* in, int64_t rows, int64_t cols, const float* gs, int layout, const int32_t* in_off,
-                       const int32_t* out_off, int groups, uint8_t* out_fp4, uint8_t* out_sf, hipStream_t stream) {
+template <typename T, bool SILU_MUL>
+int launch_nvfp4_typed(const T* in, const T* in_up, int64_t rows, int64_t cols, const float* gs, int layout,
+                       const int32_t* in_off, const int32_t* out_off, int groups, uint8_t* out_fp4, uint8_t* out_sf,
+                       hipStream_t stream) {
   if (layout == LAYOUT_SWIZZLED)
-    return launch_nvfp4_layout<T, LAYOUT_SWIZZLED>(in, rows, cols, gs, in_off, out_off, groups, out_fp4, out_sf, stream);
+    return launch_nvfp4_layout<T, LAYOUT_SWIZZLED, SILU_MUL>(in, in_up, rows, cols, gs, in_off, out_off, groups, out_fp4, out_sf,
+                                                             stream);
   if (layout == LAYOUT_GROUPED)
-    return launch_nvfp4_layout<T, LAYOUT_GROUPED>(in, rows, cols, gs, in_off, out_off, groups, out_fp4, out_sf, stream);
-  return launch_nvfp4_layout<T, LAYOUT_LINEAR>(in, rows, cols, gs, in_off, out_off, groups, out_fp4, out_sf, stream);
+    return launch_nvfp4_layout<T, LAYOUT_GROUPED, SILU_MUL>(in, in_up, rows, cols, gs, in_off, out_off, groups, out_fp4, out_sf,
+                                                            stream);
+  return launch_nvfp4_layout<T, LAYOUT_LINEAR, SILU_MUL>(in, in_up, rows, cols, gs, in_off, out_off, groups, out_fp4, out_sf,
+                                                         stream);
+}
+
+// -------------------------------------------------------------------------------------------------
+// Global (per-tensor) NVFP4 encode scale 448 * 6 / max|x| on the device, for the quantizer's global_scale
+// argument; restates compute_nvfp4_global_scale of tests/python/direct/test_narrow_precision.py:138-156
+// without its host round trip: 1.0 for an all-zero tensor, clamped to FLT_MAX, NaN if the tensor holds
+// one (torch.max propagates it), the quotient evaluated in double and rounded once to fp32 as Python
+// does.  |x| is compared through its fp32 bit pattern, whose unsigned order is the numeric order of
+// non-negative floats with NaN on top; the maximum is order-independent, hence deterministic.
+// -------------------------------------------------------------------------------------------------
+__device__ __forceinline__ uint32_t abs_bits(bf16_t v) { return (uint32_t)(v.v & 0x7fffu) << 16; }
+__device__ __forceinline__ uint32_t abs_bits(f16_t v) {
+  return f32_to_bits((float)__builtin_bit_cast(_Float16, (uint16_t)(v.v & 0x7fffu)));
+}
+__device__ __forceinline__ uint32_t abs_bits(float v) { return f32_to_bits(v) & 0x7fffffffu; }
+
+__global__ void amax_init_kernel(uint32_t* cell) { *cell = 0u; }
+
+template <typename T>
+__global__ __launch_bounds__(256) void amax_kernel(const T* __restrict__ in, int64_t n, int64_t head, int64_t nvec,
+                                                   uint32_t* __restrict__ cell) {
+  constexpr int VE = 16 / (int)sizeof(T);  // elements per 16-byte load
+  const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  uint32_t m = 0;
+  const u32x4* vec = reinterpret_cast<const u32x4*>(in + head);
+  auto fold = [&](const u32x4 q) {
+    T e[VE];
+    __builtin_memcpy(e, &q, 16);
+#pragma unroll
+    for (int j = 0; j < VE; ++j) m = max(m, abs_bits(e[j]));
+  };
+  int64_t i = tid;
+  for (; i + 3 * stride < nvec; i += 4 * stride) {  // four loads in flight per thread
+    const u32x4 q0 = __builtin_nontemporal_load(vec + i), q1 = __builtin_nontemporal_load(vec + i + stride);
+    const u32x4 q2 = __builtin_nontemporal_load(vec + i + 2 * stride), q3 = __builtin_nontemporal_load(vec + i + 3 * stride);
+    fold(q0);
+    fold(q1);
+    fold(q2);
+    fold(q3);
+  }
+  for (; i < nvec; i += stride) fold(__builtin_nontemporal_load(vec + i));
+  // elements before the first and after the last whole 16-byte vector
+  const int64_t tail0 = head + nvec * VE;
+  for (int64_t t = tid; t < head + (n - tail0); t += stride) m = max(m, abs_bits(in[t < head ? t : tail0 + (t - head)]));
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) m = max(m, (uint32_t)__shfl_xor((int)m, d, 64));
+  if ((threadIdx.x & 63) == 0 && m != 0) atomicMax(cell, m);
+}
+
+__global__ void amax_to_global_scale_kernel(uint32_t* cell) {
+  const float amax = bits_to_f32(*cell);
+  float scale;
+  if (amax != amax) scale = amax;
+  else if (amax == 0.0f) scale = 1.0f;
+  else {
+    const double q = 2688.0 / (double)amax;  // FLOAT8_E4M3_MAX * FLOAT4_E2M1_MAX
+    scale = q > (double)FLT_MAX ? FLT_MAX : (float)q;
+  }
+  *reinterpret_cast<float*>(cell) = scale;
+}
+
+template <typename T>
+int launch_global_scale_typed(const T* in, int64_t n, float* out, hipStream_t stream) {
+  constexpr int VE = 16 / (int)sizeof(T);
+  uint32_t* cell = reinterpret_cast<uint32_t*>(out);
+  hipLaunchKernelGGL(amax_init_kernel, dim3(1), dim3(1), 0, stream, cell);
+  if (n > 0) {
+    const uintptr_t addr = reinterpret_cast<uintptr_t>(in);
+    int64_t head = (int64_t)(((16 - (addr & 15)) & 15) / sizeof(T));  // elements up to 16-byte alignment
+    if (head > n) head = n;
+    const int64_t nvec = (n - head) / VE;
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    const int64_t want = ceil_div(nvec > 0 ? nvec : 1, 256 * 4);  // at least 4 loads per thread
+    const int64_t cap = (int64_t)cus * 8;
+    hipLaunchKernelGGL(amax_kernel<T>, dim3((unsigned)(want < cap ? want : cap)), dim3(256), 0, stream, in, n, head, nvec, cell);
+  }
+  hipLaunchKernelGGL(amax_to_global_scale_kernel, dim3(1), dim3(1), 0, stream, cell);
+  return check_launch("nvfp4_global_scale");
 }
 
 // -------------------------------------------------------------------------------------------------
@@ -381,11 +495,39 @@ int launch_nvfp4_quantize(const void* in, int in_dtype, int64_t rows, int64_t co
   uint8_t* s = static_cast<uint8_t*>(out_sf);
   switch (in_dtype) {
     case NVF_F32:
-      return launch_nvfp4_typed(static_cast<const float*>(in), rows, cols, gs, layout, in_off, out_off, groups, q, s, stream);
+      return launch_nvfp4_typed<float, false>(static_cast<const float*>(in), nullptr, rows, cols, gs, layout, in_off, out_off,
+                                              groups, q, s, stream);
     case NVF_BF16:
-      return launch_nvfp4_typed(static_cast<const bf16_t*>(in), rows, cols, gs, layout, in_off, out_off, groups, q, s, stream);
+      return launch_nvfp4_typed<bf16_t, false>(static_cast<const bf16_t*>(in), nullptr, rows, cols, gs, layout, in_off, out_off,
+                                               groups, q, s, stream);
     case NVF_F16:
-      return launch_nvfp4_typed(static_cast<const f16_t*>(in), rows, cols, gs, layout, in_off, out_off, groups, q, s, stream);
+      return launch_nvfp4_typed<f16_t, false>(static_cast<const f16_t*>(in), nullptr, rows, cols, gs, layout, in_off, out_off,
+                                              groups, q, s, stream);
+  }
+  return fail(NVF_ERR_INVALID_ARGUMENT, "unknown input dtype %d", in_dtype);
+}
+
+int launch_nvfp4_silu_mul_quantize(const void* gate, const void* up, int in_dtype, int64_t rows, int64_t cols, const float* gs,
+                                   int layout, const int32_t* in_off, const int32_t* out_off, int groups, void* out_fp4,
+                                   void* out_sf, hipStream_t stream) {
+  uint8_t* q = static_cast<uint8_t*>(out_fp4);
+  uint8_t* s = static_cast<uint8_t*>(out_sf);
+  switch (in_dtype) {
+    case NVF_BF16:
+      return launch_nvfp4_typed<bf16_t, true>(static_cast<const bf16_t*>(gate), static_cast<const bf16_t*>(up), rows, cols, gs,
+                                              layout, in_off, out_off, groups, q, s, stream);
+    case NVF_F16:
+      return launch_nvfp4_typed<f16_t, true>(static_cast<const f16_t*>(gate), static_cast<const f16_t*>(up), rows, cols, gs,
+                                             layout, in_off, out_off, groups, q, s, stream);
+  }
+  return fail(NVF_ERR_INVALID_ARGUMENT, "silu-mul quantize takes bf16 or f16 inputs, got dtype %d", in_dtype);
+}
+
+int launch_nvfp4_global_scale(const void* in, int in_dtype, int64_t n, float* out, hipStream_t stream) {
+  switch (in_dtype) {
+    case NVF_F32: return launch_global_scale_typed(static_cast<const float*>(in), n, out, stream);
+    case NVF_BF16: return launch_global_scale_typed(static_cast<const bf16_t*>(in), n, out, stream);
+    case NVF_F16: return launch_global_scale_typed(static_cast<const f16_t*>(in), n, out, stream);
   }
   return fail(NVF_ERR_INVALID_ARGUMENT, "unknown input dtype %d", in_dtype);
 }

@@ -31,3 +31,17 @@ def nv_grouped_block_quantize(input, input_offsets, output_offsets, global_scale
 def preprocess_grouped_matmul_input_sf(input, input_offsets, output_offsets):
     """Copies linear block scales [M, C] into the per-group padded 128x4 layout."""
     return _C.preprocess_grouped_matmul_input_sf(input, input_offsets, output_offsets)
+
+
+def silu_mul_nv_grouped_block_quantize(gate, up, input_offsets, output_offsets, global_scale=None):
+    """``nv_grouped_block_quantize(torch.nn.functional.silu(gate) * up, ...)`` in one kernel: the product is
+    formed in registers with the eager chain's roundings (silu and product each rounded to the inputs'
+    bf16 / f16 type) and never written to memory."""
+    return _C.silu_mul_nv_grouped_block_quantize(gate, up, input_offsets, output_offsets, global_scale)
+
+
+def compute_nvfp4_global_scale(tensor):
+    """0-dim fp32 device tensor ``448 * 6 / max|tensor|`` (1.0 for an all-zero tensor, clamped to the fp32
+    maximum), as tests/python/direct/test_narrow_precision.py:138-156 defines the NVFP4 global scale, computed
+    on the device without a host round trip; pass it as ``global_scale`` to the quantizers."""
+    return _C.compute_nvfp4_global_scale(tensor)

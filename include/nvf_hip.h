@@ -77,6 +77,25 @@ NVF_API int nvf_nvfp4_grouped_block_quantize(const void* in, int in_dtype, int64
                                              int groups, const float* global_scale, void* out_fp4,
                                              void* out_scales, void* stream);
 
+/* The step ahead of nv_grouped_block_quantize in the reference's NVFP4 MoE layer, fused into the quantizer:
+ * the input is silu(gate) * up as benchmarks/python/layers_for_inference_benchmark.py:504 computes it on
+ * tensors of the inputs' type (silu = x / (1 + exp(-x)) in fp32 rounded to that type, product in fp32 rounded
+ * to that type), then quantized exactly as nvf_nvfp4_grouped_block_quantize does.  gate, up: [rows, cols]
+ * bf16 or f16.  input_offsets == NULL selects the ungrouped quantizer with the 128x4 scale layout
+ * (swizzle = 1 of nvf_nvfp4_block_quantize); output_offsets and groups are then ignored.
+ */
+NVF_API int nvf_nvfp4_silu_mul_block_quantize(const void* gate, const void* up, int in_dtype, int64_t rows,
+                                              int64_t cols, const int32_t* input_offsets,
+                                              const int32_t* output_offsets, int groups, const float* global_scale,
+                                              void* out_fp4, void* out_scales, void* stream);
+
+/* The step ahead of nv_block_quantize when a global scale is used: compute_nvfp4_global_scale of
+ * tests/python/direct/test_narrow_precision.py:138-156 on the device, without its host round trip.
+ * out_scale[0] = min(448 * 6 / max|in|, FLT_MAX), 1.0 if the tensor is all zero, NaN if it holds a NaN;
+ * in: numel elements of in_dtype (f32, bf16, f16), any alignment of the element type.
+ */
+NVF_API int nvf_nvfp4_global_scale(const void* in, int in_dtype, int64_t numel, float* out_scale, void* stream);
+
 /* runtime/block_quantization_kernels.cu:321-361 bq::preprocessGroupedMatmulInputSf
  * (graph op preprocess_grouped_matmul_input_sf, python/python_direct/ops.cpp:3179-3212).
  * Pure layout: copies a linear [rows, cols] matrix of elem_size-byte elements (1, 2 or 4) into

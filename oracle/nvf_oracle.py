@@ -301,3 +301,27 @@ def ref_nvfp4_scaled_grouped_mm(a, b, a_sf, b_sf, alphas, problem_sizes, expert_
         db = dequantize_nvfp4_fast(b8[e], bsf[e])
         out[off : off + me] = (da @ db.t()) * float(alphas[e])
     return out
+
+
+def compute_nvfp4_global_scale(tensor) -> float:
+    """(448 * 6) / max|tensor| as a Python float that the caller stores as fp32; 1.0 for an all-zero tensor,
+    clamped to the fp32 maximum (tests/python/direct/test_narrow_precision.py:138-156).  Pinned by closed
+    forms in tests/test_oracle_fused_producers.py (amax 2688 -> 1, amax 1 -> 2688, zeros -> 1, tiny -> fp32 max)."""
+    amax = torch.max(torch.abs(tensor)).to(torch.float32).item()
+    if amax == 0.0:
+        return 1.0
+    return min(2688.0 / amax, torch.finfo(torch.float32).max)
+
+
+def silu_mul(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """``silu(gate) * up`` evaluated as the reference's layer does on bf16 / f16 tensors
+    (benchmarks/python/layers_for_inference_benchmark.py:504): torch's silu, x / (1 + exp(-x)) in fp32 rounded
+    to the tensor type, then the product in fp32 rounded to the tensor type.  Written out with explicit
+    roundings so that it does not depend on the CPU's vectorised silu.  PARITY UNPINNED for the fused
+    silu-mul quantizer built on it: the reference has no eager kernel or fixture for that fusion (its
+    compiler generates one per graph); the GPU tests compare against this chain and against torch's own
+    kernels on the GPU."""
+    t = gate.dtype
+    g = gate.float()
+    act = (g / (1.0 + torch.exp(-g))).to(t)
+    return (act.float() * up.float()).to(t)
