@@ -24,6 +24,8 @@ SIGNATURES = {
     "nvf_cast_f32_to_e4m3": (_int, [_p, _i64, _p, _p]),
     "nvf_cast_f32_to_e8m0": (_int, [_p, _i64, _p, _p]),
     "nvf_nvfp4_scaled_mm": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _int, _p]),
+    "nvf_nvfp4_scaled_mm_workspace_bytes": (_i64, [_i64, _i64, _i64]),
+    "nvf_nvfp4_scaled_mm_ws": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _int, _p, _i64, _p]),
     "nvf_nvfp4_scaled_mm_blockscale": (_int, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p]),
     "nvf_mxfp8_scaled_mm": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _int, _p]),
     "nvf_grouped_mm": (_int, [_p, _p, _p, _p, _p, _int, _i64, _i64, _i64, _int, _p]),

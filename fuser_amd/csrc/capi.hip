@@ -145,17 +145,30 @@ int nvf_cast_f32_to_e2m1(const float* in, int64_t n, uint8_t* out, void* stream)
 int nvf_cast_f32_to_e4m3(const float* in, int64_t n, uint8_t* out, void* stream) { return cast_common(1, in, n, out, stream); }
 int nvf_cast_f32_to_e8m0(const float* in, int64_t n, uint8_t* out, void* stream) { return cast_common(2, in, n, out, stream); }
 
-int nvf_nvfp4_scaled_mm(const void* a, const void* b, const void* scales_a, const void* scales_b, const float* alpha,
-                        void* out, int64_t m, int64_t n, int64_t k, int out_dtype, void* stream) {
+int nvf_nvfp4_scaled_mm_ws(const void* a, const void* b, const void* scales_a, const void* scales_b, const float* alpha,
+                           void* out, int64_t m, int64_t n, int64_t k, int out_dtype, void* workspace,
+                           int64_t workspace_bytes, void* stream) {
   NVF_REQUIRE(dtype16(out_dtype), NVF_ERR_INVALID_ARGUMENT, "output dtype must be bf16 or f16, got %d", out_dtype);
   NVF_REQUIRE(m >= 0 && n >= 0 && k >= 0, NVF_ERR_INVALID_ARGUMENT, "negative size");
   NVF_REQUIRE(k % 32 == 0, NVF_ERR_UNSUPPORTED_SHAPE, "The K dimension %lld is not divisible by 32", (long long)k);
   NVF_REQUIRE(n % 32 == 0, NVF_ERR_UNSUPPORTED_SHAPE, "The N dimension %lld is not divisible by 32", (long long)n);
+  NVF_REQUIRE(workspace_bytes >= 0, NVF_ERR_INVALID_ARGUMENT, "negative workspace size");
   if (m == 0 || n == 0) return NVF_OK;
   NVF_REQUIRE(a && b && scales_a && scales_b && alpha && out, NVF_ERR_INVALID_ARGUMENT, "NULL buffer");
   Gemm16Args g{a, b, scales_a, scales_b, alpha, out, nullptr, nullptr, nullptr, 1, m, n, k, out_dtype};
+  if (workspace != nullptr && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0) {  // fp32x4 accesses
+    g.workspace = workspace;
+    g.workspace_bytes = workspace_bytes;
+  }
   return launch_gemm16(0, g, static_cast<hipStream_t>(stream));
 }
+
+int nvf_nvfp4_scaled_mm(const void* a, const void* b, const void* scales_a, const void* scales_b, const float* alpha,
+                        void* out, int64_t m, int64_t n, int64_t k, int out_dtype, void* stream) {
+  return nvf_nvfp4_scaled_mm_ws(a, b, scales_a, scales_b, alpha, out, m, n, k, out_dtype, nullptr, 0, stream);
+}
+
+int64_t nvf_nvfp4_scaled_mm_workspace_bytes(int64_t m, int64_t n, int64_t k) { return nvfp4_gemm_workspace_bytes(m, n, k); }
 
 int nvf_nvfp4_scaled_mm_blockscale(const void* a, const void* b, const void* scales_a, const void* scales_b,
                                    const float* alpha, const float* global_normconst, void* out_fp4, void* out_scales,

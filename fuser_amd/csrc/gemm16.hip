@@ -44,6 +44,11 @@ struct Params {
   const int32_t* sf_offsets;
   int groups;
   int m, n, k;
+  // split of K over workgroups (dense NVFP4 tile kernel only): work item w = tile w / splits, K spans
+  // [ (w % splits) * spans_per_split, ... ); fp32 partial tiles go to partial[split][m][n]
+  float* partial = nullptr;
+  int splits = 1;
+  int spans_per_split = 0;
 };
 
 __device__ __forceinline__ uint32_t pack2(float a, float b, bool out_bf16) {
@@ -261,7 +266,7 @@ __global__ __launch_bounds__(256) void gemm16_kernel(const Params p) {
 //     odd step converts its even half: a full step of MFMAs hides the latency.
 // Requires K % 32 == 0 (a piece never straddles the end of a row).
 // -------------------------------------------------------------------------------------------------
-template <int BM, int BN, bool OUT_BF16, bool OUT_F32>
+template <int BM, int BN, bool OUT_BF16, bool OUT_F32, bool SPLIT_K = false>
 __global__ __launch_bounds__(256) void nvfp4_tile_kernel(const Params p) {
   constexpr int WTM = BM / 2, WTN = BN / 2;  // wave tile
   constexpr int TM = WTM / 32, TN = WTN / 32;
@@ -302,7 +307,8 @@ __global__ __launch_bounds__(256) void nvfp4_tile_kernel(const Params p) {
     if (lane == 0) tile_prefix[0] = 0;
   }
   __syncthreads();
-  const int total_tiles = tile_prefix[p.groups];
+  const int splits = SPLIT_K ? p.splits : 1;
+  const int total_tiles = tile_prefix[p.groups] * splits;
 
   const int kbytes = p.k >> 1;
   const int sf_cols = p.k >> 4;
@@ -313,7 +319,11 @@ __global__ __launch_bounds__(256) void nvfp4_tile_kernel(const Params p) {
   struct Raw { u32x4 a[A_CH], b[B_CH]; uint32_t sa[A_CH], sb[B_CH]; };
   const int urow = tid >> 2, upiece = tid & 3;  // unit i of a thread: row urow + 64 * i
 
-  for (int tile = blockIdx.x; tile < total_tiles; tile += gridDim.x) {
+  for (int item = blockIdx.x; item < total_tiles; item += gridDim.x) {
+    const int tile = SPLIT_K ? item / splits : item;
+    const int split = SPLIT_K ? item - tile * splits : 0;
+    const int span0 = SPLIT_K ? split * p.spans_per_split : 0;                       // this item's K spans
+    const int span1 = SPLIT_K ? min(span0 + p.spans_per_split, nspans) : nspans;     // (never empty)
     int g = 0;
     {
       int lo = 0, hi = p.groups;
@@ -416,11 +426,11 @@ __global__ __launch_bounds__(256) void nvfp4_tile_kernel(const Params p) {
     };
 
     Raw cur, nxt;
-    issue_span(cur, 0);
+    issue_span(cur, span0);
     convert(cur, 0, 0);  // every wave is past the barrier that ended the previous tile's last step
     __syncthreads();
-    for (int sp = 0; sp < nspans; ++sp) {
-      const bool more = sp + 1 < nspans;
+    for (int sp = span0; sp < span1; ++sp) {
+      const bool more = sp + 1 < span1;
       if (more) issue_span(nxt, sp + 1);
       mfma_step(0);
       convert(cur, 1, 1);
@@ -432,7 +442,7 @@ __global__ __launch_bounds__(256) void nvfp4_tile_kernel(const Params p) {
     }
 
     // ---- epilogue: acc[i][j][r] = C[m = lane%32][n = (r/4)*8 + (lane/32)*4 + r%4] of its 32x32 tile ----
-    const float alpha = dense ? p.alpha[0] : p.alpha[g];
+    const float alpha = SPLIT_K ? 1.0f : (dense ? p.alpha[0] : p.alpha[g]);  // split: applied by the reduction
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
       const int mrow = m0 + wm * WTM + i * 32 + (lane & 31);
@@ -443,7 +453,11 @@ __global__ __launch_bounds__(256) void nvfp4_tile_kernel(const Params p) {
         for (int rq = 0; rq < 4; ++rq) {
           const int ncol = n0 + wn * WTN + j * 32 + rq * 8 + (lane >> 5) * 4;
           if (ncol >= p.n) continue;
-          if constexpr (OUT_F32) {
+          if constexpr (SPLIT_K) {
+            float* frow = p.partial + ((int64_t)split * p.m + mrow) * (int64_t)p.n;
+            *reinterpret_cast<f32x4*>(frow + ncol) =
+                f32x4{acc[i][j][rq * 4 + 0], acc[i][j][rq * 4 + 1], acc[i][j][rq * 4 + 2], acc[i][j][rq * 4 + 3]};
+          } else if constexpr (OUT_F32) {
             float* frow = static_cast<float*>(p.out) + (row_off + mrow) * (int64_t)p.n;
             *reinterpret_cast<f32x4*>(frow + ncol) = f32x4{acc[i][j][rq * 4 + 0] * alpha, acc[i][j][rq * 4 + 1] * alpha,
                                                            acc[i][j][rq * 4 + 2] * alpha, acc[i][j][rq * 4 + 3] * alpha};
@@ -458,6 +472,21 @@ __global__ __launch_bounds__(256) void nvfp4_tile_kernel(const Params p) {
       }
     }
   }
+}
+
+// out[m][n] = alpha * (partial[0][m][n] + partial[1][m][n] + ...), summed in that order
+template <bool OUT_BF16>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial, int splits, int64_t mn,
+                                                            const float* __restrict__ alpha_ptr, uint16_t* __restrict__ out) {
+  const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (i >= mn) return;  // mn % 4 == 0 (N % 32 == 0)
+  f32x4 s = *reinterpret_cast<const f32x4*>(partial + i);
+  for (int k = 1; k < splits; ++k) s += *reinterpret_cast<const f32x4*>(partial + (int64_t)k * mn + i);
+  const float alpha = alpha_ptr[0];
+  u32x2 v;
+  v[0] = pack2(s[0] * alpha, s[1] * alpha, OUT_BF16);
+  v[1] = pack2(s[2] * alpha, s[3] * alpha, OUT_BF16);
+  *reinterpret_cast<u32x2*>(out + i) = v;
 }
 
 // -------------------------------------------------------------------------------------------------
@@ -1356,6 +1385,44 @@ int launch_nvfp4_tile(const Params& p, int grid, hipStream_t stream) {
   return check_launch("nvfp4_tile_kernel");
 }
 
+// Split of K for dense NVFP4 shapes with fewer 128x128 tiles than compute units and a deep K (decode and
+// small prefill batches against a down projection): about two work items per compute unit, at least eight
+// 128-deep spans each.  Every split writes and the reduction re-reads an fp32 copy of the output, so for
+// K below 8192 the split costs more than it gains (measured) and 1 is returned.
+int nvfp4_splits(int64_t m, int64_t n, int64_t k, int cus) {
+  const int64_t tiles = ceil_div(m, 128) * ceil_div(n, 128), nspans = ceil_div(k, 128);
+  if (m <= 64 || tiles >= cus || nspans < 64) return 1;
+  int64_t s = (2 * (int64_t)cus) / tiles;
+  if (s > nspans / 8) s = nspans / 8;
+  if (s > 32) s = 32;
+  return s < 2 ? 1 : (int)s;
+}
+
+template <bool OUT_BF16>
+int launch_nvfp4_splitk(const Params& p0, int splits, float* workspace, hipStream_t stream) {
+  Params p = p0;
+  const int nspans = (p.k + 127) >> 7;
+  p.spans_per_split = (nspans + splits - 1) / splits;
+  p.splits = (nspans + p.spans_per_split - 1) / p.spans_per_split;  // no empty split
+  p.partial = workspace;
+  auto kern = nvfp4_tile_kernel<128, 128, OUT_BF16, false, true>;
+  constexpr int lds_bytes = 2 * (128 + 128) * 128;
+  static bool configured = false;  // benign race: the attribute call is idempotent
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    if (e != hipSuccess) return fail(NVF_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    configured = true;
+  }
+  const int64_t items = ceil_div(p.m, 128) * ceil_div(p.n, 128) * p.splits;
+  hipLaunchKernelGGL(kern, dim3((unsigned)items), dim3(256), lds_bytes, stream, p);
+  int rc = check_launch("nvfp4_tile_kernel (split K)");
+  if (rc != NVF_OK) return rc;
+  const int64_t mn = (int64_t)p.m * p.n;
+  hipLaunchKernelGGL(splitk_reduce_kernel<OUT_BF16>, dim3((unsigned)ceil_div(mn / 4, 256)), dim3(256), 0, stream, workspace, p.splits,
+                     mn, p.alpha, static_cast<uint16_t*>(p.out));
+  return check_launch("splitk_reduce_kernel");
+}
+
 // tile kernel of the operand type: NVFP4 or 16-bit
 template <int BM, int BN, bool NVFP4, bool BF16_MMA, bool OUT_BF16>
 int launch_tile(const Params& p, int grid, hipStream_t stream) {
@@ -1364,11 +1431,16 @@ int launch_tile(const Params& p, int grid, hipStream_t stream) {
 }
 
 template <bool NVFP4, bool BF16_MMA, bool OUT_BF16>
-int launch_sized(const Params& p, int64_t m_hint, int cus, hipStream_t stream) {
+int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int64_t workspace_bytes, hipStream_t stream) {
   // Pick the largest tile that still yields about one work item per compute unit.
   auto tiles = [&](int bm, int bn) { return ceil_div(m_hint, bm) * ceil_div(p.n, bn); };
   const bool dense = p.problem_sizes == nullptr;
   if constexpr (NVFP4) {
+    if (dense && workspace != nullptr) {
+      const int splits = nvfp4_splits(p.m, p.n, p.k, cus);
+      if (splits > 1 && workspace_bytes >= (int64_t)splits * p.m * p.n * 4)
+        return launch_nvfp4_splitk<OUT_BF16>(p, splits, static_cast<float*>(workspace), stream);
+    }
     if (dense && p.m <= 128 && (p.k & 127) == 0 && (p.n & 15) == 0) return launch_nvfp4_skinny<OUT_BF16>(p, cus, stream);
     if (dense && (p.m & 255) == 0 && (p.n & 255) == 0 && (p.k & 127) == 0 && p.k >= 256) {
       // The 256x256 kernel is about 1.4 times as fast per tile-flop as the tile kernel below, so it wins
@@ -1445,9 +1517,17 @@ int launch_gemm16(int op, const Gemm16Args& a, hipStream_t stream) {
   const bool bf16 = a.dtype == NVF_BF16;
   if (op == 0 && a.dtype == NVF_F32) return launch_nvfp4_f32(p, cus, stream);
   if (op == 0 || op == 1) {
-    return bf16 ? launch_sized<true, false, true>(p, a.m, cus, stream) : launch_sized<true, false, false>(p, a.m, cus, stream);
+    return bf16 ? launch_sized<true, false, true>(p, a.m, cus, a.workspace, a.workspace_bytes, stream)
+                : launch_sized<true, false, false>(p, a.m, cus, a.workspace, a.workspace_bytes, stream);
   }
-  return bf16 ? launch_sized<false, true, true>(p, a.m, cus, stream) : launch_sized<false, false, false>(p, a.m, cus, stream);
+  return bf16 ? launch_sized<false, true, true>(p, a.m, cus, nullptr, 0, stream)
+              : launch_sized<false, false, false>(p, a.m, cus, nullptr, 0, stream);
+}
+
+int64_t nvfp4_gemm_workspace_bytes(int64_t m, int64_t n, int64_t k) {
+  if (m <= 0 || n <= 0 || k <= 0 || m > INT32_MAX || n > INT32_MAX || k > INT32_MAX) return 0;
+  const int splits = nvfp4_splits(m, n, k, cu_count());
+  return splits > 1 ? (int64_t)splits * m * n * 4 : 0;
 }
 
 }  // namespace nvf

@@ -143,9 +143,14 @@ torch::Tensor nvfp4_scaled_mm(const torch::Tensor& a, const torch::Tensor& b, co
   if (out_dtype != at::ScalarType::Half && out_dtype != at::ScalarType::BFloat16) {
     NVF_THROW("Unsupported output data type of nvfp4 scaled_mm.");
   }
-  check_status(nvf_nvfp4_scaled_mm(a.data_ptr(), b.data_ptr(), scales_a.data_ptr(), scales_b.data_ptr(),
-                                   static_cast<const float*>(alpha.data_ptr()), output.data_ptr(), m, n, k,
-                                   to_nvf_dtype(out_dtype), stream),
+  // scratch for the shapes that split K, from torch's stream-ordered allocator (the reference allocates its
+  // kernel's workspace in the same place, cutlass/nvfp4_scaled_mm.cu:241-244)
+  const int64_t ws_bytes = nvf_nvfp4_scaled_mm_workspace_bytes(m, n, k);
+  torch::Tensor workspace;
+  if (ws_bytes > 0) workspace = at::empty({ws_bytes}, at::TensorOptions().dtype(at::ScalarType::Byte).device(a.device()));
+  check_status(nvf_nvfp4_scaled_mm_ws(a.data_ptr(), b.data_ptr(), scales_a.data_ptr(), scales_b.data_ptr(),
+                                      static_cast<const float*>(alpha.data_ptr()), output.data_ptr(), m, n, k,
+                                      to_nvf_dtype(out_dtype), ws_bytes > 0 ? workspace.data_ptr() : nullptr, ws_bytes, stream),
                "nvfp4_scaled_mm");
   return output;
 }

@@ -53,8 +53,12 @@ struct Gemm16Args {
   int groups;
   int64_t m, n, k;
   int dtype;  // out dtype (NVFP4 ops) or in/out dtype (grouped_mm)
+  void* workspace = nullptr;  // dense NVFP4: optional scratch for a split of K (nvfp4_gemm_workspace_bytes)
+  int64_t workspace_bytes = 0;
 };
 int launch_gemm16(int op, const Gemm16Args& args, hipStream_t stream);
+// scratch bytes with which the dense NVFP4 GEMM of this shape runs faster (0: none needed)
+int64_t nvfp4_gemm_workspace_bytes(int64_t m, int64_t n, int64_t k);
 int launch_mxfp8_gemm(const void* a, const void* b, const void* sfa, const void* sfb, const float* alpha, void* out,
                       int64_t m, int64_t n, int64_t k, int out_dtype, hipStream_t stream);
 

@@ -132,6 +132,18 @@ NVF_API int nvf_nvfp4_scaled_mm(const void* a, const void* b, const void* scales
                                 const float* alpha, void* out, int64_t m, int64_t n, int64_t k,
                                 int out_dtype, void* stream);
 
+/* The same op with scratch memory, as the reference's entry point allocates a workspace for its kernel
+ * (cutlass/nvfp4_scaled_mm.cu:241-256).  nvf_nvfp4_scaled_mm_workspace_bytes returns the number of bytes with
+ * which this shape runs faster (0 for most shapes: then workspace may be NULL); with at least that many
+ * bytes of device memory, shapes with few output tiles and a deep K (decode and small prefill batches) split
+ * K over workgroups, keep fp32 partial products in the workspace and add them in a fixed order
+ * (deterministic).  With less, the call is nvf_nvfp4_scaled_mm.  The workspace must not be shared with a
+ * call that may run at the same time. */
+NVF_API int64_t nvf_nvfp4_scaled_mm_workspace_bytes(int64_t m, int64_t n, int64_t k);
+NVF_API int nvf_nvfp4_scaled_mm_ws(const void* a, const void* b, const void* scales_a, const void* scales_b,
+                                   const float* alpha, void* out, int64_t m, int64_t n, int64_t k, int out_dtype,
+                                   void* workspace, int64_t workspace_bytes, void* stream);
+
 /* cutlass/nvfp4_scaled_mm_blockscale.cu:332-373 nvfp4_scaled_mm_blockscale (decl cutlass/nvf_cutlass.h:147-154).
  *   Operands as nvf_nvfp4_scaled_mm.  The fp32 product alpha * A * B^T is quantized again along n with
  *   the NVFP4 block quantizer (block 16, global scale *global_normconst): out_fp4 [m, n/2], out_scales

@@ -181,6 +181,49 @@ def test_nvfp4_gemm_decode_sized_activations(dev, shape):
         assert torch.equal(out, _run_nvfp4(a, b, sa_p, sb, alpha, dtype, dev))
 
 
+@pytest.mark.parametrize("shape", [(128, 1024, 8192), (100, 256, 8224), (200, 512, 10240), (65, 160, 9216), (300, 2048, 14336)])
+def test_nvfp4_gemm_split_k_with_workspace(dev, shape):
+    """Few 128x128 output tiles and a deep K: with the scratch memory that
+    nvf_nvfp4_scaled_mm_workspace_bytes asks for, K is split over workgroups and fp32 partial tiles are
+    added in a fixed order.  Ragged M / N / K (K not a multiple of the 128-deep span, splits that do not
+    divide the spans), both output types, against the oracle; run-to-run bit equality; a workspace that is
+    too small, NULL or misaligned falls back to the kernels without one."""
+    from fuser_amd import capi
+
+    m, n, k = shape
+    gen = torch.Generator().manual_seed(m + k)
+    a, sa, ga = _nvfp4_operand(m, k, 1.0, gen)
+    b, sb, gb = _nvfp4_operand(n, k, 0.02, gen)
+    alpha = 1.0 / (ga * gb)
+    ref = O.ref_nvfp4_scaled_mm(a, b, sa, sb, alpha)
+    need = capi.lib().nvf_nvfp4_scaled_mm_workspace_bytes(m, n, k)
+    assert need >= 2 * m * n * 4 and need % (m * n * 4) == 0
+    ad, bd, sad, sbd = a.to(dev), b.to(dev), sa.to(dev), sb.to(dev)
+    al = torch.tensor(alpha, dtype=torch.float32, device=dev)
+    ws = torch.empty(need + 16, dtype=torch.uint8, device=dev)
+
+    def run(dt, ws_ptr, ws_bytes):
+        out = torch.full((m, n), 7.0, dtype=dt, device=dev)
+        code = capi.BF16 if dt == torch.bfloat16 else capi.F16
+        capi.check(capi.lib().nvf_nvfp4_scaled_mm_ws(ad.data_ptr(), bd.data_ptr(), sad.data_ptr(), sbd.data_ptr(), al.data_ptr(),
+                                                     out.data_ptr(), m, n, k, code, ws_ptr, ws_bytes, None))
+        torch.cuda.synchronize()
+        return out
+
+    for dt in (torch.bfloat16, torch.float16):
+        ws.fill_(0xFF)  # NaN patterns: every partial that is read must have been written
+        out = run(dt, ws.data_ptr(), need)
+        assert max_rel(out, ref) <= GEMM_MAX_REL, (shape, dt)
+        assert torch.equal(out, run(dt, ws.data_ptr(), need))
+        for ptr, size in ((None, 0), (ws.data_ptr(), need - 1), (ws.data_ptr() + 4, need)):
+            assert max_rel(run(dt, ptr, size), ref) <= GEMM_MAX_REL, (shape, dt, size)
+    # the at::Tensor entry point allocates the scratch itself
+    assert torch.equal(_run_nvfp4(a, b, sa, sb, alpha, torch.bfloat16, dev), run(torch.bfloat16, ws.data_ptr(), need))
+    # shapes that fill the chip or are served by the weight-streaming kernel ask for nothing
+    assert capi.lib().nvf_nvfp4_scaled_mm_workspace_bytes(4096, 4096, 4096) == 0
+    assert capi.lib().nvf_nvfp4_scaled_mm_workspace_bytes(16, 4096, 4096) == 0
+
+
 def test_nvfp4_gemm_ignores_scale_padding_and_is_deterministic(dev):
     gen = torch.Generator().manual_seed(9)
     m, n, k = 100, 160, 96  # k/16 = 6 -> padded to 8 ; rows padded to 128 / 256
