@@ -340,21 +340,42 @@ __global__ __launch_bounds__(256) void amax_kernel(const T* __restrict__ in, int
   if ((threadIdx.x & 63) == 0 && m != 0) atomicMax(cell, m);
 }
 
+__device__ __forceinline__ float amax_bits_to_global_scale(uint32_t amax_bits) {
+  const float amax = bits_to_f32(amax_bits);
+  if (amax != amax) return amax;
+  if (amax == 0.0f) return 1.0f;
+  const double q = 2688.0 / (double)amax;  // FLOAT8_E4M3_MAX * FLOAT4_E2M1_MAX
+  return q > (double)FLT_MAX ? FLT_MAX : (float)q;
+}
+
 __global__ void amax_to_global_scale_kernel(uint32_t* cell) {
-  const float amax = bits_to_f32(*cell);
-  float scale;
-  if (amax != amax) scale = amax;
-  else if (amax == 0.0f) scale = 1.0f;
-  else {
-    const double q = 2688.0 / (double)amax;  // FLOAT8_E4M3_MAX * FLOAT4_E2M1_MAX
-    scale = q > (double)FLT_MAX ? FLT_MAX : (float)q;
+  *reinterpret_cast<float*>(cell) = amax_bits_to_global_scale(*cell);
+}
+
+// small tensors: one workgroup does the whole job in one launch
+template <typename T>
+__global__ __launch_bounds__(1024) void global_scale_small_kernel(const T* __restrict__ in, int64_t n, float* __restrict__ out) {
+  __shared__ uint32_t wave_max[16];
+  uint32_t m = 0;
+  for (int64_t i = threadIdx.x; i < n; i += 1024) m = max(m, abs_bits(in[i]));
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) m = max(m, (uint32_t)__shfl_xor((int)m, d, 64));
+  if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int w = 1; w < 16; ++w) m = max(m, wave_max[w]);
+    *out = amax_bits_to_global_scale(m);
   }
-  *reinterpret_cast<float*>(cell) = scale;
 }
 
 template <typename T>
 int launch_global_scale_typed(const T* in, int64_t n, float* out, hipStream_t stream) {
   constexpr int VE = 16 / (int)sizeof(T);
+  if (n <= 65536) {
+    hipLaunchKernelGGL(global_scale_small_kernel<T>, dim3(1), dim3(1024), 0, stream, in, n, out);
+    return check_launch("nvfp4_global_scale");
+  }
   uint32_t* cell = reinterpret_cast<uint32_t*>(out);
   hipLaunchKernelGGL(amax_init_kernel, dim3(1), dim3(1), 0, stream, cell);
   if (n > 0) {
