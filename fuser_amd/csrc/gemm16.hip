@@ -49,6 +49,9 @@ struct Params {
   float* partial = nullptr;
   int splits = 1;
   int spans_per_split = 0;
+  // NVFP4 tile kernel, grouped: 1 = rows [0, rows & ~255) of every group are computed by the 256x256 kernel,
+  // take only the rows after them
+  int skip_whole_256 = 0;
 };
 
 __device__ __forceinline__ uint32_t pack2(float a, float b, bool out_bf16) {
@@ -293,7 +296,8 @@ __global__ __launch_bounds__(256) void nvfp4_tile_kernel(const Params p) {
       int cnt = 0;
       if (g < p.groups) {
         const int mg = p.problem_sizes[g * 3];
-        cnt = mg > 0 ? ((mg + BM - 1) / BM) * tiles_n : 0;
+        const int rest = mg - (p.skip_whole_256 ? (mg & ~255) : 0);
+        cnt = rest > 0 ? ((rest + BM - 1) / BM) * tiles_n : 0;
       }
       int incl = cnt;
 #pragma unroll
@@ -335,10 +339,11 @@ __global__ __launch_bounds__(256) void nvfp4_tile_kernel(const Params p) {
     }
     const int m_g = dense ? p.m : p.problem_sizes[g * 3];
     const int64_t row_off = dense ? 0 : p.expert_offsets[g];
-    const int tiles_m = (m_g + BM - 1) / BM;
+    const int skipped = (!dense && p.skip_whole_256) ? (m_g & ~255) : 0;
+    const int tiles_m = (m_g - skipped + BM - 1) / BM;
     const int local = tile - tile_prefix[g];
     const int mt = local % tiles_m, nt = local / tiles_m;
-    const int m0 = mt * BM, n0 = nt * BN;
+    const int m0 = skipped + mt * BM, n0 = nt * BN;
 
     const uint8_t* a_base = p.a + (row_off + m0) * (int64_t)kbytes;
     const uint8_t* b_base = p.b + ((int64_t)g * p.n + n0) * (int64_t)kbytes;
@@ -513,12 +518,13 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
 // LDS: two buffers of (A tile + B tile), each tile 256 rows x 128 bytes with 16-byte chunk c of row r at
 // chunk position c ^ ((r >> 1) & 7): conflict-free for the fragment reads.
 // -------------------------------------------------------------------------------------------------
-template <bool OUT_BF16>
+template <bool OUT_BF16, bool GROUPED>
 __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   constexpr int BM = 256, BN = 256;
   constexpr int TILE_UNITS = 2048;           // 16-byte units per operand tile
   constexpr int BUF_UNITS = 2 * TILE_UNITS;  // A + B
   extern __shared__ u32x4 lds[];
+  __shared__ int tile_prefix[GROUPED ? kMaxGroups + 1 : 1];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -530,24 +536,68 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   // ---- persistent tile walk: workgroup ids are dealt round-robin to the 8 XCDs, XCD x owns the tile
   // range [x*chunk, (x+1)*chunk); with the 8 (m) x 4 (n) blocked numbering the 32 tiles an XCD works on
   // at a time share 8 A panels and 4 B panels in its L2.
+  // GROUPED: the work list holds only the whole 256-row tiles of every group (rows [0, rows & ~255) of
+  // the group); what is left at the end of a group goes to the tile kernel.  A group's tiles are numbered
+  // m-tile fastest, so neighbouring tiles share the group's weight panel.
   const int tiles_m = p.m / BM, tiles_n = p.n / BN;
-  const int total = tiles_m * tiles_n;
+  int total = tiles_m * tiles_n;
+  if constexpr (GROUPED) {
+    if (wave == 0) {  // prefix sums of tiles per group, 64 groups per round
+      int running = 0;
+      for (int base = 0; base < p.groups; base += 64) {
+        const int g = base + lane;
+        const int cnt = g < p.groups ? (p.problem_sizes[g * 3] / BM) * tiles_n : 0;
+        int incl = cnt;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+          const int o = __shfl_up(incl, d, 64);
+          if (lane >= d) incl += o;
+        }
+        if (g < p.groups) tile_prefix[g + 1] = running + incl;
+        running += __shfl(incl, 63, 64);
+      }
+      if (lane == 0) tile_prefix[0] = 0;
+    }
+    __syncthreads();
+    total = __builtin_amdgcn_readfirstlane(tile_prefix[p.groups]);
+  }
   const int chunk_tiles = (total + 7) >> 3;
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, slots = gridDim.x >> 3;
   const int range_end = min((xcd + 1) * chunk_tiles, total);
   const bool blocked = (tiles_m & 7) == 0 && (tiles_n & 3) == 0;
-  auto tile_coords = [&](int t, int& m0, int& n0) {
-    int mt, nt;
-    if (blocked) {
-      const int sb = t >> 5, w = t & 31;
-      mt = (sb % (tiles_m >> 3)) * 8 + (w & 7);
-      nt = (sb / (tiles_m >> 3)) * 4 + (w >> 3);
+  // tile -> group, first row of the tile among all rows of A (m0), among the rows of the group (gm0), n0
+  struct Where { int g; int64_t m0; int gm0, n0; };
+  auto tile_where = [&](int t) {
+    Where w;
+    if constexpr (GROUPED) {
+      int lo = 0, hi = p.groups;
+      while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (t < tile_prefix[mid]) hi = mid; else lo = mid;
+      }
+      w.g = __builtin_amdgcn_readfirstlane(lo);
+      const int full_m = __builtin_amdgcn_readfirstlane(p.problem_sizes[w.g * 3]) / BM;
+      const int local = __builtin_amdgcn_readfirstlane(t - tile_prefix[w.g]);
+      const int nt = local / full_m, mt = local - nt * full_m;
+      w.gm0 = mt * BM;
+      w.m0 = (int64_t)__builtin_amdgcn_readfirstlane(p.expert_offsets[w.g]) + w.gm0;
+      w.n0 = nt * BN;
     } else {
-      mt = t % tiles_m;
-      nt = t / tiles_m;
+      int mt, nt;
+      if (blocked) {
+        const int sb = t >> 5, q = t & 31;
+        mt = (sb % (tiles_m >> 3)) * 8 + (q & 7);
+        nt = (sb / (tiles_m >> 3)) * 4 + (q >> 3);
+      } else {
+        mt = t % tiles_m;
+        nt = t / tiles_m;
+      }
+      w.g = 0;
+      w.gm0 = mt * BM;
+      w.m0 = w.gm0;
+      w.n0 = nt * BN;
     }
-    m0 = mt * BM;
-    n0 = nt * BN;
+    return w;
   };
   const int first_tile = xcd * chunk_tiles + slot;
   if (first_tile >= range_end) return;
@@ -562,14 +612,16 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   // next (np); it advances by selects only
   struct RowPtrs { const uint8_t *a, *b, *sa, *sb; };
   auto tile_ptrs = [&](int t) {
-    int m0, n0;
-    tile_coords(t, m0, n0);
+    const Where w = tile_where(t);
     RowPtrs r;
-    r.a = p.a + (int64_t)(m0 + srow) * kbytes + spiece * 16;
-    r.b = p.b + (int64_t)(n0 + srow) * kbytes + spiece * 16;
+    r.a = p.a + (w.m0 + srow) * kbytes + spiece * 16;
+    r.b = p.b + ((int64_t)w.g * p.n + w.n0 + srow) * kbytes + spiece * 16;
     // scale blocks 2*spiece, 2*spiece+1 of the span: 128x4 layout column tile spiece>>1, bytes 2*(spiece&1)..
-    r.sa = p.sfa + swizzle_128x4(m0 + srow, 0, sf_padded) + (spiece >> 1) * 512 + (spiece & 1) * 2;
-    r.sb = p.sfb + swizzle_128x4(n0 + srow, 0, sf_padded) + (spiece >> 1) * 512 + (spiece & 1) * 2;
+    // (a group's activation scales are a slab of their own, swizzled from its first row)
+    const int64_t sa_slab = GROUPED ? (int64_t)__builtin_amdgcn_readfirstlane(p.sf_offsets[w.g]) * sf_padded : 0;
+    r.sa = p.sfa + sa_slab + swizzle_128x4(w.gm0 + srow, 0, sf_padded) + (spiece >> 1) * 512 + (spiece & 1) * 2;
+    r.sb = p.sfb + (int64_t)w.g * p.n * sf_padded + swizzle_128x4(w.n0 + srow, 0, sf_padded) + (spiece >> 1) * 512 +
+           (spiece & 1) * 2;
     return r;
   };
   RowPtrs lp = tile_ptrs(first_tile);
@@ -655,7 +707,6 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   asm volatile("" : "+a"(acc[0][0]), "+a"(acc[0][1]), "+a"(acc[1][0]), "+a"(acc[1][1]), "+a"(acc[2][0]),     \
                "+a"(acc[2][1]), "+a"(acc[3][0]), "+a"(acc[3][1]))
 
-  const float alpha = p.alpha[0];
   Raw cur, nxt;  // span whose odd step is converted next / span whose even step is converted next
   Frag fr[2];
 
@@ -719,12 +770,12 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
     }
     // ---- epilogue; the next tile's first step is already in LDS.
     // acc[i][j][r] = C[m = li][n = (r/4)*8 + lg*4 + r%4] of its 32x32 sub-tile.
-    int m0, n0;
-    tile_coords(c_tile, m0, n0);
+    const Where cw = tile_where(c_tile);
+    const float alpha = p.alpha[cw.g];
     uint16_t* out = static_cast<uint16_t*>(p.out);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      uint16_t* orow = out + (int64_t)(m0 + wm * 128 + i * 32 + li) * p.n + n0 + wn * 64 + lg * 4;
+      uint16_t* orow = out + (cw.m0 + wm * 128 + i * 32 + li) * p.n + cw.n0 + wn * 64 + lg * 4;
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
 #pragma unroll
@@ -741,9 +792,9 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
 #undef NVF_PIN_ACC
 }
 
-template <bool OUT_BF16>
+template <bool OUT_BF16, bool GROUPED>
 int launch_nvfp4_fast(const Params& p, int cus, hipStream_t stream) {
-  auto kern = nvfp4_gemm_256_kernel<OUT_BF16>;
+  auto kern = nvfp4_gemm_256_kernel<OUT_BF16, GROUPED>;
   constexpr int lds_bytes = 2 * 2 * 2048 * 16;  // 128 KiB
   static bool configured = false;
   if (!configured) {
@@ -751,7 +802,7 @@ int launch_nvfp4_fast(const Params& p, int cus, hipStream_t stream) {
     if (e != hipSuccess) return fail(NVF_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
     configured = true;
   }
-  const int64_t tiles = (int64_t)(p.m / 256) * (p.n / 256);
+  const int64_t tiles = (int64_t)(p.m / 256) * (p.n / 256);  // grouped: an upper bound
   const unsigned grid = (unsigned)(tiles >= cus ? (cus & ~7) : ((tiles + 7) / 8) * 8);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds_bytes, stream, p);
   return check_launch("nvfp4_gemm_256_kernel");
@@ -1446,7 +1497,7 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int6
       // The 256x256 kernel is about 1.4 times as fast per tile-flop as the tile kernel below, so it wins
       // unless its last round of tiles leaves more than about 30 % of the compute units' slots empty.
       const int64_t t = tiles(256, 256), rounds = ceil_div(t, cus);
-      if (10 * t >= 7 * rounds * cus) return launch_nvfp4_fast<OUT_BF16>(p, cus, stream);
+      if (10 * t >= 7 * rounds * cus) return launch_nvfp4_fast<OUT_BF16, false>(p, cus, stream);
     }
   }
   if constexpr (!NVFP4) {
@@ -1454,6 +1505,19 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int6
     if (!dense && m_hint >= 256 * (int64_t)p.groups && tiles(256, 256) >= cus / 2 && (p.n & 255) == 0 && (p.k & 63) == 0 &&
         p.k >= 128 && (int64_t)p.k * 2 * 256 < (1ll << 31))
       return launch_grouped16_fast<BF16_MMA, OUT_BF16>(p, cus, stream);
+  }
+  if constexpr (NVFP4) {
+    // Grouped NVFP4 with room for whole 256-row tiles: those go to the 256x256 kernel (about 1.4 times as
+    // fast per flop), the ends of the groups to the 128x128 tile kernel.  The group sizes live on the
+    // device, so both kernels are always launched; one that finds no work returns at once.
+    if (!dense && (p.n & 255) == 0 && (p.k & 127) == 0 && p.k >= 256 && m_hint >= 2048) {
+      const int rc = launch_nvfp4_fast<OUT_BF16, true>(p, cus, stream);
+      if (rc != NVF_OK) return rc;
+      Params rest = p;
+      rest.skip_whole_256 = 1;
+      const int64_t upper = 2 * (int64_t)p.groups * ceil_div(p.n, 128), cap = 2 * (int64_t)cus;
+      return launch_nvfp4_tile<128, 128, OUT_BF16>(rest, (int)(upper < cap ? upper : cap), stream);
+    }
   }
   // grouped: the tile height follows the average group (a 256-row tile on a 77-row group is mostly padding)
   if (dense ? tiles(256, 256) >= cus : m_hint >= 512 * (int64_t)p.groups) {

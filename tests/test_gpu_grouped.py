@@ -186,6 +186,48 @@ def test_nvfp4_grouped_mm_empty_and_tiny_groups(dev):
     assert max_rel(out, ref) <= GEMM_MAX_REL
 
 
+@pytest.mark.parametrize("sizes,n,k", [([600, 0, 256, 255, 1, 1030, 512], 512, 384), ([300, 2100, 0, 257], 256, 256),
+                                       ([2560, 700, 3000, 0, 1280, 2900], 2048, 256), ([511] * 5, 512, 640)])
+def test_nvfp4_grouped_mm_whole_tiles_and_group_ends(dev, sizes, n, k):
+    """At least 2048 rows, N % 256 == 0, K % 128 == 0: the whole 256-row tiles of every group run on the
+    persistent 256x256 kernel and the group ends on the 128x128 tile kernel.  Groups with no whole tile,
+    only whole tiles, one row past a tile, empty groups; two, three and five spans per tile; the third case
+    has 320 whole tiles, i.e. two per workgroup for some.  Every output element is compared; rows after the
+    last group stay untouched."""
+    from fuser_amd import nvf_cutlass
+
+    g, m = len(sizes), sum(sizes) + 33
+    gen = torch.Generator().manual_seed(n + k)
+    x = torch.randn(m, k, generator=gen).bfloat16()
+    w = (torch.randn(g, n, k, generator=gen) * 0.05).bfloat16()
+    ps, eo, st, ct = _grouped_args(sizes, n, k, dev)
+    so = start_offsets([O.round_up(t, 128) for t in sizes])
+    aq, asf = O.grouped_block_quantize_nvfp4(x, eo, so, None)
+    asf[asf == 0] = 0x7F  # poison: padding rows of the scale slabs must not reach any output
+    valid = O.grouped_block_quantize_nvfp4(x, eo, so, None)[1]
+    lin = torch.zeros_like(asf, dtype=torch.bool)
+    for e, t in enumerate(sizes):
+        if t:
+            ones = O.linear_to_swizzled_128_4(torch.ones(t, k // 16, dtype=torch.uint8))
+            lin[int(so[e]) : int(so[e]) + ones.shape[0]] |= ones.bool()
+    asf = torch.where(lin, valid, torch.full_like(valid, 0x7F))
+    bq = torch.empty(g, n, k // 2, dtype=torch.uint8)
+    bsf = torch.empty(g, n, k // 16, dtype=torch.uint8)
+    alphas = torch.empty(g)
+    for e in range(g):
+        gs = gs_of(w[e])
+        bq[e], bsf[e] = O.block_quantize_nvfp4(w[e], gs, True)
+        alphas[e] = (e + 1) / gs  # a different alpha for every group
+    ref = O.ref_nvfp4_scaled_grouped_mm(aq, bq, valid, bsf, alphas, ps, eo, so)
+    rows = sum(sizes)
+    for dtype in (torch.bfloat16, torch.float16):
+        out = nvf_cutlass.nvfp4_scaled_grouped_mm(fp4(aq.to(dev)), fp4(bq.to(dev)), e4m3(asf.to(dev)), e4m3(bsf.to(dev)), alphas.to(dev),
+                                                  st, ct, ps.to(dev), eo.to(dev), so.to(dev), dtype)
+        torch.cuda.synchronize()
+        scale = ref[:rows].abs().amax(dim=1, keepdim=True).clamp(min=1e-30)
+        assert ((out[:rows].float().cpu() - ref[:rows]).abs() / scale).max().item() <= GEMM_MAX_REL, (sizes, dtype)
+
+
 def _zipf_sizes(tokens, topk, experts, s, seed):
     gen = torch.Generator().manual_seed(seed)
     p = 1.0 / torch.arange(1, experts + 1).float() ** s
