@@ -815,13 +815,20 @@ int launch_nvfp4_fast(const Params& p, int cus, hipStream_t stream) {
 //   * A workgroup owns 16*RT weight rows for the whole of K and all M activation rows; its 8
 //     wavefronts split K in interleaved 128-element chunks and their partial sums are added in a fixed
 //     order through LDS (no atomics, no workspace, deterministic).
-//   * In v_mfma_f32_16x16x32_f16 lane (i, g) supplies 8 elements of row i,
-//     and both operands use the same (lane group, element) -> k assignment, so a lane loads the 16
-//     payload bytes [32g, 32g+32) of its row's chunk, converts them to fp16 in registers and feeds MFMA
-//     t = 0..3 with elements 8t..8t+7.  Weight rows are the first operand (output rows), activation rows
-//     the second, so a lane ends up with 4 consecutive N-elements of one output row.
+//   * In v_mfma_f32_16x16x32_f16 lane (i, g) supplies 8 elements of row i, and both operands use the same
+//     (lane group, element) -> k assignment, so a lane holds the 16 payload bytes [32g, 32g+32) of its
+//     row's chunk, converts them to fp16 in registers and feeds MFMA t = 0..3 with elements 8t..8t+7.
+//     Weight rows are the first operand (output rows), activation rows the second, so a lane ends up
+//     with 4 consecutive N-elements of one output row.
+//   * A load in that lane order (lane = row % 16 + 16 * piece) touches 64 unrelated 16-byte pieces and
+//     occupies the address unit for 64 cycles, which - not HBM, not latency - bounded an earlier version
+//     that loaded straight into registers.  The tiles are therefore fetched with LDS-direct loads in
+//     memory order (4 neighbouring lanes = 64 contiguous bytes of a row; scales as the 256 contiguous
+//     bytes that hold a 16-row tile's scale words) into a private LDS ring of each wavefront and read
+//     back in MFMA order; no barrier is involved because a wavefront only reads what it loaded itself.
+//   LDS per slot: NT payload tiles of 16 rows x 64 B, piece p of row r at piece position p ^ ((r >> 2) & 3)
+//   (conflict-free reads), then per operand one 1 KiB scale block per pair of tiles: [tile][col tile][row][16 B].
 // -------------------------------------------------------------------------------------------------
-
 // LDS-direct load.  lds_byte_addr and base are wave-uniform; lane L's 16 bytes land at lds_byte_addr + 16 * L.
 // Issued from inline assembly: the compiler neither waits for it nor orders LDS reads against it, the
 // kernels do that with explicit s_waitcnt vmcnt(n).
@@ -845,118 +852,16 @@ __device__ __forceinline__ void dequant_frags(const u32x4 q, uint32_t s2, u32x4 
   }
 }
 
-template <int RT, int TT, bool OUT_BF16>
-__global__ __launch_bounds__(512) void nvfp4_skinny_kernel(const Params p) {
-  constexpr int W = 8;  // wavefronts
-  extern __shared__ f32x4 red[];  // [W][tt_count][64 lanes], reused for each of the RT row tiles
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int r = lane & 15, g = lane >> 4;
-  const int n0 = blockIdx.x * (16 * RT);
-  const int tt_count = (p.m + 15) >> 4;  // 16-row activation tiles, at most TT
-  const int kbytes = p.k >> 1;
-  const int chunks = p.k >> 7;
-  const int sf_padded = p.k >> 4;  // K % 128 == 0: no padding columns
-  // chunk c, lane group g: payload bytes [64c + 16g, +16), scale blocks 8c + 2g, 8c + 2g + 1
-  const int sf_lane_off = (g >> 1) * 512 + (g & 1) * 2;
-
-  const uint8_t* b_row[RT];
-  const uint8_t* b_sf[RT];
-#pragma unroll
-  for (int rt = 0; rt < RT; ++rt) {
-    b_row[rt] = p.b + (int64_t)(n0 + rt * 16 + r) * kbytes + g * 16;
-    b_sf[rt] = p.sfb + swizzle_128x4(n0 + rt * 16 + r, 0, sf_padded) + sf_lane_off;
-  }
-  f32x4 acc[RT][TT];
-#pragma unroll
-  for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-    for (int tt = 0; tt < TT; ++tt) acc[rt][tt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-
-  for (int c = wave; c < chunks; c += W) {
-    u32x4 bq[RT];
-    uint32_t bs[RT];
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt) {
-      bq[rt] = *reinterpret_cast<const u32x4*>(b_row[rt] + (int64_t)c * 64);
-      bs[rt] = *reinterpret_cast<const uint16_t*>(b_sf[rt] + (int64_t)c * 1024);
-    }
-    // activation tiles: the loads of tile tt+1 are in flight while tile tt is converted and multiplied
-    auto load_a = [&](int tt, u32x4& q, uint32_t& sc) {
-      const int tok = min(tt * 16 + r, p.m - 1);  // rows past M repeat the last one; they are not stored
-      q = *reinterpret_cast<const u32x4*>(p.a + (int64_t)tok * kbytes + g * 16 + (int64_t)c * 64);
-      sc = *reinterpret_cast<const uint16_t*>(p.sfa + swizzle_128x4(tok, 0, sf_padded) + sf_lane_off + (int64_t)c * 1024);
-    };
-    u32x4 aq_next;
-    uint32_t as_next;
-    load_a(0, aq_next, as_next);
-    u32x4 fb[RT][4];
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt) dequant_frags(bq[rt], bs[rt], fb[rt]);
-#pragma unroll
-    for (int tt = 0; tt < TT; ++tt) {
-      if (tt < tt_count) {
-        const u32x4 aq = aq_next;
-        const uint32_t as = as_next;
-        if (tt + 1 < TT && tt + 1 < tt_count) load_a(tt + 1, aq_next, as_next);
-        u32x4 fa[4];
-        dequant_frags(aq, as, fa);
-#pragma unroll
-        for (int t = 0; t < 4; ++t)
-#pragma unroll
-          for (int rt = 0; rt < RT; ++rt)
-            acc[rt][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, fb[rt][t]),
-                                                                 __builtin_bit_cast(f16x8, fa[t]), acc[rt][tt], 0, 0, 0);
-      }
-    }
-  }
-
-  // ---- per row tile: sum the wavefronts' partial tiles in wave order and store
-  const float alpha = p.alpha[0];
-  uint16_t* out = static_cast<uint16_t*>(p.out);
-  const int units = tt_count * 64;
-#pragma unroll
-  for (int rt = 0; rt < RT; ++rt) {
-    if (rt > 0) __syncthreads();
-#pragma unroll
-    for (int tt = 0; tt < TT; ++tt)
-      if (tt < tt_count) red[(wave * tt_count + tt) * 64 + lane] = acc[rt][tt];
-    __syncthreads();
-    for (int u = tid; u < units; u += 512) {
-      const int l = u & 63, tt = u >> 6;
-      f32x4 s = red[u];
-#pragma unroll
-      for (int w = 1; w < W; ++w) s += red[w * units + u];
-      // element e of lane l: weight row 4*(l/16) + e (output column), activation row l%16 (output row)
-      const int tok = tt * 16 + (l & 15);
-      if (tok < p.m) {
-        u32x2 v;
-        v[0] = pack2(s[0] * alpha, s[1] * alpha, OUT_BF16);
-        v[1] = pack2(s[2] * alpha, s[3] * alpha, OUT_BF16);
-        *reinterpret_cast<u32x2*>(out + (int64_t)tok * p.n + n0 + rt * 16 + 4 * (l >> 4)) = v;
-      }
-    }
-  }
-}
-
-// Variant for few activation rows (M <= 64).  A load in MFMA lane order (lane = row % 16 + 16 * piece)
-// touches 64 unrelated 16-byte pieces and occupies the address unit for 64 cycles, which - not HBM, not
-// latency - bounds the plain kernel above.  Here the tiles are fetched with LDS-direct loads in memory
-// order (4 neighbouring lanes = 64 contiguous bytes of a row; scales as the 256 contiguous bytes that
-// hold a 16-row tile's scale words) into a private LDS ring of each wavefront and read back in MFMA
-// order; no barrier is involved because a wavefront only reads what it loaded itself.
-//   LDS per slot: NT payload tiles of 16 rows x 64 B, piece p of row r at piece position p ^ ((r >> 2) & 3)
-//   (conflict-free reads), then per operand one 1 KiB scale block per pair of tiles: [tile][col tile][row][16 B].
-template <int RT, int TT, bool OUT_BF16>
+template <int RT, int TT, bool OUT_BF16, int DEPTH>
 __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) {
   constexpr int W = 8;
   constexpr int NT = RT + TT;
   constexpr int B_SC = (RT + 1) / 2, A_SC = (TT + 1) / 2;     // scale blocks (1 KiB) per operand
   constexpr int SLOT_BYTES = (NT + B_SC + A_SC) * 1024;
   constexpr int NDMA = NT + B_SC + A_SC;                      // loads per chunk and wavefront
-  constexpr int DEPTH = 2;
-  static_assert(DEPTH == 2 && W * DEPTH * SLOT_BYTES <= 160 * 1024 && DEPTH * NDMA <= 63, "ring does not fit");
+  // DEPTH 2: two chunks in flight per wavefront.  DEPTH 1 (many tiles per chunk): the next chunk is requested
+  // as soon as the current one has been read out of LDS, and lands under its long conversion + MFMA phase.
+  static_assert((DEPTH == 1 || DEPTH == 2) && W * DEPTH * SLOT_BYTES <= 160 * 1024 && DEPTH * NDMA <= 63, "ring does not fit");
   extern __shared__ f32x4 red[];  // ring during the K loop, then [W][tiles][64 lanes] partial sums
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -1031,30 +936,48 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
   int slot = 0;
   for (int c = wave; c < chunks; c += W) {
     // the oldest chunk in flight has landed when only the loads of the next one (if there is one) are pending
-    if (c + W < chunks)
+    if (DEPTH == 2 && c + W < chunks)
       asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NDMA) : "memory");
     else
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     const char* sp = reinterpret_cast<const char*>(red) + (wave * DEPTH + slot) * SLOT_BYTES;
-    u32x4 q[NT];
-    uint32_t sc[NT];
+    // the activation tiles are read out of LDS together with the weight tiles (few of them) or one at a time
+    // right before their conversion (many: their registers would not fit)
+    constexpr bool kLazyA = TT > 2;
+    constexpr int NQ = kLazyA ? RT : NT;
+    u32x4 q[NQ];
+    uint32_t sc[NQ];
 #pragma unroll
-    for (int t = 0; t < NT; ++t) q[t] = *reinterpret_cast<const u32x4*>(sp + t * 1024 + rd_payload);
+    for (int t = 0; t < NQ; ++t) q[t] = *reinterpret_cast<const u32x4*>(sp + t * 1024 + rd_payload);
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) sc[rt] = *reinterpret_cast<const uint32_t*>(sp + rd_bsc[rt]) >> sc_shift;
+    if constexpr (!kLazyA) {
 #pragma unroll
-    for (int tt = 0; tt < TT; ++tt) sc[RT + tt] = *reinterpret_cast<const uint32_t*>(sp + rd_asc[tt]) >> sc_shift;
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // read out: the slot may be refilled
-    issue_chunk(c + DEPTH * W, slot);
-    slot ^= 1;
+      for (int tt = 0; tt < TT; ++tt) sc[RT + tt] = *reinterpret_cast<const uint32_t*>(sp + rd_asc[tt]) >> sc_shift;
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // read out: the slot may be refilled
+      issue_chunk(c + DEPTH * W, slot);
+    }
     u32x4 fb[RT][4];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) dequant_frags(q[rt], sc[rt], fb[rt]);
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) {
       if (tt < tt_count) {
+        u32x4 aq;
+        uint32_t as;
+        if constexpr (kLazyA) {
+          aq = *reinterpret_cast<const u32x4*>(sp + (RT + tt) * 1024 + rd_payload);
+          as = *reinterpret_cast<const uint32_t*>(sp + rd_asc[tt]) >> sc_shift;
+          if (tt + 1 == tt_count) {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the last read of the slot is complete
+            issue_chunk(c + DEPTH * W, slot);
+          }
+        } else {
+          aq = q[kLazyA ? 0 : RT + tt];
+          as = sc[kLazyA ? 0 : RT + tt];
+        }
         u32x4 fa[4];
-        dequant_frags(q[RT + tt], sc[RT + tt], fa);
+        dequant_frags(aq, as, fa);
 #pragma unroll
         for (int t = 0; t < 4; ++t)
 #pragma unroll
@@ -1063,41 +986,55 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
                                                                  __builtin_bit_cast(f16x8, fa[t]), acc[rt][tt], 0, 0, 0);
       }
     }
+    if constexpr (DEPTH == 2) slot ^= 1;
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no LDS-direct load may be pending when the ring is reused
   __syncthreads();
 
-  // ---- all partial tiles in one round (RT * TT <= 8): sum in wave order and store
+  // ---- sum the wavefronts' partial tiles in wave order and store: all tiles in one round if they fit the
+  // ring's memory (RT * TT <= 8), else one round per weight-row tile
   const float alpha = p.alpha[0];
   uint16_t* out = static_cast<uint16_t*>(p.out);
-  const int tiles = RT * tt_count;  // tile index: rt * tt_count + tt
+  constexpr int ROUNDS = RT * TT <= 8 ? 1 : RT;
+  constexpr int RPR = RT / ROUNDS;  // weight-row tiles per round
+  const int tiles = RPR * tt_count;   // tile index inside a round: rt * tt_count + tt
   const int units = tiles * 64;
 #pragma unroll
-  for (int rt = 0; rt < RT; ++rt)
+  for (int round = 0; round < ROUNDS; ++round) {
+    if (round > 0) __syncthreads();
 #pragma unroll
-    for (int tt = 0; tt < TT; ++tt)
-      if (tt < tt_count) red[(wave * tiles + rt * tt_count + tt) * 64 + lane] = acc[rt][tt];
-  __syncthreads();
-  for (int u = tid; u < units; u += 512) {
-    const int l = u & 63, tile = u >> 6;
-    const int rt = tile / tt_count, tt = tile - rt * tt_count;
-    f32x4 s = red[u];
+    for (int r2 = 0; r2 < RPR; ++r2)
 #pragma unroll
-    for (int w = 1; w < W; ++w) s += red[w * units + u];
-    const int tok = tt * 16 + (l & 15);
-    if (tok < p.m) {
-      u32x2 v;
-      v[0] = pack2(s[0] * alpha, s[1] * alpha, OUT_BF16);
-      v[1] = pack2(s[2] * alpha, s[3] * alpha, OUT_BF16);
-      *reinterpret_cast<u32x2*>(out + (int64_t)tok * p.n + n0 + rt * 16 + 4 * (l >> 4)) = v;
+      for (int tt = 0; tt < TT; ++tt)
+        if (tt < tt_count) red[(wave * tiles + r2 * tt_count + tt) * 64 + lane] = acc[round * RPR + r2][tt];
+    __syncthreads();
+    for (int u = tid; u < units; u += 512) {
+      const int l = u & 63, tile = u >> 6;
+      const int r2 = tile / tt_count, tt = tile - r2 * tt_count;
+      f32x4 s = red[u];
+#pragma unroll
+      for (int w = 1; w < W; ++w) s += red[w * units + u];
+      const int tok = tt * 16 + (l & 15);
+      if (tok < p.m) {
+        u32x2 v;
+        v[0] = pack2(s[0] * alpha, s[1] * alpha, OUT_BF16);
+        v[1] = pack2(s[2] * alpha, s[3] * alpha, OUT_BF16);
+        *reinterpret_cast<u32x2*>(out + (int64_t)tok * p.n + n0 + (round * RPR + r2) * 16 + 4 * (l >> 4)) = v;
+      }
     }
   }
 }
 
 template <int RT, int TT, bool OUT_BF16>
 int launch_nvfp4_skinny_ring_cfg(const Params& p, hipStream_t stream) {
-  auto kern = nvfp4_skinny_ring_kernel<RT, TT, OUT_BF16>;
-  constexpr int lds_bytes = 8 * 2 * (RT + TT + (RT + 1) / 2 + (TT + 1) / 2) * 1024;  // >= the 8 * RT * TT KiB of the reduction
+  constexpr int SLOT_KIB = RT + TT + (RT + 1) / 2 + (TT + 1) / 2;
+  constexpr int DEPTH = 8 * 2 * SLOT_KIB <= 160 ? 2 : 1;
+  auto kern = nvfp4_skinny_ring_kernel<RT, TT, OUT_BF16, DEPTH>;
+  // the ring; the reduction reuses it and needs 8 KiB per partial tile of a round
+  constexpr int red_kib = 8 * (RT * TT <= 8 ? RT * TT : TT);
+  constexpr int ring_kib = 8 * DEPTH * SLOT_KIB;
+  constexpr int lds_bytes = (ring_kib > red_kib ? ring_kib : red_kib) * 1024;
+  static_assert(lds_bytes <= 160 * 1024, "LDS");
   static bool configured = false;
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
@@ -1108,42 +1045,14 @@ int launch_nvfp4_skinny_ring_cfg(const Params& p, hipStream_t stream) {
   return check_launch("nvfp4_skinny_ring_kernel");
 }
 
-template <int RT, int TT, bool OUT_BF16>
-int launch_nvfp4_skinny_cfg(const Params& p, hipStream_t stream) {
-  auto kern = nvfp4_skinny_kernel<RT, TT, OUT_BF16>;
-  const int tt_count = (p.m + 15) >> 4;
-  const int lds_bytes = 8 * tt_count * 64 * 16;  // one set of partial tiles per wavefront: at most 64 KiB
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 8 * TT * 64 * 16);
-    if (e != hipSuccess) return fail(NVF_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    configured = true;
-  }
-  hipLaunchKernelGGL(kern, dim3((unsigned)(p.n / (16 * RT))), dim3(512), lds_bytes, stream, p);
-  return check_launch("nvfp4_skinny_kernel");
-}
-
 template <int TT, bool OUT_BF16>
 int launch_nvfp4_skinny_tt(const Params& p, int cus, hipStream_t stream) {
   // The conversion work bounds this kernel, and every workgroup converts all activation rows it uses:
   // take as many weight rows per workgroup as still leaves about one workgroup per compute unit.
   const int64_t want = (int64_t)cus * 4 / 5;
-  const bool rt4 = (p.n & 63) == 0 && p.n / 64 >= want, rt2 = (p.n & 31) == 0 && p.n / 32 >= want;
-  // The ring variant wins wherever its LDS ring fits the tile counts, except that with four activation
-  // tiles it cannot take four weight-row tiles, which matter more (measured).
-  const bool ring_ok = (int64_t)p.k * 64 < (1ll << 31);  // 32-bit lane offsets
-  if constexpr (TT <= 2) {
-    if (ring_ok && rt4) return launch_nvfp4_skinny_ring_cfg<4, TT, OUT_BF16>(p, stream);
-  }
-  if constexpr (TT <= 4) {
-    if (ring_ok && !(TT == 4 && rt4)) {
-      if (rt2) return launch_nvfp4_skinny_ring_cfg<2, TT, OUT_BF16>(p, stream);
-      return launch_nvfp4_skinny_ring_cfg<1, TT, OUT_BF16>(p, stream);
-    }
-  }
-  if (rt4) return launch_nvfp4_skinny_cfg<4, TT, OUT_BF16>(p, stream);
-  if (rt2) return launch_nvfp4_skinny_cfg<2, TT, OUT_BF16>(p, stream);
-  return launch_nvfp4_skinny_cfg<1, TT, OUT_BF16>(p, stream);
+  if ((p.n & 63) == 0 && p.n / 64 >= want) return launch_nvfp4_skinny_ring_cfg<4, TT, OUT_BF16>(p, stream);
+  if ((p.n & 31) == 0 && p.n / 32 >= want) return launch_nvfp4_skinny_ring_cfg<2, TT, OUT_BF16>(p, stream);
+  return launch_nvfp4_skinny_ring_cfg<1, TT, OUT_BF16>(p, stream);
 }
 
 template <bool OUT_BF16>
@@ -1492,7 +1401,8 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int6
       if (splits > 1 && workspace_bytes >= (int64_t)splits * p.m * p.n * 4)
         return launch_nvfp4_splitk<OUT_BF16>(p, splits, static_cast<float*>(workspace), stream);
     }
-    if (dense && p.m <= 128 && (p.k & 127) == 0 && (p.n & 15) == 0) return launch_nvfp4_skinny<OUT_BF16>(p, cus, stream);
+    if (dense && p.m <= 128 && (p.k & 127) == 0 && (p.n & 15) == 0 && (int64_t)p.k * 64 < (1ll << 31))  // 32-bit lane offsets
+      return launch_nvfp4_skinny<OUT_BF16>(p, cus, stream);
     if (dense && (p.m & 255) == 0 && (p.n & 255) == 0 && (p.k & 127) == 0 && p.k >= 256) {
       // The 256x256 kernel is about 1.4 times as fast per tile-flop as the tile kernel below, so it wins
       // unless its last round of tiles leaves more than about 30 % of the compute units' slots empty.
