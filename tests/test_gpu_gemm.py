@@ -351,6 +351,33 @@ def test_nvfp4_gemm_persistent_kernel_every_scale_code_is_decoded_exactly(dev, s
     assert ((out.float().cpu() - ref).abs() / scale).max().item() <= 2.0 ** -7
 
 
+@pytest.mark.parametrize("shape", [(1, 16, 128), (7, 96, 256), (16, 48, 384), (17, 304, 1152), (32, 6560, 128), (33, 160, 2048),
+                                   (64, 4096, 512), (5, 6592, 1152), (20, 6560, 640), (50, 6560, 256), (16, 64, 8192),
+                                   (9, 288, 3200), (48, 144, 1024), (100, 96, 384), (128, 6560, 256), (200, 64, 1152),
+                                   (256, 160, 512), (129, 32, 128)])
+def test_mxfp8_gemm_decode_sized_activations(dev, shape):
+    """M <= 256 (in launches of 64 rows) with K % 128 == 0 and N % 16 == 0 takes the kernel that streams the weights once through
+    per-wavefront LDS rings into v_mfma_scale_f32_16x16x128_f8f6f4: 1 / 2 / 4 activation tiles, 1 / 2
+    weight-row tiles per workgroup (rings of 3, 2 and 1 slots), activation rows that do not fill a tile,
+    all four scale row groups, 1 to 8 chunks per wavefront (wavefronts without work, ring wrap), scales
+    spread over many octaves, poisoned scale padding, both output types, run-to-run determinism."""
+    m, n, k = shape
+    gen = torch.Generator().manual_seed(m * 31 + n)
+    a, sa = _mxfp8_operand(m, k, gen, 1.0)
+    b, sb = _mxfp8_operand(n, k, gen, 1.0)
+    ref = O.ref_mxfp8_scaled_mm(a, b, sa, sb, 0.75)
+    sa_p = sa.clone()  # NaN code in every scale byte of the padding rows / columns
+    sa_p[O.linear_to_swizzled_128_4(torch.ones(m, k // 32, dtype=torch.uint8)) == 0] = 0xFF
+    scale = ref.abs().amax(dim=1, keepdim=True).clamp(min=1e-30)
+    for dtype in (torch.bfloat16, torch.float16):
+        if dtype == torch.float16 and ref.abs().max() > 6e4:
+            continue
+        out = _run_mxfp8(a, b, sa_p, sb, 0.75, dtype, dev)
+        assert out.shape == (m, n)
+        assert ((out.float().cpu() - ref).abs() / scale).max().item() <= GEMM_MAX_REL, (shape, dtype)
+        assert torch.equal(out, _run_mxfp8(a, b, sa_p, sb, 0.75, dtype, dev))
+
+
 @pytest.mark.parametrize("shape", [(4096, 2048, 512), (2560, 3328, 384), (2048, 4096, 256), (8192, 1024, 1152),
                                    (4096, 8192, 256), (8192, 4096, 384), (4352, 4096, 640)])
 def test_mxfp8_gemm_persistent_256_tile_kernel_full_compare(dev, shape):
