@@ -41,16 +41,17 @@ __device__ __forceinline__ uint32_t pack2(float a, float b, bool out_bf16) {
   return __builtin_bit_cast(uint32_t, v);
 }
 
-__device__ __forceinline__ int lds_pos(int row, int chunk) { return row * 8 + (chunk ^ (row & 7)); }
+// LDS tile: rows of 128 bytes; 16-byte chunk c of row r sits at chunk position c ^ ((r >> 1) & 7): two rows fill
+// the 64 banks once, so the fragment reads (16 consecutive lanes = 16 consecutive rows, one chunk) are conflict-free
+__device__ __forceinline__ int lds_pos(int row, int chunk) { return row * 8 + (chunk ^ ((row >> 1) & 7)); }
 
 template <int BM, int BN, bool OUT_BF16>
 __global__ __launch_bounds__(256) void mxfp8_gemm_kernel(const Params p) {
   constexpr int BK = 128;  // bytes == elements
   constexpr int WTM = BM / 2, WTN = BN / 2;
   constexpr int TM = WTM / 32, TN = WTN / 32;
-  extern __shared__ u32x4 lds[];
-  u32x4* lds_a = lds;
-  u32x4* lds_b = lds + BM * 8;
+  extern __shared__ u32x4 lds[];  // two buffers of (A tile, B tile)
+  constexpr int BUF_UNITS = (BM + BN) * 8;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -122,9 +123,9 @@ __global__ __launch_bounds__(256) void mxfp8_gemm_kernel(const Params p) {
     }
   };
 
-  issue_loads(0);
-  for (int ks = 0; ks < nk; ++ks) {
-    __syncthreads();
+  auto store_lds = [&](int buf) {
+    u32x4* lds_a = lds + buf * BUF_UNITS;
+    u32x4* lds_b = lds_a + BM * 8;
 #pragma unroll
     for (int i = 0; i < A_CH; ++i) {
       const int c = tid + 256 * i;
@@ -135,11 +136,20 @@ __global__ __launch_bounds__(256) void mxfp8_gemm_kernel(const Params p) {
       const int c = tid + 256 * i;
       if (c < B_TOTAL) lds_b[lds_pos(c >> 3, c & 7)] = sb[i];
     }
+  };
+
+  // K loop: the loads of step ks+1 are in flight under the MFMAs of step ks, then stored into the other
+  // LDS buffer; one barrier per step
+  issue_loads(0);
+  store_lds(0);
+  __syncthreads();
+  for (int ks = 0; ks < nk; ++ks) {
+    const u32x4* lds_a = lds + (ks & 1) * BUF_UNITS;
+    const u32x4* lds_b = lds_a + BM * 8;
 #pragma unroll
     for (int i = 0; i < TM; ++i) sca[i] = sca_next[i];
 #pragma unroll
     for (int j = 0; j < TN; ++j) scb[j] = scb_next[j];
-    __syncthreads();
     if (ks + 1 < nk) issue_loads(ks + 1);
 
 #pragma unroll
@@ -171,6 +181,8 @@ __global__ __launch_bounds__(256) void mxfp8_gemm_kernel(const Params p) {
         }
       }
     }
+    if (ks + 1 < nk) store_lds((ks + 1) & 1);
+    __syncthreads();
   }
 
   const float alpha = p.alpha[0];
@@ -667,7 +679,7 @@ int launch_skinny(const Params& p0, hipStream_t stream) {
 template <int BM, int BN, bool OUT_BF16>
 int launch_cfg(const Params& p, hipStream_t stream) {
   auto kern = mxfp8_gemm_kernel<BM, BN, OUT_BF16>;
-  constexpr int lds_bytes = (BM + BN) * 128;
+  constexpr int lds_bytes = 2 * (BM + BN) * 128;
   static bool configured = false;
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
