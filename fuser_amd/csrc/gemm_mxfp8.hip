@@ -210,7 +210,7 @@ __global__ __launch_bounds__(256) void mxfp8_gemm_kernel(const Params p) {
 
 
 // -------------------------------------------------------------------------------------------------
-// Fast path: 256x256 tile, M % 256 == N % 256 == K % 128 == 0.
+// Fast path: 256x256 or 128x256 tile, M % 256 (128) == N % 256 == K % 128 == 0.
 //   * Tiles travel global -> LDS with 16-byte LDS-direct loads (no staging registers) into a double
 //     buffer.  They are issued from inline assembly so that the compiler does not serialise them
 //     against the LDS reads of the other buffer; completion is enforced by the explicit
@@ -230,11 +230,18 @@ __device__ __forceinline__ void lds_dma16(uint32_t lds_byte_addr, const uint8_t*
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_byte_addr), "v"(voff), "s"(base) : "memory");
 }
 
-template <bool OUT_BF16>
+// TM = 32-row accumulator tiles of a wavefront along M: 4 -> 256x256 workgroup tile, 2 -> 128x256 (for shapes
+// whose 256x256 tiles would leave compute units idle).  The statement order for TM = 4 is the one the 8192^3
+// measurements were made with.
+template <int TM, bool OUT_BF16>
 __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) {
-  constexpr int BM = 256, BN = 256;
-  constexpr int TILE_UNITS = 2048;            // 16-byte units per operand tile (256 rows x 8 chunks)
-  constexpr int BUF_UNITS = 2 * TILE_UNITS;   // A + B
+  constexpr int BM = 64 * TM, BN = 256;
+  constexpr int A_UNITS = BM * 8;             // 16-byte units of the A tile (BM rows x 8 chunks)
+  constexpr int TILE_UNITS = 2048;            // ... of the B tile
+  constexpr int BUF_UNITS = A_UNITS + TILE_UNITS;
+  constexpr int NM = 4 * TM;                  // MFMAs per half step
+  constexpr int NF = 2 * TM + 8;              // fragment reads (ds_read_b128) per half step
+  constexpr int ND = 2 * TM + 8;              // LDS-direct loads per wavefront and K step
   extern __shared__ u32x4 lds[];
 
   const int tid = threadIdx.x;
@@ -291,11 +298,11 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
     int m0, n0;
     tile_coords(t, m0, n0);
     TilePtrs r;
-    r.a = p.a + ((int64_t)m0 + wave * 64) * p.k;
+    r.a = p.a + ((int64_t)m0 + wave * (BM / 4)) * p.k;
     r.b = p.b + ((int64_t)n0 + wave * 64) * p.k;
     // one 16-byte scale load per lane per K step: rows {li, li+32, li+64, li+96} of the wave's 128-row
     // scale tile x 4 K-blocks
-    r.sa = p.sfa + ((int64_t)((m0 >> 7) + wm) * sf_tiles_k) * 512;
+    r.sa = p.sfa + ((int64_t)((m0 >> 7) + (TM == 4 ? wm : 0)) * sf_tiles_k) * 512;
     r.sb = p.sfb + ((int64_t)((n0 >> 7) + wn) * sf_tiles_k) * 512;
     return r;
   };
@@ -304,13 +311,15 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
   int l_ks = 0, l_count = 0;            // K step inside lp; steps issued so far
   const uint32_t sc_lane_off = (uint32_t)li * 16u;
   u32x4 sc_la, sc_lb;  // scales in flight (for step l_count - 1)
-  // Unit q (0..15) of a step's tile loads: operand q&1, rows (wave*8 + q/2)*8 .. +7.  Past the end of
-  // the stream the last tile is loaded again (into a buffer nobody reads any more).
+  // Unit q (0..ND-1) of a step's tile loads: 8 rows of one operand.  A and B alternate while A has rows left
+  // (operand q&1, rows (q/2)*8 .. +7 of the wavefront's share), then the rest of B.  Past the end of the
+  // stream the last tile is loaded again (into a buffer nobody reads any more).
   auto issue_step_unit = [&](int q) {
     const int buf = l_count & 1;
-    const int j = q >> 1;
-    const uint32_t l = lds_base + (uint32_t)(buf * BUF_UNITS + (q & 1) * TILE_UNITS + wave * 512) * 16u + j * 1024u;
-    const uint8_t* gp = ((q & 1) ? lp.b : lp.a) + ((int64_t)l_ks << 7);
+    const int op = q < 4 * TM ? (q & 1) : 1;
+    const int j = q < 4 * TM ? (q >> 1) : q - 2 * TM;
+    const uint32_t l = lds_base + (uint32_t)(buf * BUF_UNITS + (op ? A_UNITS + wave * 512 : wave * (BM * 2))) * 16u + j * 1024u;
+    const uint8_t* gp = (op ? lp.b : lp.a) + ((int64_t)l_ks << 7);
     lds_dma16(l, gp, ((j & 1) ? voff_odd : voff_even) + (uint32_t)j * step8);
   };
   // After the 16 units: the step's scale loads, then advance the stream (selects only).
@@ -325,13 +334,15 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
     lp.sa = wrap ? np.sa : lp.sa;
     lp.sb = wrap ? np.sb : lp.sb;
   };
-  // Fragment storage: [operand: 0 = A, 1 = B][sub-tile][half].  Unit q (0..15) of a half step is one
-  // ds_read_b128: operand q>>3, sub-tile (q>>1)&3, half q&1.
+  // Fragment storage: [operand: 0 = A, 1 = B][sub-tile][half].  Unit q (0..NF-1) of a half step is one
+  // ds_read_b128: the 2*TM units of A (sub-tile q/2, half q&1), then the 8 units of B.
   struct Frags { u32x4 h[2][4][2]; };
   auto load_unit = [&](int buf, int sub, int q, Frags& f) {
-    const int op = q >> 3, t = (q >> 1) & 3, half = q & 1;
-    const u32x4* base = lds + buf * BUF_UNITS + op * TILE_UNITS;
-    const int row = (op ? wn : wm) * 128 + t * 32 + li;
+    const int op = q >= 2 * TM ? 1 : 0;
+    const int u = op ? q - 2 * TM : q;
+    const int t = u >> 1, half = u & 1;
+    const u32x4* base = lds + buf * BUF_UNITS + op * A_UNITS;
+    const int row = (op ? wn * 128 : wm * (32 * TM)) + t * 32 + li;
     f.h[op][t][half] = base[lds_pos2(row, sub * 4 + lg + 2 * half)];
   };
   auto frag = [&](const Frags& f, int op, int t) {
@@ -339,10 +350,10 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
     return i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
   };
 
-  f32x16 acc[4][4];
+  f32x16 acc[TM][4];
   auto zero_acc = [&]() {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
       for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -356,8 +367,9 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
   do {                                                                                                         \
     asm volatile("" : "+a"(acc[0][0]), "+a"(acc[0][1]), "+a"(acc[0][2]), "+a"(acc[0][3]), "+a"(acc[1][0]),     \
                  "+a"(acc[1][1]), "+a"(acc[1][2]), "+a"(acc[1][3]));                                           \
-    asm volatile("" : "+a"(acc[2][0]), "+a"(acc[2][1]), "+a"(acc[2][2]), "+a"(acc[2][3]), "+a"(acc[3][0]),     \
-                 "+a"(acc[3][1]), "+a"(acc[3][2]), "+a"(acc[3][3]));                                           \
+    if constexpr (TM == 4)                                                                                     \
+      asm volatile("" : "+a"(acc[TM - 2][0]), "+a"(acc[TM - 2][1]), "+a"(acc[TM - 2][2]), "+a"(acc[TM - 2][3]), \
+                   "+a"(acc[TM - 1][0]), "+a"(acc[TM - 1][1]), "+a"(acc[TM - 1][2]), "+a"(acc[TM - 1][3]));     \
   } while (0)
 
   const float alpha = p.alpha[0];
@@ -372,19 +384,26 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
   const int tiles_ahead = nk == 2 ? 2 : 1;
   np = (first_tile + slots < range_end) ? tile_ptrs(first_tile + slots) : lp;
 #pragma unroll
-  for (int q = 0; q < 16; ++q) issue_step_unit(q);  // step 0
+  for (int q = 0; q < ND; ++q) issue_step_unit(q);  // step 0
   issue_step_tail();
   na = sc_la; nb = sc_lb;
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  // scale word of accumulator row tile i: rows {li + 32 c} of a 128-row scale tile are component c of the load;
+  // with 64 rows per wavefront (TM == 2) the wavefront's half of the tile is components 2 wm, 2 wm + 1
+  auto take_scales = [&]() {
 #pragma unroll
-  for (int i = 0; i < 4; ++i) { wa[i] = na[i] >> sh; wb[i] = nb[i] >> sh; }
+    for (int i = 0; i < TM; ++i) wa[i] = (TM == 4 ? na[i] : (wm ? na[2 + (i & 1)] : na[i & 1])) >> sh;
 #pragma unroll
-  for (int q = 0; q < 16; ++q) issue_step_unit(q);  // step 1
+    for (int j = 0; j < 4; ++j) wb[j] = nb[j] >> sh;
+  };
+  take_scales();
+#pragma unroll
+  for (int q = 0; q < ND; ++q) issue_step_unit(q);  // step 1
   issue_step_tail();
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
 #pragma unroll
-  for (int q = 0; q < 16; ++q) load_unit(0, 0, q, f0);
+  for (int q = 0; q < NF; ++q) load_unit(0, 0, q, f0);
 
   int g = 0;
   for (int c_tile = first_tile; c_tile < range_end; c_tile += slots) {
@@ -395,9 +414,10 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
       // ---- first half: MFMAs on f0, interleaved one-to-one with the LDS reads that fill f1
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int q = 0; q < 16; ++q) {
+      for (int q = 0; q < NM; ++q) {
         const int i = q >> 2, j = q & 3;
-        load_unit(buf, 1, q, f1);
+#pragma unroll
+        for (int u = q * NF / NM; u < (q + 1) * NF / NM; ++u) load_unit(buf, 1, u, f1);
         acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(frag(f0, 1, j), frag(f0, 0, i), acc[i][j], 0, 0, 0, (int)wb[j], 0, (int)wa[i]);
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -414,17 +434,18 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
       // after the last step they read stale data that is never used) and the loads of step g+2 into buf
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int q = 0; q < 16; ++q) {
+      for (int q = 0; q < NM; ++q) {
         const int i = q >> 2, j = q & 3;
-        load_unit(buf ^ 1, 0, q, f0);
-        issue_step_unit(q);
-        if (q == 15) issue_step_tail();  // scalar bookkeeping in the shadow of the MFMAs already queued
+#pragma unroll
+        for (int u = q * NF / NM; u < (q + 1) * NF / NM; ++u) load_unit(buf ^ 1, 0, u, f0);
+#pragma unroll
+        for (int u = q * ND / NM; u < (q + 1) * ND / NM; ++u) issue_step_unit(u);
+        if (q == NM - 1) issue_step_tail();  // scalar bookkeeping in the shadow of the MFMAs already queued
         acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(frag(f1, 1, j), frag(f1, 0, i), acc[i][j], 0, 0, 2, (int)wb[j], 2, (int)wa[i]);
         __builtin_amdgcn_sched_barrier(0);
       }
       NVF_PIN_ACC();
-#pragma unroll
-      for (int i = 0; i < 4; ++i) { wa[i] = na[i] >> sh; wb[i] = nb[i] >> sh; }
+      take_scales();
     }
     // ---- epilogue of this tile; the loads of the next tile's first two steps are already in flight.
     // acc[i][j][r] = C[m = li][n = (r/4)*8 + lg*4 + r%4] of its 32x32 sub-tile.
@@ -432,8 +453,8 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
     tile_coords(c_tile, m0, n0);
     uint16_t* out = static_cast<uint16_t*>(p.out);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      uint16_t* orow = out + (int64_t)(m0 + wm * 128 + i * 32 + li) * p.n + n0 + wn * 128 + lg * 4;
+    for (int i = 0; i < TM; ++i) {
+      uint16_t* orow = out + (int64_t)(m0 + wm * (32 * TM) + i * 32 + li) * p.n + n0 + wn * 128 + lg * 4;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
 #pragma unroll
@@ -451,17 +472,17 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
 #undef NVF_PIN_ACC
 }
 
-template <bool OUT_BF16>
+template <int TM, bool OUT_BF16>
 int launch_fast(const Params& p, hipStream_t stream) {
-  auto kern = mxfp8_gemm_256_kernel<OUT_BF16>;
-  constexpr int lds_bytes = 2 * 2 * 2048 * 16;  // 128 KiB
+  auto kern = mxfp8_gemm_256_kernel<TM, OUT_BF16>;
+  constexpr int lds_bytes = 2 * (64 * TM + 256) * 128;  // 128 KiB / 96 KiB
   static bool configured = false;
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     if (e != hipSuccess) return fail(NVF_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
     configured = true;
   }
-  const int64_t tiles = (int64_t)(p.m / 256) * (p.n / 256);
+  const int64_t tiles = (int64_t)(p.m / (64 * TM)) * (p.n / 256);
   const int cus = 256;
   const unsigned grid = (unsigned)(tiles >= cus ? cus : ((tiles + 7) / 8) * 8);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_bytes, stream, p);
@@ -698,8 +719,17 @@ int launch_sized(const Params& p, hipStream_t stream) {
   // the tile kernels below (measured: 128 x 4096 x 14336 in 35 instead of 117 us, 256 x 14336 x 4096 equal)
   if (p.m <= 256 && (p.k & 127) == 0 && (p.n & 15) == 0 && (int64_t)p.k * 64 < (1ll << 31))  // 32-bit lane offsets
     return launch_skinny<OUT_BF16>(p, stream);
-  if (tiles(256, 256) >= 128 && (p.k & 127) == 0 && p.k >= 256 && (p.m & 255) == 0 && (p.n & 255) == 0 && (int64_t)p.k * 256 < (1ll << 31))
-    return launch_fast<OUT_BF16>(p, stream);
+  if ((p.k & 127) == 0 && p.k >= 256 && (p.m & 127) == 0 && (p.n & 255) == 0 && (int64_t)p.k * 256 < (1ll << 31)) {
+    // Persistent LDS-direct kernel with 256x256 or 128x256 tiles: a 128-row tile costs about 0.61 of a 256-row
+    // tile (half the flops at 82 % of the rate, measured), and the time goes with the rounds of tiles over the
+    // compute units; below 48 tiles the tile kernels further down do as well.
+    const int64_t cus = 256;
+    const int64_t t256 = (p.m & 255) == 0 ? tiles(256, 256) : 0, t128 = tiles(128, 256);
+    const int64_t cost256 = t256 ? 100 * ceil_div(t256, cus) : INT64_MAX;
+    const int64_t cost128 = 61 * ceil_div(t128, cus);
+    if (t256 >= 128 && cost256 <= cost128) return launch_fast<4, OUT_BF16>(p, stream);
+    if (t128 >= 48) return launch_fast<2, OUT_BF16>(p, stream);
+  }
   if (tiles(256, 256) >= 256) return launch_cfg<256, 256, OUT_BF16>(p, stream);
   if (tiles(128, 128) >= 256) return launch_cfg<128, 128, OUT_BF16>(p, stream);
   return launch_cfg<64, 64, OUT_BF16>(p, stream);

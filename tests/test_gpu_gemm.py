@@ -380,13 +380,13 @@ def test_mxfp8_gemm_decode_sized_activations(dev, shape):
 
 
 @pytest.mark.parametrize("shape", [(4096, 2048, 512), (2560, 3328, 384), (2048, 4096, 256), (8192, 1024, 1152),
-                                   (4096, 8192, 256), (8192, 4096, 384), (4352, 4096, 640)])
+                                   (4096, 8192, 256), (8192, 4096, 384), (4352, 4096, 640), (1152, 2048, 384)])
 def test_mxfp8_gemm_persistent_256_tile_kernel_full_compare(dev, shape):
-    """Shapes with M % 256 == N % 256 == K % 128 == 0 and at least 128 tiles take the persistent
-    LDS-direct kernel; every output element is compared with the oracle.  (2560, 3328) has a tile grid
-    that is not a multiple of the 8 x 4 blocking; the 512- and 272-tile shapes give every workgroup two
-    (or one and two) tiles, so that the load stream wraps across tiles, with two, three and five K steps
-    or spans per tile."""
+    """Shapes with N % 256 == K % 128 == 0 and M % 128 == 0 take the persistent LDS-direct kernel with
+    256x256 tiles ((2560, 3328): a tile grid that is not a multiple of the 8 x 4 blocking; the two 512-tile
+    shapes: two tiles per workgroup, so that the load stream wraps across tiles) or with 128x256 tiles where
+    those fill the compute units better (the 128-tile shapes, 272 tiles, and M = 1152, which is no multiple
+    of 256); two, three, five and nine K steps per tile.  Every output element is compared with the oracle."""
     m, n, k = shape
     gen = torch.Generator().manual_seed(k)
     a, sa = _mxfp8_operand(m, k, gen, 1.0)
