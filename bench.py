@@ -179,6 +179,20 @@ def main():
                 res[f"M{m}_N{n}_K{k}"] = {"quant_us": round(ms_q * 1e3, 2), "gemm_us": round(ms_g * 1e3, 2), "seq_us": round(ms_s * 1e3, 2),
                                           "gemm_TFLOP/s": round(2.0 * m * n * k / ms_g / 1e9, 1), "gemm_GB/s": round(byts / ms_g / 1e6, 1)}
         extra["nvfp4_gemm_llm_shapes"] = res
+        # the same shapes through mxfp8_scaled_mm (not a BASELINE config: the decode / prefill use of the headline op)
+        one = torch.ones((), device=dev)
+        res8 = {}
+        for (n, k) in ((4096, 4096), (14336, 4096), (4096, 14336)):
+            w8, sw8 = ops.nv_block_quantize((torch.randn(n, k, device=dev, generator=gen) * 0.02).bfloat16(), None, True, 32,
+                                            torch.float8_e4m3fn)
+            for m in (16, 128, 2048):
+                x8, sx8 = ops.nv_block_quantize(torch.randn(m, k, device=dev, generator=gen).bfloat16(), None, True, 32,
+                                                torch.float8_e4m3fn)
+                ms_g, _ = timed(lambda: nvf_cutlass.mxfp8_scaled_mm(x8, w8, sx8, sw8, one, torch.bfloat16), 50, 5)
+                byts = n * k * 1.03125 + m * k * 1.03125 + 2 * m * n
+                res8[f"M{m}_N{n}_K{k}"] = {"gemm_us": round(ms_g * 1e3, 2), "gemm_TFLOP/s": round(2.0 * m * n * k / ms_g / 1e9, 1),
+                                           "gemm_GB/s": round(byts / ms_g / 1e6, 1)}
+        extra["mxfp8_gemm_llm_shapes"] = res8
 
     def run_grouped():
         g, k, n = 8, 4096, 14336
