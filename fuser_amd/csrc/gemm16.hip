@@ -520,11 +520,20 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
 // LDS: two buffers of (A tile + B tile), each tile 256 rows x 128 bytes with 16-byte chunk c of row r at
 // chunk position c ^ ((r >> 1) & 7): conflict-free for the fragment reads.
 // -------------------------------------------------------------------------------------------------
-template <bool OUT_BF16, bool GROUPED>
+// TM = 32-row accumulator tiles of a wavefront along M: 4 -> 256x256 workgroup tile, 2 -> 128x256 (dense shapes
+// whose 256x256 tiles would leave compute units idle; 1.5 times the conversion work per MFMA).  The statement
+// order for TM = 4 is the one the 8192^3 measurements were made with.
+template <bool OUT_BF16, bool GROUPED, int TM = 4>
 __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
-  constexpr int BM = 256, BN = 256;
-  constexpr int TILE_UNITS = 2048;           // 16-byte units per operand tile
-  constexpr int BUF_UNITS = 2 * TILE_UNITS;  // A + B
+  static_assert(TM == 4 || (TM == 2 && !GROUPED), "tile height");
+  constexpr int BM = 64 * TM, BN = 256;
+  constexpr int A_UNITS = BM * 8;            // 16-byte units of the A tile (fp16, 64 of K per row)
+  constexpr int TILE_UNITS = 2048;           // ... of the B tile
+  constexpr int BUF_UNITS = A_UNITS + TILE_UNITS;
+  constexpr int AR = TM / 2;                 // A rows a thread stages per span (rows srow + 128 i)
+  constexpr int NMK = 2 * TM;                // MFMAs per 16-deep sub-step
+  constexpr int NCU = 2 * AR + 4;            // conversion units per step: operand, row, half scale block
+  constexpr int NFU = TM + 2;                // fragment reads per sub-step
   extern __shared__ u32x4 lds[];
   __shared__ int tile_prefix[GROUPED ? kMaxGroups + 1 : 1];
 
@@ -634,11 +643,11 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   auto issue_load_unit = [&](Raw& r, int q) {
     const int64_t o = (int64_t)l_mac * 64, so = (int64_t)l_mac * 1024;
     if (q == 0) r.a[0] = *reinterpret_cast<const u32x4*>(lp.a + o);
-    if (q == 1) r.a[1] = *reinterpret_cast<const u32x4*>(lp.a + o + row128);
+    if (q == 1 && AR == 2) r.a[1] = *reinterpret_cast<const u32x4*>(lp.a + o + row128);
     if (q == 2) r.b[0] = *reinterpret_cast<const u32x4*>(lp.b + o);
     if (q == 3) r.b[1] = *reinterpret_cast<const u32x4*>(lp.b + o + row128);
     if (q == 4) r.sa[0] = *reinterpret_cast<const uint16_t*>(lp.sa + so);
-    if (q == 5) r.sa[1] = *reinterpret_cast<const uint16_t*>(lp.sa + so + sfrow128);
+    if (q == 5 && AR == 2) r.sa[1] = *reinterpret_cast<const uint16_t*>(lp.sa + so + sfrow128);
     if (q == 6) r.sb[0] = *reinterpret_cast<const uint16_t*>(lp.sb + so);
     if (q == 7) r.sb[1] = *reinterpret_cast<const uint16_t*>(lp.sb + so + sfrow128);
   };
@@ -651,8 +660,9 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
     lp.sb = wrap ? np.sb : lp.sb;
   };
 
-  // ---- conversion for a step of parity P: unit u (0..7) = operand u>>2, row (u>>1)&1, half block u&1.
-  // A unit is spread over three MFMA slots (about 3 VALU instructions each).
+  // ---- conversion for a step of parity P: unit u (0..7) = operand u>>2, row (u>>1)&1, half block u&1 (with 128
+  // rows of A, its second row does not exist: conversion unit v of the NCU real ones is unit v + 2 from v = 2 on).
+  // A unit is cut into three parts of about 3 VALU instructions each.
   auto scale_pair = [&](uint32_t s2, int b) {
     const float f = b ? __builtin_amdgcn_cvt_f32_fp8((int)s2, 1) : __builtin_amdgcn_cvt_f32_fp8((int)s2, 0);
     return __builtin_bit_cast(f16x2, __builtin_amdgcn_cvt_pkrtz(f, f));  // exact: e4m3 fits fp16
@@ -675,27 +685,27 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
     } else {
       ch[2] = ch[2] * sv[op][i];
       ch[3] = ch[3] * sv[op][i];
-      lds[wbuf * BUF_UNITS + op * TILE_UNITS + lds_pos2(srow + 128 * i, spiece * 2 + cc)] =
+      lds[wbuf * BUF_UNITS + op * A_UNITS + lds_pos2(srow + 128 * i, spiece * 2 + cc)] =
           u32x4{__builtin_bit_cast(uint32_t, ch[0]), __builtin_bit_cast(uint32_t, ch[1]), __builtin_bit_cast(uint32_t, ch[2]),
                 __builtin_bit_cast(uint32_t, ch[3])};
     }
   };
 
   // ---- MFMA fragments of one 16-deep sub-step, loaded in the order of their first use by the MFMA
-  // sequence (a0 b0) (a0 b1) (a1 b0) ...: units 0..5 = a0, b0, b1, a1, a2, a3
+  // sequence (a0 b0) (a0 b1) (a1 b0) ...: units 0..NFU-1 = a0, b0, b1, a1, a2, a3
   struct Frag { u32x4 a[4], b[2]; };
   auto load_frag_unit = [&](int buf, int kk, int q, Frag& f) {
     const int op = (q == 1 || q == 2) ? 1 : 0;
     const int t = op ? q - 1 : (q == 0 ? 0 : q - 2);
-    const int row = (op ? wn * 64 : wm * 128) + t * 32 + li;
-    const u32x4 v = lds[buf * BUF_UNITS + op * TILE_UNITS + lds_pos2(row, kk * 2 + lg)];
+    const int row = (op ? wn * 64 : wm * (32 * TM)) + t * 32 + li;
+    const u32x4 v = lds[buf * BUF_UNITS + op * A_UNITS + lds_pos2(row, kk * 2 + lg)];
     if (op) f.b[t] = v; else f.a[t] = v;
   };
 
-  f32x16 acc[4][2];
+  f32x16 acc[TM][2];
   auto zero_acc = [&]() {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
       for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -706,8 +716,10 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   // Keeps the accumulator tiles "used" at this point of the program, so that the MFMAs producing them
   // cannot be moved past the statement that follows (they have no side effects of their own).
 #define NVF_PIN_ACC()                                                                                        \
-  asm volatile("" : "+a"(acc[0][0]), "+a"(acc[0][1]), "+a"(acc[1][0]), "+a"(acc[1][1]), "+a"(acc[2][0]),     \
-               "+a"(acc[2][1]), "+a"(acc[3][0]), "+a"(acc[3][1]))
+  do {                                                                                                       \
+    asm volatile("" : "+a"(acc[0][0]), "+a"(acc[0][1]), "+a"(acc[1][0]), "+a"(acc[1][1]));                   \
+    if constexpr (TM == 4) asm volatile("" : "+a"(acc[TM - 2][0]), "+a"(acc[TM - 2][1]), "+a"(acc[TM - 1][0]), "+a"(acc[TM - 1][1])); \
+  } while (0)
 
   Raw cur, nxt;  // span whose odd step is converted next / span whose even step is converted next
   Frag fr[2];
@@ -724,15 +736,16 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
 #pragma unroll
   for (int q = 0; q < 8; ++q) issue_load_unit(nxt, q);
   advance_stream();
+  auto unit_of = [&](int v) { return (AR == 2 || v < 2) ? v : v + 2; };  // conversion unit v -> (operand, row, half) code
 #pragma unroll
-  for (int u = 0; u < 8; ++u)
+  for (int v = 0; v < NCU; ++v)
 #pragma unroll
-    for (int ph = 0; ph < 3; ++ph) convert_phase(cur, 0, u, ph, 0);
+    for (int ph = 0; ph < 3; ++ph) convert_phase(cur, 0, unit_of(v), ph, 0);
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
 #pragma unroll
-  for (int q = 0; q < 6; ++q) load_frag_unit(0, 0, q, fr[0]);
+  for (int q = 0; q < NFU; ++q) load_frag_unit(0, 0, q, fr[0]);
 
   for (int c_tile = first_tile; c_tile < range_end; c_tile += slots) {
     np = ptrs_or_current(c_tile + tiles_ahead * slots);
@@ -754,14 +767,19 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
           }
           __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-          for (int q = 0; q < 8; ++q) {
+          for (int q = 0; q < NMK; ++q) {
             const int i = q >> 1, j = q & 1;
-            const int slot_id = kk * 8 + q;
-            if (q < 6) load_frag_unit(kk < 3 ? h : (h ^ 1), (kk + 1) & 3, q, fr[(kk + 1) & 1]);
-            if (kk < 3) convert_phase(h ? nxt : cur, h ^ 1, slot_id / 3, slot_id % 3, h ^ 1);
+            const int slot_id = kk * NMK + q;  // 3 * NMK slots for the 3 * NCU conversion parts of the step
+            if (q < NFU) load_frag_unit(kk < 3 ? h : (h ^ 1), (kk + 1) & 3, q, fr[(kk + 1) & 1]);
+            if (kk < 3) {
+#pragma unroll
+              for (int part = slot_id * NCU / NMK; part < (slot_id + 1) * NCU / NMK; ++part)
+                convert_phase(h ? nxt : cur, h ^ 1, unit_of(part / 3), part % 3, h ^ 1);
+            }
             if (kk == 3 && h == 1) {
-              issue_load_unit(nxt, q);
-              if (q == 7) advance_stream();
+#pragma unroll
+              for (int l = q * 8 / NMK; l < (q + 1) * 8 / NMK; ++l) issue_load_unit(nxt, l);
+              if (q == NMK - 1) advance_stream();
             }
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, fr[kk & 1].b[j]),
                                                                __builtin_bit_cast(f16x8, fr[kk & 1].a[i]), acc[i][j], 0, 0, 0);
@@ -776,8 +794,8 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
     const float alpha = p.alpha[cw.g];
     uint16_t* out = static_cast<uint16_t*>(p.out);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      uint16_t* orow = out + (cw.m0 + wm * 128 + i * 32 + li) * p.n + cw.n0 + wn * 64 + lg * 4;
+    for (int i = 0; i < TM; ++i) {
+      uint16_t* orow = out + (cw.m0 + wm * (32 * TM) + i * 32 + li) * p.n + cw.n0 + wn * 64 + lg * 4;
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
 #pragma unroll
@@ -794,17 +812,17 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
 #undef NVF_PIN_ACC
 }
 
-template <bool OUT_BF16, bool GROUPED>
+template <bool OUT_BF16, bool GROUPED, int TM = 4>
 int launch_nvfp4_fast(const Params& p, int cus, hipStream_t stream) {
-  auto kern = nvfp4_gemm_256_kernel<OUT_BF16, GROUPED>;
-  constexpr int lds_bytes = 2 * 2 * 2048 * 16;  // 128 KiB
+  auto kern = nvfp4_gemm_256_kernel<OUT_BF16, GROUPED, TM>;
+  constexpr int lds_bytes = 2 * (64 * TM + 256) * 128;  // 128 KiB / 96 KiB
   static bool configured = false;
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     if (e != hipSuccess) return fail(NVF_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
     configured = true;
   }
-  const int64_t tiles = (int64_t)(p.m / 256) * (p.n / 256);  // grouped: an upper bound
+  const int64_t tiles = (int64_t)(p.m / (64 * TM)) * (p.n / 256);  // grouped: an upper bound
   const unsigned grid = (unsigned)(tiles >= cus ? (cus & ~7) : ((tiles + 7) / 8) * 8);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds_bytes, stream, p);
   return check_launch("nvfp4_gemm_256_kernel");
@@ -1417,11 +1435,16 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int6
     // 46 instead of 65 us; at 512 rows the tile kernel wins)
     if (dense && p.m <= 256 && (p.k & 127) == 0 && (p.n & 15) == 0 && (int64_t)p.k * 64 < (1ll << 31))  // 32-bit lane offsets
       return launch_nvfp4_skinny<OUT_BF16>(p, cus, stream);
-    if (dense && (p.m & 255) == 0 && (p.n & 255) == 0 && (p.k & 127) == 0 && p.k >= 256) {
-      // The 256x256 kernel is about 1.4 times as fast per tile-flop as the tile kernel below, so it wins
-      // unless its last round of tiles leaves more than about 30 % of the compute units' slots empty.
-      const int64_t t = tiles(256, 256), rounds = ceil_div(t, cus);
-      if (10 * t >= 7 * rounds * cus) return launch_nvfp4_fast<OUT_BF16, false>(p, cus, stream);
+    if (dense && (p.m & 127) == 0 && (p.n & 255) == 0 && (p.k & 127) == 0 && p.k >= 256) {
+      // Persistent kernel with 256x256 or 128x256 tiles, or the tile kernel below?  Costs in units of one round
+      // of 256x256 tiles over the compute units = 100: a 128-row tile costs 62 (half the flops at 81 % of the
+      // rate), and the tile kernel, which has no rounds to speak of, runs at about 70 % of the rate (all measured).
+      const int64_t t256 = (p.m & 255) == 0 ? tiles(256, 256) : 0, t128 = tiles(128, 256);
+      const int64_t cost256 = t256 ? 100 * ceil_div(t256, cus) : INT64_MAX;
+      const int64_t cost128 = 62 * ceil_div(t128, cus);
+      const int64_t cost_tile = 144 * t128 / (2 * cus);
+      if (cost256 <= cost128 && cost256 <= cost_tile) return launch_nvfp4_fast<OUT_BF16, false, 4>(p, cus, stream);
+      if (cost128 <= cost_tile) return launch_nvfp4_fast<OUT_BF16, false, 2>(p, cus, stream);
     }
   }
   if constexpr (!NVFP4) {

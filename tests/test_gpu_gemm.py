@@ -309,14 +309,15 @@ def test_mxfp8_gemm_ragged_shapes_alpha_and_scale_spread(dev, shape):
 
 @pytest.mark.parametrize("shape", [(4096, 3072, 512), (3328, 3840, 384), (2048, 6144, 256), (8192, 1536, 1152),
                                    (4096, 8192, 256), (8192, 4096, 384), (4608, 5120, 128 * 5),
-                                   (4096, 2048, 512), (4352, 4096, 384)])
+                                   (4096, 2048, 512), (4352, 4096, 384), (1920, 4096, 256), (1024, 2048, 384)])
 def test_nvfp4_gemm_persistent_256_tile_kernel_full_compare(dev, shape):
-    """Dense shapes with M % 256 == N % 256 == K % 128 == 0 take the persistent 256x256 kernel that converts
-    the operands to fp16 between its MFMAs when their tiles fill at least 70 % of the compute units' slots
-    (192, 195, 192, 192, 512, 512 and 360 tiles on 256 units here: blocked and unblocked tile grids, one
-    and several tiles per workgroup with two, three, five and nine 128-deep spans per tile); the last two
-    shapes (128 and 272 tiles) fall to the 128x128 tile kernel.  Every output element is compared with the
-    oracle."""
+    """Dense shapes with M % 128 == N % 256 == K % 128 == 0 take the persistent kernel that converts the
+    operands to fp16 between its MFMAs, with 256x256 tiles (192, 195, 192, 192, 512, 512 and 360 tiles on 256
+    compute units: blocked and unblocked tile grids, one and several tiles per workgroup with two, three, five
+    and nine 128-deep spans per tile) or with 128x256 tiles where those fill the compute units better
+    ((4096, 2048): 256 tiles; (4352, 4096): 544, i.e. two and three per workgroup; (1920, 4096): 240, M no
+    multiple of 256); (1024, 2048) with 64 such tiles falls to the 128x128 tile kernel.  Every output element
+    is compared with the oracle."""
     m, n, k = shape
     gen = torch.Generator().manual_seed(k + 1)
     a, sa, ga = _nvfp4_operand(m, k, 1.0, gen)
