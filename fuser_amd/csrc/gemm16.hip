@@ -816,12 +816,8 @@ template <bool OUT_BF16, bool GROUPED, int TM = 4>
 int launch_nvfp4_fast(const Params& p, int cus, hipStream_t stream) {
   auto kern = nvfp4_gemm_256_kernel<OUT_BF16, GROUPED, TM>;
   constexpr int lds_bytes = 2 * (64 * TM + 256) * 128;  // 128 KiB / 96 KiB
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    if (e != hipSuccess) return fail(NVF_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    configured = true;
-  }
+  static uint64_t configured = 0;  // one bit per device; a benign race: the attribute call is idempotent
+  if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
   const int64_t tiles = (int64_t)(p.m / (64 * TM)) * (p.n / 256);  // grouped: an upper bound
   const unsigned grid = (unsigned)(tiles >= cus ? (cus & ~7) : ((tiles + 7) / 8) * 8);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds_bytes, stream, p);
@@ -1058,12 +1054,8 @@ int launch_nvfp4_skinny_ring_cfg(const Params& p, hipStream_t stream) {
   constexpr int ring_kib = 8 * DEPTH * SLOT_KIB;
   constexpr int lds_bytes = (ring_kib > red_kib ? ring_kib : red_kib) * 1024;
   static_assert(lds_bytes <= 160 * 1024, "LDS");
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    if (e != hipSuccess) return fail(NVF_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    configured = true;
-  }
+  static uint64_t configured = 0;  // one bit per device; a benign race: the attribute call is idempotent
+  if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
   hipLaunchKernelGGL(kern, dim3((unsigned)(p.n / (16 * RT))), dim3(512), lds_bytes, stream, p);
   return check_launch("nvfp4_skinny_ring_kernel");
 }
@@ -1337,12 +1329,8 @@ template <bool BF16_MMA, bool OUT_BF16>
 int launch_grouped16_fast(const Params& p, int cus, hipStream_t stream) {
   auto kern = grouped16_gemm_256_kernel<BF16_MMA, OUT_BF16>;
   constexpr int lds_bytes = 2 * 2 * 2048 * 16;  // 128 KiB
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    if (e != hipSuccess) return fail(NVF_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    configured = true;
-  }
+  static uint64_t configured = 0;  // one bit per device; a benign race: the attribute call is idempotent
+  if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
   hipLaunchKernelGGL(kern, dim3((unsigned)(cus & ~7)), dim3(256), lds_bytes, stream, p);
   return check_launch("grouped16_gemm_256_kernel");
 }
@@ -1351,12 +1339,8 @@ template <int BM, int BN, bool BF16_MMA, bool OUT_BF16>
 int launch_cfg(const Params& p, int grid, hipStream_t stream) {
   auto kern = gemm16_kernel<BM, BN, BF16_MMA, OUT_BF16>;
   constexpr int lds_bytes = 2 * (BM + BN) * 128;
-  static bool configured = false;  // benign race: the attribute call is idempotent
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    if (e != hipSuccess) return fail(NVF_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    configured = true;
-  }
+  static uint64_t configured = 0;  // one bit per device; a benign race: the attribute call is idempotent
+  if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_bytes, stream, p);
   return check_launch("gemm16_kernel");
 }
@@ -1365,12 +1349,8 @@ template <int BM, int BN, bool OUT_BF16, bool OUT_F32 = false>
 int launch_nvfp4_tile(const Params& p, int grid, hipStream_t stream) {
   auto kern = nvfp4_tile_kernel<BM, BN, OUT_BF16, OUT_F32>;
   constexpr int lds_bytes = 2 * (BM + BN) * 128;
-  static bool configured = false;  // benign race: the attribute call is idempotent
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    if (e != hipSuccess) return fail(NVF_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    configured = true;
-  }
+  static uint64_t configured = 0;  // one bit per device; a benign race: the attribute call is idempotent
+  if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_bytes, stream, p);
   return check_launch("nvfp4_tile_kernel");
 }
@@ -1397,12 +1377,8 @@ int launch_nvfp4_splitk(const Params& p0, int splits, float* workspace, hipStrea
   p.partial = workspace;
   auto kern = nvfp4_tile_kernel<128, 128, OUT_BF16, false, true>;
   constexpr int lds_bytes = 2 * (128 + 128) * 128;
-  static bool configured = false;  // benign race: the attribute call is idempotent
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    if (e != hipSuccess) return fail(NVF_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    configured = true;
-  }
+  static uint64_t configured = 0;  // one bit per device; a benign race: the attribute call is idempotent
+  if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
   const int64_t items = ceil_div(p.m, 128) * ceil_div(p.n, 128) * p.splits;
   hipLaunchKernelGGL(kern, dim3((unsigned)items), dim3(256), lds_bytes, stream, p);
   int rc = check_launch("nvfp4_tile_kernel (split K)");

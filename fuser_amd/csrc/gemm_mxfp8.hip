@@ -476,12 +476,8 @@ template <int TM, bool OUT_BF16>
 int launch_fast(const Params& p, hipStream_t stream) {
   auto kern = mxfp8_gemm_256_kernel<TM, OUT_BF16>;
   constexpr int lds_bytes = 2 * (64 * TM + 256) * 128;  // 128 KiB / 96 KiB
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    if (e != hipSuccess) return fail(NVF_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    configured = true;
-  }
+  static uint64_t configured = 0;  // one bit per device; a benign race: the attribute call is idempotent
+  if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
   const int64_t tiles = (int64_t)(p.m / (64 * TM)) * (p.n / 256);
   const int cus = 256;
   const unsigned grid = (unsigned)(tiles >= cus ? cus : ((tiles + 7) / 8) * 8);
@@ -665,12 +661,8 @@ int launch_skinny_cfg(const Params& p, hipStream_t stream) {
   constexpr int ring = 8 * DEPTH * SLOT, red = 8 * RT * TT * 1024;
   constexpr int lds_bytes = ring > red ? ring : red;
   static_assert(lds_bytes <= 160 * 1024, "LDS");
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    if (e != hipSuccess) return fail(NVF_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    configured = true;
-  }
+  static uint64_t configured = 0;  // one bit per device; a benign race: the attribute call is idempotent
+  if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
   hipLaunchKernelGGL(kern, dim3((unsigned)(p.n / (16 * RT))), dim3(512), lds_bytes, stream, p);
   return check_launch("mxfp8_skinny_kernel");
 }
@@ -701,12 +693,8 @@ template <int BM, int BN, bool OUT_BF16>
 int launch_cfg(const Params& p, hipStream_t stream) {
   auto kern = mxfp8_gemm_kernel<BM, BN, OUT_BF16>;
   constexpr int lds_bytes = 2 * (BM + BN) * 128;
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    if (e != hipSuccess) return fail(NVF_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    configured = true;
-  }
+  static uint64_t configured = 0;  // one bit per device; a benign race: the attribute call is idempotent
+  if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
   const int64_t tiles = ceil_div(p.m, BM) * ceil_div(p.n, BN);
   hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(256), lds_bytes, stream, p);
   return check_launch("mxfp8_gemm_kernel");

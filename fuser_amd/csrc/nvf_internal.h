@@ -15,6 +15,18 @@ int fail(int status, const char* fmt, ...) __attribute__((format(printf, 2, 3)))
 // Checks the launch that was just issued on the calling thread.
 int check_launch(const char* what);
 
+// Raises a kernel's dynamic LDS limit on the current device, once per device (`done`: one bit per device id).
+inline int allow_dynamic_lds(const void* kernel, int bytes, uint64_t& done) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return fail(NVF_ERR_NO_DEVICE, "hipGetDevice failed");
+  const uint64_t bit = 1ull << (dev & 63);
+  if (done & bit) return NVF_OK;
+  const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e != hipSuccess) return fail(NVF_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  done |= bit;
+  return NVF_OK;
+}
+
 inline int64_t ceil_div(int64_t x, int64_t y) { return (x + y - 1) / y; }
 inline int64_t round_up(int64_t x, int64_t y) { return ceil_div(x, y) * y; }
 
