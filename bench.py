@@ -157,6 +157,10 @@ def main():
                                     "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
                                                  "frac": round(tf / PEAK_F16_TFLOPS, 4), "traffic": None,
                                                  "note": "fp16 MFMA issued (exact fp16 dequantisation of e2m1 x e4m3)"}}
+        gn = torch.ones((), device=dev)
+        ms_b, _ = timed(lambda: nvf_cutlass.nvfp4_scaled_mm_blockscale(a, b, sa, sb, alpha, gn), 20, 3)
+        extra["nvfp4_gemm_blockscale_8192"] = {"ms": round(ms_b, 4), "TFLOP/s": round(2.0 * m * n * k / ms_b / 1e9, 1),
+                                               "note": "GEMM to an fp32 workspace + NVFP4 re-quantization of the product (two launches)"}
 
     def run_llm():
         res = {}

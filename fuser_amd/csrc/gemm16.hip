@@ -523,7 +523,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
 // TM = 32-row accumulator tiles of a wavefront along M: 4 -> 256x256 workgroup tile, 2 -> 128x256 (dense shapes
 // whose 256x256 tiles would leave compute units idle; 1.5 times the conversion work per MFMA).  The statement
 // order for TM = 4 is the one the 8192^3 measurements were made with.
-template <bool OUT_BF16, bool GROUPED, int TM = 4>
+template <bool OUT_BF16, bool GROUPED, int TM = 4, bool OUT_F32 = false>
 __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   static_assert(TM == 4 || (TM == 2 && !GROUPED), "tile height");
   constexpr int BM = 64 * TM, BN = 256;
@@ -792,18 +792,23 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
     // acc[i][j][r] = C[m = li][n = (r/4)*8 + lg*4 + r%4] of its 32x32 sub-tile.
     const Where cw = tile_where(c_tile);
     const float alpha = p.alpha[cw.g];
-    uint16_t* out = static_cast<uint16_t*>(p.out);
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-      uint16_t* orow = out + (cw.m0 + wm * (32 * TM) + i * 32 + li) * p.n + cw.n0 + wn * 64 + lg * 4;
+      const int64_t at = (cw.m0 + wm * (32 * TM) + i * 32 + li) * p.n + cw.n0 + wn * 64 + lg * 4;
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
 #pragma unroll
         for (int rq = 0; rq < 4; ++rq) {
-          u32x2 v;
-          v[0] = pack2(acc[i][j][rq * 4 + 0] * alpha, acc[i][j][rq * 4 + 1] * alpha, OUT_BF16);
-          v[1] = pack2(acc[i][j][rq * 4 + 2] * alpha, acc[i][j][rq * 4 + 3] * alpha, OUT_BF16);
-          *reinterpret_cast<u32x2*>(orow + j * 32 + rq * 8) = v;
+          if constexpr (OUT_F32) {
+            *reinterpret_cast<f32x4*>(static_cast<float*>(p.out) + at + j * 32 + rq * 8) =
+                f32x4{acc[i][j][rq * 4 + 0] * alpha, acc[i][j][rq * 4 + 1] * alpha, acc[i][j][rq * 4 + 2] * alpha,
+                      acc[i][j][rq * 4 + 3] * alpha};
+          } else {
+            u32x2 v;
+            v[0] = pack2(acc[i][j][rq * 4 + 0] * alpha, acc[i][j][rq * 4 + 1] * alpha, OUT_BF16);
+            v[1] = pack2(acc[i][j][rq * 4 + 2] * alpha, acc[i][j][rq * 4 + 3] * alpha, OUT_BF16);
+            *reinterpret_cast<u32x2*>(static_cast<uint16_t*>(p.out) + at + j * 32 + rq * 8) = v;
+          }
         }
       }
     }
@@ -812,9 +817,9 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
 #undef NVF_PIN_ACC
 }
 
-template <bool OUT_BF16, bool GROUPED, int TM = 4>
+template <bool OUT_BF16, bool GROUPED, int TM = 4, bool OUT_F32 = false>
 int launch_nvfp4_fast(const Params& p, int cus, hipStream_t stream) {
-  auto kern = nvfp4_gemm_256_kernel<OUT_BF16, GROUPED, TM>;
+  auto kern = nvfp4_gemm_256_kernel<OUT_BF16, GROUPED, TM, OUT_F32>;
   constexpr int lds_bytes = 2 * (64 * TM + 256) * 128;  // 128 KiB / 96 KiB
   static uint64_t configured = 0;  // one bit per device; a benign race: the attribute call is idempotent
   if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
@@ -1460,6 +1465,10 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int6
 // dense NVFP4 with an fp32 result (the product that the block-scaled epilogue op re-quantizes)
 int launch_nvfp4_f32(const Params& p, int cus, hipStream_t stream) {
   auto tiles = [&](int bm, int bn) { return ceil_div(p.m, bm) * ceil_div(p.n, bn); };
+  if ((p.m & 255) == 0 && (p.n & 255) == 0 && (p.k & 127) == 0 && p.k >= 256) {
+    const int64_t t = tiles(256, 256);  // as for the 16-bit results: only if the tiles fill the compute units
+    if (100 * ceil_div(t, cus) <= 144 * t / cus) return launch_nvfp4_fast<false, false, 4, true>(p, cus, stream);
+  }
   if (tiles(256, 256) >= cus) return launch_nvfp4_tile<256, 256, false, true>(p, cus, stream);
   if (tiles(128, 128) >= cus) {
     const int64_t t = tiles(128, 128);

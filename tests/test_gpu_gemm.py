@@ -82,13 +82,15 @@ def test_nvfp4_gemm_epilogue_reference_shapes(dev, dtype, shape):
     assert (unpack(q) != unpack(eq)).float().mean() < 2e-3 and (sf != esf).float().mean() < 2e-3
 
 
-def test_nvfp4_gemm_epilogue_quantizes_its_own_fp32_product_bit_exactly(dev):
+@pytest.mark.parametrize("shape", [(200, 160, 192), (4096, 3072, 256)])
+def test_nvfp4_gemm_epilogue_quantizes_its_own_fp32_product_bit_exactly(dev, shape):
     """Through the C ABI, where the caller owns the workspace: the fp32 product left there agrees with the
     oracle product to fp32 summation noise, and payload and scales are bit-identical to the oracle
-    quantizer applied to exactly that product (rows not a multiple of 128, scale columns padded)."""
+    quantizer applied to exactly that product (rows not a multiple of 128 and padded scale columns on the
+    tile kernel; a shape whose fp32 product comes from the persistent 256x256 kernel)."""
     from fuser_amd import capi
 
-    m, n, k = 200, 160, 192
+    m, n, k = shape
     gen = torch.Generator().manual_seed(11)
     a, sa, ga = _nvfp4_operand(m, k, 1.0, gen)
     b, sb, gb = _nvfp4_operand(n, k, 1.0, gen)
