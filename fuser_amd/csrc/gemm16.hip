@@ -497,8 +497,9 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
 }
 
 // -------------------------------------------------------------------------------------------------
-// NVFP4 fast path: dense, 256x256 tile, M % 256 == N % 256 == 0, K % 128 == 0, K >= 256.
-//   * 512 threads: 8 wavefronts as 2 (m) x 4 (n), each with a 128x64 accumulator tile, two per SIMD.
+// NVFP4 fast path: 256x256 (or 128x256) tile, N % 256 == 0, K % 128 == 0, K >= 256; dense with M % 256 (128) == 0,
+// or the whole 256-row tiles of every group of the grouped op; 16-bit or fp32 result.
+//   * 512 threads: 8 wavefronts as 2 (m) x 4 (n), each with a 128x64 (64x64) accumulator tile, two per SIMD.
 //     A single wavefront issues at most one non-MFMA instruction per ~8 cycles, which is too little for
 //     the conversion work next to 32-cycle MFMAs; with two wavefronts per SIMD one converts while the
 //     other's MFMA runs.
