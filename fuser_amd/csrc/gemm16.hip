@@ -54,6 +54,8 @@ struct Params {
   int skip_whole_256 = 0;
   // skinny kernel: first of the (at most 128) activation rows this launch computes, a multiple of 128
   int m_base = 0;
+  // grouped skinny kernel: the group sizes it serves; the tile kernel skips groups of fewer than min_rows rows
+  int rows_lo = 0, rows_hi = 0, min_rows = 0;
 };
 
 __device__ __forceinline__ uint32_t pack2(float a, float b, bool out_bf16) {
@@ -298,7 +300,7 @@ __global__ __launch_bounds__(256) void nvfp4_tile_kernel(const Params p) {
       int cnt = 0;
       if (g < p.groups) {
         const int mg = p.problem_sizes[g * 3];
-        const int rest = mg - (p.skip_whole_256 ? (mg & ~255) : 0);
+        const int rest = mg < p.min_rows ? 0 : mg - (p.skip_whole_256 ? (mg & ~255) : 0);
         cnt = rest > 0 ? ((rest + BM - 1) / BM) * tiles_n : 0;
       }
       int incl = cnt;
@@ -874,7 +876,9 @@ __device__ __forceinline__ void dequant_frags(const u32x4 q, uint32_t s2, u32x4 
   }
 }
 
-template <int RT, int TT, bool OUT_BF16, int DEPTH>
+// GROUPED: one workgroup per (group, block of 16*RT weight rows); it serves groups of rows_lo .. rows_hi rows
+// (at most 16*TT) and returns at once for the others, which other launches take.
+template <int RT, int TT, bool OUT_BF16, int DEPTH, bool GROUPED = false>
 __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) {
   constexpr int W = 8;
   constexpr int NT = RT + TT;
@@ -889,19 +893,32 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, g = lane >> 4;
-  const int n0 = blockIdx.x * (16 * RT);
-  const int m_loc = min(p.m - p.m_base, 128);  // activation rows of this launch: [m_base, m_base + m_loc)
-  const int tt_count = (m_loc + 15) >> 4;
   const int kbytes = p.k >> 1;
   const int chunks = p.k >> 7;
   const int sf_padded = p.k >> 4;  // K % 128 == 0: no padding columns
+  int n0, m_loc, grp = 0;
+  int64_t a_row0 = p.m_base, asf_row0 = p.m_base, b_row0 = 0;  // first activation row, its scale row, first weight row
+  if constexpr (GROUPED) {
+    const int nblocks = p.n / (16 * RT);
+    grp = blockIdx.x / nblocks;
+    n0 = (blockIdx.x - grp * nblocks) * (16 * RT);
+    m_loc = __builtin_amdgcn_readfirstlane(p.problem_sizes[grp * 3]);
+    if (m_loc < p.rows_lo || m_loc > p.rows_hi) return;
+    a_row0 = __builtin_amdgcn_readfirstlane(p.expert_offsets[grp]);
+    asf_row0 = __builtin_amdgcn_readfirstlane(p.sf_offsets[grp]);  // the group's own scale slab
+    b_row0 = (int64_t)grp * p.n;
+  } else {
+    n0 = blockIdx.x * (16 * RT);
+    m_loc = min(p.m - p.m_base, 128);  // activation rows of this launch: [m_base, m_base + m_loc)
+  }
+  const int tt_count = (m_loc + 15) >> 4;
 
   // ---- load side (memory order): lane L fetches row L/4, piece (L%4) ^ ((L/16)&3) of a payload tile
   const int lrow = lane >> 2, lpiece = (lane & 3) ^ ((lane >> 4) & 3);
-  const uint8_t* b_base = p.b + (int64_t)n0 * kbytes;
-  const uint8_t* bsf_base = p.sfb + swizzle_128x4(n0 & ~127, 0, sf_padded);
-  const uint8_t* a_base = p.a + (int64_t)p.m_base * kbytes;
-  const uint8_t* asf_base = p.sfa + swizzle_128x4(p.m_base, 0, sf_padded);  // the 128-row scale tile of these rows
+  const uint8_t* b_base = p.b + (b_row0 + n0) * kbytes;
+  const uint8_t* bsf_base = p.sfb + b_row0 * sf_padded + swizzle_128x4(n0 & ~127, 0, sf_padded);
+  const uint8_t* a_base = p.a + a_row0 * kbytes;
+  const uint8_t* asf_base = p.sfa + asf_row0 * sf_padded;  // the 128-row scale tile of these rows (row0 % 128 == 0)
   uint32_t b_off[RT], a_off[TT], bsf_off[B_SC], asf_off[A_SC];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) b_off[rt] = (uint32_t)(rt * 16 + lrow) * (uint32_t)kbytes + lpiece * 16;
@@ -930,11 +947,16 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) lds_dma16(sb + rt * 1024, b_base, b_off[rt] + c * 64u);
 #pragma unroll
-    for (int tt = 0; tt < TT; ++tt) lds_dma16(sb + (RT + tt) * 1024, a_base, a_off[tt] + c * 64u);
+    for (int tt = 0; tt < TT; ++tt) {
+      // with one slot every wait is for everything, so tiles without rows need not be fetched
+      if (DEPTH == 2 || tt < tt_count) lds_dma16(sb + (RT + tt) * 1024, a_base, a_off[tt] + c * 64u);
+    }
 #pragma unroll
     for (int j = 0; j < B_SC; ++j) lds_dma16(sb + (NT + j) * 1024, bsf_base, bsf_off[j] + c * 1024u);
 #pragma unroll
-    for (int j = 0; j < A_SC; ++j) lds_dma16(sb + (NT + B_SC + j) * 1024, asf_base, asf_off[j] + c * 1024u);
+    for (int j = 0; j < A_SC; ++j) {
+      if (DEPTH == 2 || 2 * j < tt_count) lds_dma16(sb + (NT + B_SC + j) * 1024, asf_base, asf_off[j] + c * 1024u);
+    }
   };
 
   // ---- read side (MFMA order): lane (r, g) = row r, payload piece g, scale blocks 2g, 2g+1 of the chunk
@@ -1018,7 +1040,7 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
 
   // ---- sum the wavefronts' partial tiles in wave order and store: all tiles in one round if they fit the
   // ring's memory (RT * TT <= 8), else one round per weight-row tile
-  const float alpha = p.alpha[0];
+  const float alpha = p.alpha[grp];
   uint16_t* out = static_cast<uint16_t*>(p.out);
   constexpr int ROUNDS = RT * TT <= 8 ? 1 : RT;
   constexpr int RPR = RT / ROUNDS;  // weight-row tiles per round
@@ -1044,7 +1066,7 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
         u32x2 v;
         v[0] = pack2(s[0] * alpha, s[1] * alpha, OUT_BF16);
         v[1] = pack2(s[2] * alpha, s[3] * alpha, OUT_BF16);
-        *reinterpret_cast<u32x2*>(out + (int64_t)(p.m_base + tok) * p.n + n0 + (round * RPR + r2) * 16 + 4 * (l >> 4)) = v;
+        *reinterpret_cast<u32x2*>(out + (a_row0 + tok) * p.n + n0 + (round * RPR + r2) * 16 + 4 * (l >> 4)) = v;
       }
     }
   }
@@ -1064,6 +1086,26 @@ int launch_nvfp4_skinny_ring_cfg(const Params& p, hipStream_t stream) {
   if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
   hipLaunchKernelGGL(kern, dim3((unsigned)(p.n / (16 * RT))), dim3(512), lds_bytes, stream, p);
   return check_launch("nvfp4_skinny_ring_kernel");
+}
+
+template <int RT, int TT, bool OUT_BF16>
+int launch_nvfp4_skinny_grouped(const Params& p0, int rows_lo, int rows_hi, hipStream_t stream) {
+  constexpr int SLOT_KIB = RT + TT + (RT + 1) / 2 + (TT + 1) / 2;
+  constexpr int DEPTH = 8 * 2 * SLOT_KIB <= 160 ? 2 : 1;
+  auto kern = nvfp4_skinny_ring_kernel<RT, TT, OUT_BF16, DEPTH, true>;
+  constexpr int red_kib = 8 * (RT * TT <= 8 ? RT * TT : TT);
+  constexpr int ring_kib = 8 * DEPTH * SLOT_KIB;
+  constexpr int lds_bytes = (ring_kib > red_kib ? ring_kib : red_kib) * 1024;
+  static_assert(lds_bytes <= 160 * 1024, "LDS");
+  static uint64_t configured = 0;  // one bit per device; a benign race: the attribute call is idempotent
+  if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
+  Params p = p0;
+  p.rows_lo = rows_lo;
+  p.rows_hi = rows_hi;
+  const int64_t wgs = (int64_t)p.groups * (p.n / (16 * RT));
+  if (wgs >= ((int64_t)1 << 31)) return fail(NVF_ERR_UNSUPPORTED_SHAPE, "too many (group, row block) pairs for one launch");
+  hipLaunchKernelGGL(kern, dim3((unsigned)wgs), dim3(512), lds_bytes, stream, p);
+  return check_launch("nvfp4_skinny_ring_kernel (grouped)");
 }
 
 template <int TT, bool OUT_BF16>
@@ -1436,6 +1478,18 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int6
       return launch_grouped16_fast<BF16_MMA, OUT_BF16>(p, cus, stream);
   }
   if constexpr (NVFP4) {
+    // Grouped NVFP4: groups of up to 128 rows (MoE decode, the small experts of a prefill) stream their expert's
+    // weights once through the skinny kernel; the launches below then skip them.  The group sizes live on
+    // the device, so every kernel is always launched; workgroups without work return at once.
+    if (!dense && p.min_rows == 0 && (p.n & 63) == 0 && (p.k & 127) == 0 && (int64_t)p.k * 64 < (1ll << 31)) {
+      int rc = launch_nvfp4_skinny_grouped<4, 2, OUT_BF16>(p, 1, 32, stream);
+      if (rc != NVF_OK) return rc;
+      rc = launch_nvfp4_skinny_grouped<4, 8, OUT_BF16>(p, 33, 128, stream);
+      if (rc != NVF_OK) return rc;
+      Params rest = p;
+      rest.min_rows = 129;
+      return launch_sized<NVFP4, BF16_MMA, OUT_BF16>(rest, m_hint, cus, workspace, workspace_bytes, stream);
+    }
     // Grouped NVFP4 with room for whole 256-row tiles: those go to the 256x256 kernel (about 1.4 times as
     // fast per flop), the ends of the groups to the 128x128 tile kernel.  The group sizes live on the
     // device, so both kernels are always launched; one that finds no work returns at once.

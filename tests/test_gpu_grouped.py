@@ -228,6 +228,47 @@ def test_nvfp4_grouped_mm_whole_tiles_and_group_ends(dev, sizes, n, k):
         assert ((out[:rows].float().cpu() - ref[:rows]).abs() / scale).max().item() <= GEMM_MAX_REL, (sizes, dtype)
 
 
+@pytest.mark.parametrize("n,k", [(128, 128), (384, 384), (256, 1152), (128, 2048)])
+def test_nvfp4_grouped_mm_small_groups_stream_their_weights(dev, n, k):
+    """K % 128 == 0: groups of 1..32 and of 33..128 rows each run on the weight-streaming kernel (one workgroup
+    per group and 64 weight rows), larger groups on the tile kernels, which skip the small ones.  Sizes on
+    both sides of every class border, empty groups, a different alpha per group, poisoned padding of the
+    activation scale slabs, one to sixteen 128-deep chunks (wavefronts without work); every element compared,
+    rows after the last group untouched, run-to-run bit equality."""
+    from fuser_amd import nvf_cutlass
+
+    sizes = [0, 1, 16, 17, 32, 33, 64, 65, 128, 129, 300, 0, 2, 100]
+    g, m = len(sizes), sum(sizes) + 5
+    gen = torch.Generator().manual_seed(n * 7 + k)
+    x = torch.randn(m, k, generator=gen).bfloat16()
+    w = (torch.randn(g, n, k, generator=gen) * 0.05).bfloat16()
+    ps, eo, st, ct = _grouped_args(sizes, n, k, dev)
+    so = start_offsets([O.round_up(t, 128) for t in sizes])
+    aq, valid = O.grouped_block_quantize_nvfp4(x, eo, so, None)
+    lin = torch.zeros_like(valid, dtype=torch.bool)
+    for e, t in enumerate(sizes):
+        if t:
+            ones = O.linear_to_swizzled_128_4(torch.ones(t, k // 16, dtype=torch.uint8))
+            lin[int(so[e]) : int(so[e]) + ones.shape[0]] |= ones.bool()
+    asf = torch.where(lin, valid, torch.full_like(valid, 0x7F))  # NaN code wherever no row owns the byte
+    bq = torch.empty(g, n, k // 2, dtype=torch.uint8)
+    bsf = torch.empty(g, n, k // 16, dtype=torch.uint8)
+    alphas = torch.empty(g)
+    for e in range(g):
+        gs = gs_of(w[e])
+        bq[e], bsf[e] = O.block_quantize_nvfp4(w[e], gs, True)
+        alphas[e] = (e + 1) / gs
+    ref = O.ref_nvfp4_scaled_grouped_mm(aq, bq, valid, bsf, alphas, ps, eo, so)
+    rows = sum(sizes)
+    args = (fp4(aq.to(dev)), fp4(bq.to(dev)), e4m3(asf.to(dev)), e4m3(bsf.to(dev)), alphas.to(dev), st, ct, ps.to(dev), eo.to(dev), so.to(dev))
+    for dtype in (torch.bfloat16, torch.float16):
+        out = nvf_cutlass.nvfp4_scaled_grouped_mm(*args, dtype)
+        torch.cuda.synchronize()
+        scale = ref[:rows].abs().amax(dim=1, keepdim=True).clamp(min=1e-30)
+        assert ((out[:rows].float().cpu() - ref[:rows]).abs() / scale).max().item() <= GEMM_MAX_REL, (n, k, dtype)
+        assert torch.equal(out[:rows], nvf_cutlass.nvfp4_scaled_grouped_mm(*args, dtype)[:rows])
+
+
 def _zipf_sizes(tokens, topk, experts, s, seed):
     gen = torch.Generator().manual_seed(seed)
     p = 1.0 / torch.arange(1, experts + 1).float() ** s
