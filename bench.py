@@ -238,6 +238,19 @@ def main():
             ms, _ = timed(lambda: nvf_cutlass.nvfp4_scaled_grouped_mm(aq, bq4, asf, bsf8, alphas, st, ct, ps, eo, so, torch.bfloat16), 10, 2)
             tf = 2.0 * rows * n * k / ms / 1e9
             res[f"K{k}_N{n}"] = {"ms": round(ms, 4), "useful_TFLOP/s": round(tf, 1), "frac_of_f16_peak": round(tf / PEAK_F16_TFLOPS, 4)}
+            # the same experts at decode size: 64 tokens x top-8 = 512 rows spread uniformly (bound by streaming the
+            # weights of the active experts once)
+            d_sizes = torch.bincount(torch.randint(0, g, (512,), generator=torch.Generator().manual_seed(0)), minlength=g).int()
+            d_pad = (d_sizes + 127) // 128 * 128
+            d_eo = (torch.cumsum(d_sizes, 0) - d_sizes).int().to(dev)
+            d_so = (torch.cumsum(d_pad, 0) - d_pad).int().to(dev)
+            d_q, d_sf = ops.nv_grouped_block_quantize(x[:512].contiguous(), d_eo, d_so, None, 16)
+            d_ps = torch.stack([d_sizes, torch.full_like(d_sizes, n), torch.full_like(d_sizes, k)], 1).int().to(dev)
+            ms_d, _ = timed(lambda: nvf_cutlass.nvfp4_scaled_grouped_mm(d_q, bq4, d_sf, bsf8, alphas, st, ct, d_ps, d_eo, d_so,
+                                                                        torch.bfloat16), 10, 2)
+            wbytes = int((d_sizes > 0).sum()) * n * k * 0.5625
+            res[f"decode_512rows_K{k}_N{n}"] = {"us": round(ms_d * 1e3, 1), "active_experts": int((d_sizes > 0).sum()),
+                                                "weight_GB/s": round(wbytes / ms_d / 1e6, 1)}
             del bq, bsf, bq4, bsf8, x, aq, asf
         extra["nvfp4_grouped_mm"] = res
 

@@ -878,8 +878,12 @@ __device__ __forceinline__ void dequant_frags(const u32x4 q, uint32_t s2, u32x4 
 
 // GROUPED: one workgroup per (group, block of 16*RT weight rows); it serves groups of rows_lo .. rows_hi rows
 // (at most 16*TT) and returns at once for the others, which other launches take.
-template <int RT, int TT, bool OUT_BF16, int DEPTH, bool GROUPED = false>
+// NSPLIT (grouped only, where the groups supply enough workgroups): the 8 wavefronts own 8 different blocks of
+// 16*RT weight rows and each walks all of K on its own - a long pipeline per wavefront and no reduction -
+// instead of sharing one block and splitting K.
+template <int RT, int TT, bool OUT_BF16, int DEPTH, bool GROUPED = false, bool NSPLIT = false>
 __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) {
+  static_assert(GROUPED || !NSPLIT, "the dense op has too few row blocks to give every wavefront its own");
   constexpr int W = 8;
   constexpr int NT = RT + TT;
   constexpr int B_SC = (RT + 1) / 2, A_SC = (TT + 1) / 2;     // scale blocks (1 KiB) per operand
@@ -899,9 +903,9 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
   int n0, m_loc, grp = 0;
   int64_t a_row0 = p.m_base, asf_row0 = p.m_base, b_row0 = 0;  // first activation row, its scale row, first weight row
   if constexpr (GROUPED) {
-    const int nblocks = p.n / (16 * RT);
+    const int nblocks = p.n / (16 * RT * (NSPLIT ? W : 1));
     grp = blockIdx.x / nblocks;
-    n0 = (blockIdx.x - grp * nblocks) * (16 * RT);
+    n0 = ((blockIdx.x - grp * nblocks) * (NSPLIT ? W : 1) + (NSPLIT ? wave : 0)) * (16 * RT);
     m_loc = __builtin_amdgcn_readfirstlane(p.problem_sizes[grp * 3]);
     if (m_loc < p.rows_lo || m_loc > p.rows_hi) return;
     a_row0 = __builtin_amdgcn_readfirstlane(p.expert_offsets[grp]);
@@ -978,12 +982,14 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) acc[rt][tt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
+  constexpr int CSTEP = NSPLIT ? 1 : W;  // distance of a wavefront's consecutive chunks
+  const int c_first = NSPLIT ? 0 : wave;
 #pragma unroll
-  for (int d = 0; d < DEPTH; ++d) issue_chunk(wave + d * W, d);
+  for (int d = 0; d < DEPTH; ++d) issue_chunk(c_first + d * CSTEP, d);
   int slot = 0;
-  for (int c = wave; c < chunks; c += W) {
+  for (int c = c_first; c < chunks; c += CSTEP) {
     // the oldest chunk in flight has landed when only the loads of the next one (if there is one) are pending
-    if (DEPTH == 2 && c + W < chunks)
+    if (DEPTH == 2 && c + CSTEP < chunks)
       asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NDMA) : "memory");
     else
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -1002,7 +1008,7 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
 #pragma unroll
       for (int tt = 0; tt < TT; ++tt) sc[RT + tt] = *reinterpret_cast<const uint32_t*>(sp + rd_asc[tt]) >> sc_shift;
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // read out: the slot may be refilled
-      issue_chunk(c + DEPTH * W, slot);
+      issue_chunk(c + DEPTH * CSTEP, slot);
     }
     u32x4 fb[RT][4];
 #pragma unroll
@@ -1017,7 +1023,7 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
           as = *reinterpret_cast<const uint32_t*>(sp + rd_asc[tt]) >> sc_shift;
           if (tt + 1 == tt_count) {
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the last read of the slot is complete
-            issue_chunk(c + DEPTH * W, slot);
+            issue_chunk(c + DEPTH * CSTEP, slot);
           }
         } else {
           aq = q[kLazyA ? 0 : RT + tt];
@@ -1035,13 +1041,30 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
     }
     if constexpr (DEPTH == 2) slot ^= 1;
   }
+  const float alpha = p.alpha[grp];
+  uint16_t* out = static_cast<uint16_t*>(p.out);
+  if constexpr (NSPLIT) {
+    // every wavefront holds finished sums: element e of lane l = weight row 4*(l/16) + e, activation row l%16
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) {
+      const int tok = tt * 16 + r;
+      if (tok < m_loc) {
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+          u32x2 v;
+          v[0] = pack2(acc[rt][tt][0] * alpha, acc[rt][tt][1] * alpha, OUT_BF16);
+          v[1] = pack2(acc[rt][tt][2] * alpha, acc[rt][tt][3] * alpha, OUT_BF16);
+          *reinterpret_cast<u32x2*>(out + (a_row0 + tok) * p.n + n0 + rt * 16 + 4 * g) = v;
+        }
+      }
+    }
+    return;
+  }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no LDS-direct load may be pending when the ring is reused
   __syncthreads();
 
   // ---- sum the wavefronts' partial tiles in wave order and store: all tiles in one round if they fit the
   // ring's memory (RT * TT <= 8), else one round per weight-row tile
-  const float alpha = p.alpha[grp];
-  uint16_t* out = static_cast<uint16_t*>(p.out);
   constexpr int ROUNDS = RT * TT <= 8 ? 1 : RT;
   constexpr int RPR = RT / ROUNDS;  // weight-row tiles per round
   const int tiles = RPR * tt_count;   // tile index inside a round: rt * tt_count + tt
@@ -1088,12 +1111,12 @@ int launch_nvfp4_skinny_ring_cfg(const Params& p, hipStream_t stream) {
   return check_launch("nvfp4_skinny_ring_kernel");
 }
 
-template <int RT, int TT, bool OUT_BF16>
+template <int RT, int TT, bool OUT_BF16, bool NSPLIT>
 int launch_nvfp4_skinny_grouped(const Params& p0, int rows_lo, int rows_hi, hipStream_t stream) {
   constexpr int SLOT_KIB = RT + TT + (RT + 1) / 2 + (TT + 1) / 2;
   constexpr int DEPTH = 8 * 2 * SLOT_KIB <= 160 ? 2 : 1;
-  auto kern = nvfp4_skinny_ring_kernel<RT, TT, OUT_BF16, DEPTH, true>;
-  constexpr int red_kib = 8 * (RT * TT <= 8 ? RT * TT : TT);
+  auto kern = nvfp4_skinny_ring_kernel<RT, TT, OUT_BF16, DEPTH, true, NSPLIT>;
+  constexpr int red_kib = NSPLIT ? 0 : 8 * (RT * TT <= 8 ? RT * TT : TT);
   constexpr int ring_kib = 8 * DEPTH * SLOT_KIB;
   constexpr int lds_bytes = (ring_kib > red_kib ? ring_kib : red_kib) * 1024;
   static_assert(lds_bytes <= 160 * 1024, "LDS");
@@ -1102,7 +1125,7 @@ int launch_nvfp4_skinny_grouped(const Params& p0, int rows_lo, int rows_hi, hipS
   Params p = p0;
   p.rows_lo = rows_lo;
   p.rows_hi = rows_hi;
-  const int64_t wgs = (int64_t)p.groups * (p.n / (16 * RT));
+  const int64_t wgs = (int64_t)p.groups * (p.n / (16 * RT * (NSPLIT ? 8 : 1)));
   if (wgs >= ((int64_t)1 << 31)) return fail(NVF_ERR_UNSUPPORTED_SHAPE, "too many (group, row block) pairs for one launch");
   hipLaunchKernelGGL(kern, dim3((unsigned)wgs), dim3(512), lds_bytes, stream, p);
   return check_launch("nvfp4_skinny_ring_kernel (grouped)");
@@ -1482,9 +1505,13 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int6
     // weights once through the skinny kernel; the launches below then skip them.  The group sizes live on
     // the device, so every kernel is always launched; workgroups without work return at once.
     if (!dense && p.min_rows == 0 && (p.n & 63) == 0 && (p.k & 127) == 0 && (int64_t)p.k * 64 < (1ll << 31)) {
-      int rc = launch_nvfp4_skinny_grouped<4, 2, OUT_BF16>(p, 1, 32, stream);
+      // With a shallow K a split of K over the wavefronts leaves each only a chunk or two: they then own
+      // different weight rows instead (K=2048, N=7168: 549 -> 464 us for 64 tokens x top-8; deeper K: slower).
+      int rc;
+      if (p.k < 4096 && (p.n & 255) == 0) rc = launch_nvfp4_skinny_grouped<2, 2, OUT_BF16, true>(p, 1, 32, stream);
+      else rc = launch_nvfp4_skinny_grouped<4, 2, OUT_BF16, false>(p, 1, 32, stream);
       if (rc != NVF_OK) return rc;
-      rc = launch_nvfp4_skinny_grouped<4, 8, OUT_BF16>(p, 33, 128, stream);
+      rc = launch_nvfp4_skinny_grouped<4, 8, OUT_BF16, false>(p, 33, 128, stream);
       if (rc != NVF_OK) return rc;
       Params rest = p;
       rest.min_rows = 129;

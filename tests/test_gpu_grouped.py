@@ -228,13 +228,14 @@ def test_nvfp4_grouped_mm_whole_tiles_and_group_ends(dev, sizes, n, k):
         assert ((out[:rows].float().cpu() - ref[:rows]).abs() / scale).max().item() <= GEMM_MAX_REL, (sizes, dtype)
 
 
-@pytest.mark.parametrize("n,k", [(128, 128), (384, 384), (256, 1152), (128, 2048)])
+@pytest.mark.parametrize("n,k", [(128, 128), (384, 384), (256, 1152), (128, 2048), (256, 4096), (512, 5120)])
 def test_nvfp4_grouped_mm_small_groups_stream_their_weights(dev, n, k):
     """K % 128 == 0: groups of 1..32 and of 33..128 rows each run on the weight-streaming kernel (one workgroup
     per group and 64 weight rows), larger groups on the tile kernels, which skip the small ones.  Sizes on
     both sides of every class border, empty groups, a different alpha per group, poisoned padding of the
-    activation scale slabs, one to sixteen 128-deep chunks (wavefronts without work); every element compared,
-    rows after the last group untouched, run-to-run bit equality."""
+    activation scale slabs, one to forty 128-deep chunks (wavefronts without work); N % 256 == 0 with K < 4096
+    takes the variant whose wavefronts own different weight rows, the rest the one that splits K; every
+    element compared, rows after the last group untouched, run-to-run bit equality."""
     from fuser_amd import nvf_cutlass
 
     sizes = [0, 1, 16, 17, 32, 33, 64, 65, 128, 129, 300, 0, 2, 100]
