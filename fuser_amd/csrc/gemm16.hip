@@ -1511,7 +1511,8 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int6
       if (p.k < 4096 && (p.n & 255) == 0) rc = launch_nvfp4_skinny_grouped<2, 2, OUT_BF16, true>(p, 1, 32, stream);
       else rc = launch_nvfp4_skinny_grouped<4, 2, OUT_BF16, false>(p, 1, 32, stream);
       if (rc != NVF_OK) return rc;
-      rc = launch_nvfp4_skinny_grouped<4, 8, OUT_BF16, false>(p, 33, 128, stream);
+      if (p.k < 4096 && (p.n & 255) == 0) rc = launch_nvfp4_skinny_grouped<2, 8, OUT_BF16, true>(p, 33, 128, stream);
+      else rc = launch_nvfp4_skinny_grouped<4, 8, OUT_BF16, false>(p, 33, 128, stream);
       if (rc != NVF_OK) return rc;
       Params rest = p;
       rest.min_rows = 129;
