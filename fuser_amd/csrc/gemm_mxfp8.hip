@@ -28,7 +28,7 @@ struct Params {
   const float* alpha;
   void* out;
   int m, n, k;
-  int m_base = 0;  // skinny kernel: first of the (at most 64) activation rows this launch computes
+  int m_base = 0;  // skinny kernel: first of the (at most 128) activation rows this launch computes, a multiple of 128
 };
 
 __device__ __forceinline__ uint32_t pack2(float a, float b, bool out_bf16) {
@@ -486,7 +486,7 @@ int launch_fast(const Params& p, hipStream_t stream) {
 }
 
 // -------------------------------------------------------------------------------------------------
-// Skinny path: up to 64 activation rows per launch (decode-sized activations; more rows in launches of 64),
+// Skinny path: up to 128 activation rows per launch (decode-sized activations; more rows in launches of 128),
 // K % 128 == 0, N % (16*RT) == 0.  A launch streams the weight matrix exactly once, so the op is bound by HBM
 // (by the last-level cache for the launches after the first):
 //   * A workgroup owns 16*RT weight rows for the whole of K and all M activation rows; its 8 wavefronts
@@ -510,9 +510,11 @@ template <int RT, int TT, bool OUT_BF16, int DEPTH>
 __global__ __launch_bounds__(512) void mxfp8_skinny_kernel(const Params p) {
   constexpr int W = 8;
   constexpr int NT = RT + TT;
-  constexpr int SLOT_BYTES = NT * (2048 + 256);
+  // activation rows r and r + 32 share their 16-byte scale group, so 32 groups serve any number of tiles
+  constexpr int A_SC_BYTES = (TT < 2 ? TT : 2) * 256;
+  constexpr int SLOT_BYTES = NT * 2048 + RT * 256 + A_SC_BYTES;
   constexpr int NDMA = 2 * NT + 2;  // loads per chunk and wavefront
-  static_assert(DEPTH >= 1 && DEPTH <= 3 && W * DEPTH * SLOT_BYTES <= 160 * 1024 && DEPTH * NDMA <= 63 && RT <= 4 && TT <= 4,
+  static_assert(DEPTH >= 1 && DEPTH <= 3 && W * DEPTH * SLOT_BYTES <= 160 * 1024 && DEPTH * NDMA <= 63 && RT <= 4 && TT <= 8,
                 "ring does not fit");
   extern __shared__ u32x4 lds[];  // ring during the K loop, then [W][tiles][64 lanes] partial sums
   const int tid = threadIdx.x;
@@ -544,7 +546,7 @@ __global__ __launch_bounds__(512) void mxfp8_skinny_kernel(const Params p) {
   const uint32_t bsf_off = (uint32_t)((((n0 & 127) + min(st, RT - 1) * 16 + r) & 31) * 16);
   const uint8_t* a_base = p.a + (int64_t)p.m_base * p.k;
   const uint8_t* asf_base = p.sfa + (int64_t)(p.m_base >> 7) * ((int64_t)sf_padded << 7);
-  const uint32_t asf_off = (uint32_t)((((p.m_base & 127) + min(st, TT - 1) * 16 + r) & 31) * 16);
+  const uint32_t asf_off = (uint32_t)((lane & 31) * 16);  // scale group of rows {lane, lane + 32, ...} of the 128-row tile
   const uint32_t lds_base = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)lds);
   const uint32_t ring_base = lds_base + (uint32_t)wave * (DEPTH * SLOT_BYTES);
   auto issue_chunk = [&](int c_in, int slot) {  // c_in is wave-uniform
@@ -562,7 +564,7 @@ __global__ __launch_bounds__(512) void mxfp8_skinny_kernel(const Params p) {
     // one load each for the scales of all weight tiles / all activation tiles (lanes of tiles that do not
     // exist stay off: a disabled lane writes nothing)
     if (lane < 16 * RT) lds_dma16(sb + NT * 2048, bsf_base, bsf_off + c * 512u);
-    if (lane < 16 * TT) lds_dma16(sb + NT * 2048 + RT * 256, asf_base, asf_off + c * 512u);
+    if (lane < A_SC_BYTES / 16) lds_dma16(sb + NT * 2048 + RT * 256, asf_base, asf_off + c * 512u);
   };
 
   // ---- read side (MFMA order)
@@ -573,7 +575,7 @@ __global__ __launch_bounds__(512) void mxfp8_skinny_kernel(const Params p) {
   for (int rt = 0; rt < RT; ++rt) rd_bsc[rt] = NT * 2048 + rt * 256 + r * 16 + ((((n0 & 127) + rt * 16) >> 5) & 3) * 4;
 #pragma unroll
   for (int tt = 0; tt < TT; ++tt)
-    rd_asc[tt] = NT * 2048 + (RT + tt) * 256 + r * 16 + ((((p.m_base & 127) + tt * 16) >> 5) & 3) * 4;
+    rd_asc[tt] = NT * 2048 + RT * 256 + ((tt & 1) * 16 + r) * 16 + ((((p.m_base & 127) + tt * 16) >> 5) & 3) * 4;
   const int sc_shift = g * 8;
 
   f32x4 acc[RT][TT];
@@ -655,7 +657,7 @@ __global__ __launch_bounds__(512) void mxfp8_skinny_kernel(const Params p) {
 
 template <int RT, int TT, bool OUT_BF16>
 int launch_skinny_cfg(const Params& p, hipStream_t stream) {
-  constexpr int SLOT = (RT + TT) * (2048 + 256);
+  constexpr int SLOT = (RT + TT) * 2048 + RT * 256 + (TT < 2 ? TT : 2) * 256;
   constexpr int DEPTH = 8 * 3 * SLOT <= 160 * 1024 ? 3 : (8 * 2 * SLOT <= 160 * 1024 ? 2 : 1);
   auto kern = mxfp8_skinny_kernel<RT, TT, OUT_BF16, DEPTH>;
   constexpr int ring = 8 * DEPTH * SLOT, red = 8 * RT * TT * 1024;
@@ -678,12 +680,18 @@ int launch_skinny_tt(const Params& p, hipStream_t stream) {
 
 template <bool OUT_BF16>
 int launch_skinny(const Params& p0, hipStream_t stream) {
+  // Up to 128 rows per launch.  With 8 activation tiles only one weight-row tile fits the LDS ring, and every
+  // workgroup fetches all activation rows: where N supplies enough workgroups of four weight-row tiles, launches
+  // of 64 rows with those are faster (128 x 14336 x 4096: 30 against 36 us; 128 x 4096 x 4096: 16 against 12).
+  const bool wide_n = (p0.n & 63) == 0 && p0.n / 64 >= 256 * 4 / 5;
+  const int slab = wide_n ? 64 : 128;
   Params p = p0;
-  for (p.m_base = 0; p.m_base < p.m; p.m_base += 64) {
-    const int rows = p.m - p.m_base;
+  for (p.m_base = 0; p.m_base < p.m; p.m_base += slab) {
+    const int rows = min(p.m - p.m_base, slab);
     const int rc = rows <= 16 ? launch_skinny_tt<1, OUT_BF16>(p, stream)
                  : rows <= 32 ? launch_skinny_tt<2, OUT_BF16>(p, stream)
-                              : launch_skinny_tt<4, OUT_BF16>(p, stream);
+                 : rows <= 64 ? launch_skinny_tt<4, OUT_BF16>(p, stream)
+                              : launch_skinny_cfg<1, 8, OUT_BF16>(p, stream);
     if (rc != NVF_OK) return rc;
   }
   return NVF_OK;
