@@ -592,7 +592,10 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
       w.g = __builtin_amdgcn_readfirstlane(lo);
       const int full_m = __builtin_amdgcn_readfirstlane(p.problem_sizes[w.g * 3]) / BM;
       const int local = __builtin_amdgcn_readfirstlane(t - tile_prefix[w.g]);
-      const int nt = local / full_m, mt = local - nt * full_m;
+      // bands of 4 m-tiles, n-major inside a band: 32 consecutive tiles share 4 A and 8 B panels
+      const int band = local / (4 * tiles_n), in_band = local - band * 4 * tiles_n;
+      const int band_h = min(4, full_m - 4 * band);
+      const int nt = in_band / band_h, mt = 4 * band + (in_band - nt * band_h);
       w.gm0 = mt * BM;
       w.m0 = (int64_t)__builtin_amdgcn_readfirstlane(p.expert_offsets[w.g]) + w.gm0;
       w.n0 = nt * BN;
@@ -1229,7 +1232,10 @@ __global__ __launch_bounds__(256, 1) void grouped16_gemm_256_kernel(const Params
     const int64_t row_off = __builtin_amdgcn_readfirstlane(p.expert_offsets[g]);
     const int tiles_m = (m_g + BM - 1) / BM;
     const int local = __builtin_amdgcn_readfirstlane(t - tile_prefix[g]);
-    const int nt = local / tiles_m, mt = local - nt * tiles_m;
+    // bands of 4 m-tiles, n-major inside a band: 32 consecutive tiles share 4 A and 8 B panels
+    const int band = local / (4 * tiles_n), in_band = local - band * 4 * tiles_n;
+    const int band_h = min(4, tiles_m - 4 * band);
+    const int nt = in_band / band_h, mt = 4 * band + (in_band - nt * band_h);
     Tile r;
     r.a = p.a + (row_off + (int64_t)mt * BM) * kb;
     r.b = p.b + ((int64_t)g * p.n + (int64_t)nt * BN) * kb;
