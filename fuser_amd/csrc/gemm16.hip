@@ -257,6 +257,15 @@ __global__ __launch_bounds__(256) void gemm16_kernel(const Params p) {
   }
 }
 
+// Grouped NVFP4: the rows of a group (m_g rows, the first at row row_off of the m_total activation rows) that the
+// 256x256 kernel computes: its whole 256-row tiles, and a last tile of more than 128 rows if the 256 rows that
+// tile loads lie inside the activation tensor (rows past the group are loaded and computed, not stored).  The
+// tile kernel takes the rows from there on; a value >= m_g means none are left.
+__device__ __forceinline__ int rows_in_256_tiles(int m_g, int64_t row_off, int m_total) {
+  const int whole = m_g & ~255;
+  return (m_g - whole > 128 && row_off + whole + 256 <= m_total) ? whole + 256 : whole;
+}
+
 // -------------------------------------------------------------------------------------------------
 // NVFP4 tile kernel for every shape the specialised NVFP4 kernels below do not take (ragged sizes, groups,
 // fp32 result).  Same persistent walk over (group, m-tile, n-tile) items, LDS layout and MFMA loop as the
@@ -300,7 +309,7 @@ __global__ __launch_bounds__(256) void nvfp4_tile_kernel(const Params p) {
       int cnt = 0;
       if (g < p.groups) {
         const int mg = p.problem_sizes[g * 3];
-        const int rest = mg < p.min_rows ? 0 : mg - (p.skip_whole_256 ? (mg & ~255) : 0);
+        const int rest = mg < p.min_rows ? 0 : mg - (p.skip_whole_256 ? rows_in_256_tiles(mg, p.expert_offsets[g], p.m) : 0);
         cnt = rest > 0 ? ((rest + BM - 1) / BM) * tiles_n : 0;
       }
       int incl = cnt;
@@ -343,7 +352,7 @@ __global__ __launch_bounds__(256) void nvfp4_tile_kernel(const Params p) {
     }
     const int m_g = dense ? p.m : p.problem_sizes[g * 3];
     const int64_t row_off = dense ? 0 : p.expert_offsets[g];
-    const int skipped = (!dense && p.skip_whole_256) ? (m_g & ~255) : 0;
+    const int skipped = (!dense && p.skip_whole_256) ? rows_in_256_tiles(m_g, row_off, p.m) : 0;
     const int tiles_m = (m_g - skipped + BM - 1) / BM;
     const int local = tile - tile_prefix[g];
     const int mt = local % tiles_m, nt = local / tiles_m;
@@ -550,9 +559,9 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   // ---- persistent tile walk: workgroup ids are dealt round-robin to the 8 XCDs, XCD x owns the tile
   // range [x*chunk, (x+1)*chunk); with the 8 (m) x 4 (n) blocked numbering the 32 tiles an XCD works on
   // at a time share 8 A panels and 4 B panels in its L2.
-  // GROUPED: the work list holds only the whole 256-row tiles of every group (rows [0, rows & ~255) of
-  // the group); what is left at the end of a group goes to the tile kernel.  A group's tiles are numbered
-  // m-tile fastest, so neighbouring tiles share the group's weight panel.
+  // GROUPED: the work list holds the 256-row tiles of every group that rows_in_256_tiles() names: the whole
+  // ones and a last one of more than 128 rows, whose rows past the group are computed and not stored; what
+  // is left at the end of a group goes to the tile kernel.
   const int tiles_m = p.m / BM, tiles_n = p.n / BN;
   int total = tiles_m * tiles_n;
   if constexpr (GROUPED) {
@@ -560,7 +569,7 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
       int running = 0;
       for (int base = 0; base < p.groups; base += 64) {
         const int g = base + lane;
-        const int cnt = g < p.groups ? (p.problem_sizes[g * 3] / BM) * tiles_n : 0;
+        const int cnt = g < p.groups ? (rows_in_256_tiles(p.problem_sizes[g * 3], p.expert_offsets[g], p.m) / BM) * tiles_n : 0;
         int incl = cnt;
 #pragma unroll
         for (int d = 1; d < 64; d <<= 1) {
@@ -580,7 +589,7 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   const int range_end = min((xcd + 1) * chunk_tiles, total);
   const bool blocked = (tiles_m & 7) == 0 && (tiles_n & 3) == 0;
   // tile -> group, first row of the tile among all rows of A (m0), among the rows of the group (gm0), n0
-  struct Where { int g; int64_t m0; int gm0, n0; };
+  struct Where { int g; int64_t m0; int gm0, n0, valid; };  // valid: rows of the tile that exist (grouped: the last tile of a group)
   auto tile_where = [&](int t) {
     Where w;
     if constexpr (GROUPED) {
@@ -590,15 +599,18 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
         if (t < tile_prefix[mid]) hi = mid; else lo = mid;
       }
       w.g = __builtin_amdgcn_readfirstlane(lo);
-      const int full_m = __builtin_amdgcn_readfirstlane(p.problem_sizes[w.g * 3]) / BM;
+      const int m_g = __builtin_amdgcn_readfirstlane(p.problem_sizes[w.g * 3]);
+      const int64_t row_off = __builtin_amdgcn_readfirstlane(p.expert_offsets[w.g]);
+      const int full_m = rows_in_256_tiles(m_g, row_off, p.m) / BM;
       const int local = __builtin_amdgcn_readfirstlane(t - tile_prefix[w.g]);
       // bands of 4 m-tiles, n-major inside a band: 32 consecutive tiles share 4 A and 8 B panels
       const int band = local / (4 * tiles_n), in_band = local - band * 4 * tiles_n;
       const int band_h = min(4, full_m - 4 * band);
       const int nt = in_band / band_h, mt = 4 * band + (in_band - nt * band_h);
       w.gm0 = mt * BM;
-      w.m0 = (int64_t)__builtin_amdgcn_readfirstlane(p.expert_offsets[w.g]) + w.gm0;
+      w.m0 = row_off + w.gm0;
       w.n0 = nt * BN;
+      w.valid = min(BM, m_g - w.gm0);
     } else {
       int mt, nt;
       if (blocked) {
@@ -613,6 +625,7 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
       w.gm0 = mt * BM;
       w.m0 = w.gm0;
       w.n0 = nt * BN;
+      w.valid = BM;
     }
     return w;
   };
@@ -801,6 +814,7 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
       const int64_t at = (cw.m0 + wm * (32 * TM) + i * 32 + li) * p.n + cw.n0 + wn * 64 + lg * 4;
+      if (GROUPED && wm * (32 * TM) + i * 32 + li >= cw.valid) continue;
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
 #pragma unroll

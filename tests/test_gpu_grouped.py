@@ -187,13 +187,16 @@ def test_nvfp4_grouped_mm_empty_and_tiny_groups(dev):
 
 
 @pytest.mark.parametrize("sizes,n,k", [([600, 0, 256, 255, 1, 1030, 512], 512, 384), ([300, 2100, 0, 257], 256, 256),
-                                       ([2560, 700, 3000, 0, 1280, 2900], 2048, 256), ([511] * 5, 512, 640)])
+                                       ([2560, 700, 3000, 0, 1280, 2900], 2048, 256), ([511] * 5, 512, 640),
+                                       ([2248, 130, 400], 256, 384)])
 def test_nvfp4_grouped_mm_whole_tiles_and_group_ends(dev, sizes, n, k):
-    """At least 2048 rows, N % 256 == 0, K % 128 == 0: the whole 256-row tiles of every group run on the
-    persistent 256x256 kernel and the group ends on the 128x128 tile kernel.  Groups with no whole tile,
-    only whole tiles, one row past a tile, empty groups; two, three and five spans per tile; the third case
-    has 320 whole tiles, i.e. two per workgroup for some.  Every output element is compared; rows after the
-    last group stay untouched."""
+    """At least 2048 rows, N % 256 == 0, K % 128 == 0: the whole 256-row tiles of every group, and a last tile of
+    more than 128 rows, run on the persistent 256x256 kernel (which loads and computes the rows past such a
+    group and does not store them: the next group's rows, or the poisoned scale padding), the other group ends
+    on the 128x128 tile kernel.  Groups with no whole tile, only whole tiles, one row past a tile, 255 of 256
+    rows, empty groups; two, three and five spans per tile; the third case has more than 320 tiles, i.e. two
+    per workgroup for some; in the last case the final group's 144-row end would load past the activation
+    tensor as a 256-row tile and therefore stays with the tile kernel.  Every output element is compared."""
     from fuser_amd import nvf_cutlass
 
     g, m = len(sizes), sum(sizes) + 33
