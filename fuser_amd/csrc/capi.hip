@@ -25,6 +25,11 @@ int check_launch(const char* what) {
 }
 
 static bool dtype16(int d) { return d == NVF_BF16 || d == NVF_F16; }
+// The GEMM kernels move operands, scales and results in 16-byte pieces.
+template <typename... P>
+static bool aligned16(P... ptrs) { return ((reinterpret_cast<uintptr_t>(ptrs) | ...) & 15) == 0; }
+#define NVF_REQUIRE_ALIGNED16(...) \
+  NVF_REQUIRE(aligned16(__VA_ARGS__), NVF_ERR_INVALID_ARGUMENT, "operand, scale and output buffers must be 16-byte aligned")
 static bool dtype_in(int d) { return d == NVF_F32 || d == NVF_BF16 || d == NVF_F16; }
 
 }  // namespace nvf
@@ -155,6 +160,7 @@ int nvf_nvfp4_scaled_mm_ws(const void* a, const void* b, const void* scales_a, c
   NVF_REQUIRE(workspace_bytes >= 0, NVF_ERR_INVALID_ARGUMENT, "negative workspace size");
   if (m == 0 || n == 0) return NVF_OK;
   NVF_REQUIRE(a && b && scales_a && scales_b && alpha && out, NVF_ERR_INVALID_ARGUMENT, "NULL buffer");
+  NVF_REQUIRE_ALIGNED16(a, b, scales_a, scales_b, out);
   Gemm16Args g{a, b, scales_a, scales_b, alpha, out, nullptr, nullptr, nullptr, 1, m, n, k, out_dtype};
   if (workspace != nullptr && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0) {  // fp32x4 accesses
     g.workspace = workspace;
@@ -179,6 +185,7 @@ int nvf_nvfp4_scaled_mm_blockscale(const void* a, const void* b, const void* sca
   if (m == 0 || n == 0) return NVF_OK;
   NVF_REQUIRE(a && b && scales_a && scales_b && alpha && global_normconst && out_fp4 && out_scales && workspace,
               NVF_ERR_INVALID_ARGUMENT, "NULL buffer");
+  NVF_REQUIRE_ALIGNED16(a, b, scales_a, scales_b, out_fp4, out_scales, workspace);
   Gemm16Args g{a, b, scales_a, scales_b, alpha, workspace, nullptr, nullptr, nullptr, 1, m, n, k, NVF_F32};
   const int rc = launch_gemm16(0, g, static_cast<hipStream_t>(stream));
   if (rc != NVF_OK) return rc;
@@ -195,6 +202,7 @@ int nvf_mxfp8_scaled_mm(const void* a, const void* b, const void* scales_a, cons
   NVF_REQUIRE(k % 32 == 0, NVF_ERR_UNSUPPORTED_SHAPE, "The K dimension %lld is not a whole number of 32-element scale blocks", (long long)k);
   if (m == 0 || n == 0) return NVF_OK;
   NVF_REQUIRE(a && b && scales_a && scales_b && alpha && out, NVF_ERR_INVALID_ARGUMENT, "NULL buffer");
+  NVF_REQUIRE_ALIGNED16(a, b, scales_a, scales_b, out);
   return launch_mxfp8_gemm(a, b, scales_a, scales_b, alpha, out, m, n, k, out_dtype, static_cast<hipStream_t>(stream));
 }
 
@@ -206,6 +214,7 @@ int nvf_grouped_mm(const void* a, const void* b, void* out, const int32_t* probl
   NVF_REQUIRE(n % 8 == 0, NVF_ERR_UNSUPPORTED_SHAPE, "The inner dimension %lld of the output tensor is not a multiple of 8", (long long)n);
   if (m == 0 || n == 0 || groups == 0) return NVF_OK;
   NVF_REQUIRE(a && b && out && problem_sizes && expert_offsets, NVF_ERR_INVALID_ARGUMENT, "NULL buffer");
+  NVF_REQUIRE_ALIGNED16(a, b, out);
   Gemm16Args g{a, b, nullptr, nullptr, nullptr, out, problem_sizes, expert_offsets, nullptr, groups, m, n, k, ab_dtype};
   return launch_gemm16(2, g, static_cast<hipStream_t>(stream));
 }
@@ -222,6 +231,7 @@ int nvf_nvfp4_scaled_grouped_mm(const void* a, const void* b, const void* a_scal
   if (m == 0 || n == 0 || groups == 0) return NVF_OK;
   NVF_REQUIRE(a && b && a_scales && b_scales && alphas && out && problem_sizes && expert_offsets && sf_offsets,
               NVF_ERR_INVALID_ARGUMENT, "NULL buffer");
+  NVF_REQUIRE_ALIGNED16(a, b, a_scales, b_scales, out);
   Gemm16Args g{a, b, a_scales, b_scales, alphas, out, problem_sizes, expert_offsets, sf_offsets, groups, m, n, k, out_dtype};
   return launch_gemm16(1, g, static_cast<hipStream_t>(stream));
 }

@@ -122,6 +122,8 @@ NVF_API int nvf_cast_f32_to_e8m0(const float* in, int64_t n, uint8_t* out, void*
 /* ----------------------------------------------------------------------------------------------
  * GEMMs.  out_dtype / ab_dtype in {NVF_BF16, NVF_F16}.  B is always [N, K] with K contiguous
  * ("ColumnMajor" in the reference), so every op computes A * B^T with fp32 accumulation.
+ * Operand, scale, result and workspace buffers must be 16-byte aligned (NVF_ERR_INVALID_ARGUMENT
+ * otherwise; the reference's TMA descriptors need the same of its tensors).
  * -------------------------------------------------------------------------------------------- */
 
 /* cutlass/nvfp4_scaled_mm.cu:283-312 nvfp4_scaled_mm (shape rules: cutlass/nvf_cutlass.cpp:13-122).

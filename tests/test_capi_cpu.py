@@ -67,6 +67,13 @@ def test_invalid_arguments_are_rejected_without_a_device():
     assert lib.nvf_grouped_mm(p, p, p, p, p, 4, 128, 128, 64, capi.F32, None) == -1
     assert lib.nvf_nvfp4_scaled_grouped_mm(p, p, p, p, p, p, p, p, p, 4, 128, 128, 96, capi.BF16, None) == -2  # k % 64
     assert lib.nvf_nvfp4_scaled_grouped_mm(p, p, p, p, p, p, p, p, p, 2000, 128, 128, 128, capi.BF16, None) == -2  # groups
+    q = ctypes.c_void_p(24)  # 8-byte aligned only: the GEMMs move 16-byte pieces
+    assert lib.nvf_nvfp4_scaled_mm(q, p, p, p, p, p, 128, 128, 64, capi.BF16, None) == -1
+    assert b"16-byte aligned" in lib.nvf_last_error()
+    assert lib.nvf_mxfp8_scaled_mm(p, p, p, q, p, p, 128, 128, 64, capi.BF16, None) == -1
+    assert lib.nvf_grouped_mm(p, p, q, p, p, 4, 128, 128, 64, capi.BF16, None) == -1
+    assert lib.nvf_nvfp4_scaled_grouped_mm(p, q, p, p, p, p, p, p, p, 4, 128, 128, 128, capi.BF16, None) == -1
+    assert lib.nvf_nvfp4_scaled_mm_blockscale(p, p, p, p, p, p, p, q, p, 128, 128, 64, None) == -1
     assert lib.nvf_preprocess_grouped_matmul_input_sf(p, 3, 4, 4, p, p, 1, p, None) == -1
     assert lib.nvf_status_string(-2) == b"unsupported shape"
     with pytest.raises(capi.NvfError):
