@@ -314,6 +314,27 @@ def main():
                "gpu_vs_cpu_max_rel": round(err, 6)}
         del da, db, ref, got
 
+    # ------------------------------------------------------------------ the vendor library on the same payloads
+    # hipBLASLt through torch._scaled_mm: its MXFP8 kernel (unit e8m0 scales in its own layout: timing only) and its
+    # plain fp8 kernel with one scale per tensor.  A comparison figure for what the chip sustains on this data.
+    if not args.no_extra:
+        vendor = {}
+        try:
+            bt = qb.t()
+            u8 = torch.full((m, k // 32), 127, dtype=torch.uint8, device=dev).view(torch.float8_e8m0fnu)
+            v_ms, _ = timed(lambda: torch._scaled_mm(qa, bt, u8, u8, out_dtype=torch.bfloat16), args.steps, args.warmup)
+            vendor["hipblaslt_mxfp8_TFLOP/s"] = round(flops / v_ms / 1e9, 1)
+        except Exception as exc:  # not every build of the library has the block-scaled kernel
+            vendor["hipblaslt_mxfp8_TFLOP/s"] = None
+            vendor["hipblaslt_mxfp8_error"] = str(exc)[:120]
+        try:
+            v_ms, _ = timed(lambda: torch._scaled_mm(qa, qb.t(), one, one, out_dtype=torch.bfloat16), args.steps, args.warmup)
+            vendor["hipblaslt_fp8_per_tensor_scale_TFLOP/s"] = round(flops / v_ms / 1e9, 1)
+        except Exception as exc:
+            vendor["hipblaslt_fp8_per_tensor_scale_TFLOP/s"] = None
+            vendor["hipblaslt_fp8_error"] = str(exc)[:120]
+        extra["vendor_library_8192"] = vendor
+
     if not args.no_extra:
         for name in ("quant", "fused", "nvfp4", "llm", "grouped", "gnvfp4"):
             runners[name]()
