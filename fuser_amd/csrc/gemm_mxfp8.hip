@@ -233,7 +233,7 @@ __device__ __forceinline__ void lds_dma16(uint32_t lds_byte_addr, const uint8_t*
 // TM = 32-row accumulator tiles of a wavefront along M: 4 -> 256x256 workgroup tile, 2 -> 128x256 (for shapes
 // whose 256x256 tiles would leave compute units idle).  The statement order for TM = 4 is the one the 8192^3
 // measurements were made with.
-template <int TM, bool OUT_BF16>
+template <int TM, bool OUT_BF16, bool STREAM_OUT>
 __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) {
   constexpr int BM = 64 * TM, BN = 256;
   constexpr int A_UNITS = BM * 8;             // 16-byte units of the A tile (BM rows x 8 chunks)
@@ -449,12 +449,17 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
     }
     // ---- epilogue of this tile; the loads of the next tile's first two steps are already in flight.
     // acc[i][j][r] = C[m = li][n = (r/4)*8 + lg*4 + r%4] of its 32x32 sub-tile.
+    // A lane holds 8-byte pieces of 32 different rows; stored like that, a tile is 8192 sixteen-byte write
+    // requests per compute unit and the L2 takes longer over them than over a whole K step of MFMAs.  Each
+    // 32-row block of the wavefront's tile is therefore turned round in a private 8 KiB of LDS (16-byte chunk c
+    // of row r at chunk position c ^ (r & 15)) and leaves in 16-byte pieces, 16 lanes to a 256-byte row segment.
     int m0, n0;
     tile_coords(c_tile, m0, n0);
     uint16_t* out = static_cast<uint16_t*>(p.out);
+    u32x4* stage = lds + 2 * BUF_UNITS + wave * 512;
+    const int srow = lane >> 4, schunk = lane & 15;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-      uint16_t* orow = out + (int64_t)(m0 + wm * (32 * TM) + i * 32 + li) * p.n + n0 + wn * 128 + lg * 4;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
 #pragma unroll
@@ -462,9 +467,19 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
           u32x2 v;
           v[0] = pack2(acc[i][j][rq * 4 + 0] * alpha, acc[i][j][rq * 4 + 1] * alpha, OUT_BF16);
           v[1] = pack2(acc[i][j][rq * 4 + 2] * alpha, acc[i][j][rq * 4 + 3] * alpha, OUT_BF16);
-          *reinterpret_cast<u32x2*>(orow + j * 32 + rq * 8) = v;
+          reinterpret_cast<u32x2*>(stage)[(li * 16 + ((j * 4 + rq) ^ (li & 15))) * 2 + lg] = v;
         }
       }
+      asm volatile("" ::: "memory");  // the reads below see the writes above: one wavefront's LDS accesses stay in order
+      uint16_t* oblk = out + (int64_t)(m0 + wm * (32 * TM) + i * 32) * p.n + n0 + wn * 128 + schunk * 8;
+#pragma unroll
+      for (int t = 0; t < 8; ++t) {
+        const int row = 4 * t + srow;
+        const u32x4 v = stage[row * 16 + (schunk ^ (row & 15))];
+        if constexpr (STREAM_OUT) __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(oblk + (int64_t)row * p.n));
+        else *reinterpret_cast<u32x4*>(oblk + (int64_t)row * p.n) = v;
+      }
+      asm volatile("" ::: "memory");
     }
     zero_acc();
   }
@@ -472,10 +487,10 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
 #undef NVF_PIN_ACC
 }
 
-template <int TM, bool OUT_BF16>
-int launch_fast(const Params& p, hipStream_t stream) {
-  auto kern = mxfp8_gemm_256_kernel<TM, OUT_BF16>;
-  constexpr int lds_bytes = 2 * (64 * TM + 256) * 128;  // 128 KiB / 96 KiB
+template <int TM, bool OUT_BF16, bool STREAM_OUT>
+int launch_fast_cfg(const Params& p, hipStream_t stream) {
+  auto kern = mxfp8_gemm_256_kernel<TM, OUT_BF16, STREAM_OUT>;
+  constexpr int lds_bytes = 2 * (64 * TM + 256) * 128 + 4 * 8192;  // 128 KiB / 96 KiB of tiles + the epilogue's 32 KiB
   static uint64_t configured = 0;  // one bit per device; a benign race: the attribute call is idempotent
   if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
   const int64_t tiles = (int64_t)(p.m / (64 * TM)) * (p.n / 256);
@@ -483,6 +498,15 @@ int launch_fast(const Params& p, hipStream_t stream) {
   const unsigned grid = (unsigned)(tiles >= cus ? cus : ((tiles + 7) / 8) * 8);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_bytes, stream, p);
   return check_launch("mxfp8_gemm_256_kernel");
+}
+
+template <int TM, bool OUT_BF16>
+int launch_fast(const Params& p, hipStream_t stream) {
+  // Operands and result together beyond what the 256 MB last-level cache holds: the result would push the
+  // operand panels out of it (and out of the L2s) on its way to memory, so it leaves with non-temporal stores
+  // (8192^3: +5 %, 16384 x 16384 x 2048: +17 %; smaller problems lose 1-5 % that way).
+  const bool stream_out = ((int64_t)p.m + p.n) * p.k + 2 * (int64_t)p.m * p.n > (int64_t)224 << 20;
+  return stream_out ? launch_fast_cfg<TM, OUT_BF16, true>(p, stream) : launch_fast_cfg<TM, OUT_BF16, false>(p, stream);
 }
 
 // -------------------------------------------------------------------------------------------------
