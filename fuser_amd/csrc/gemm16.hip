@@ -638,22 +638,25 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   const int64_t row128 = (int64_t)128 * kbytes;       // payload distance of the thread's two rows
   const int64_t sfrow128 = (int64_t)128 * sf_padded;  // same for the scales (next 128-row tile)
 
-  // ---- operand stream: this thread's piece in the tile the stream is in (lp) and in the tile it enters
-  // next (np); it advances by selects only
+  // ---- operand stream: the tile the stream is in (lp) and the tile it enters next (np), as wave-uniform
+  // addresses of the tiles' first rows (scalar registers; they advance by scalar selects), and this thread's
+  // fixed 32-bit offsets inside any tile: its row and 16-byte piece, and its scale word (blocks 2*spiece,
+  // 2*spiece+1 of the span: 128x4 layout column tile spiece>>1, bytes 2*(spiece&1)..).  A tile's first row is
+  // a multiple of 128, so the swizzled scale address splits into the tile's part and the thread's part.
   struct RowPtrs { const uint8_t *a, *b, *sa, *sb; };
   auto tile_ptrs = [&](int t) {
     const Where w = tile_where(t);
     RowPtrs r;
-    r.a = p.a + (w.m0 + srow) * kbytes + spiece * 16;
-    r.b = p.b + ((int64_t)w.g * p.n + w.n0 + srow) * kbytes + spiece * 16;
-    // scale blocks 2*spiece, 2*spiece+1 of the span: 128x4 layout column tile spiece>>1, bytes 2*(spiece&1)..
+    r.a = p.a + w.m0 * kbytes;
+    r.b = p.b + ((int64_t)w.g * p.n + w.n0) * kbytes;
     // (a group's activation scales are a slab of their own, swizzled from its first row)
     const int64_t sa_slab = GROUPED ? (int64_t)__builtin_amdgcn_readfirstlane(p.sf_offsets[w.g]) * sf_padded : 0;
-    r.sa = p.sfa + sa_slab + swizzle_128x4(w.gm0 + srow, 0, sf_padded) + (spiece >> 1) * 512 + (spiece & 1) * 2;
-    r.sb = p.sfb + (int64_t)w.g * p.n * sf_padded + swizzle_128x4(w.n0 + srow, 0, sf_padded) + (spiece >> 1) * 512 +
-           (spiece & 1) * 2;
+    r.sa = p.sfa + sa_slab + swizzle_128x4(w.gm0, 0, sf_padded);
+    r.sb = p.sfb + (int64_t)w.g * p.n * sf_padded + swizzle_128x4(w.n0, 0, sf_padded);
     return r;
   };
+  const uint32_t off_ab = (uint32_t)srow * (uint32_t)kbytes + (uint32_t)spiece * 16u;
+  const uint32_t off_sf = (uint32_t)swizzle_128x4(srow, 0, sf_padded) + (uint32_t)(spiece >> 1) * 512u + (uint32_t)(spiece & 1) * 2u;
   RowPtrs lp = tile_ptrs(first_tile);
   RowPtrs np = lp;
   int l_mac = 0;
@@ -661,14 +664,14 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   // load unit q (0..7) of the span the stream is at; advance_stream() after the eighth
   auto issue_load_unit = [&](Raw& r, int q) {
     const int64_t o = (int64_t)l_mac * 64, so = (int64_t)l_mac * 1024;
-    if (q == 0) r.a[0] = *reinterpret_cast<const u32x4*>(lp.a + o);
-    if (q == 1 && AR == 2) r.a[1] = *reinterpret_cast<const u32x4*>(lp.a + o + row128);
-    if (q == 2) r.b[0] = *reinterpret_cast<const u32x4*>(lp.b + o);
-    if (q == 3) r.b[1] = *reinterpret_cast<const u32x4*>(lp.b + o + row128);
-    if (q == 4) r.sa[0] = *reinterpret_cast<const uint16_t*>(lp.sa + so);
-    if (q == 5 && AR == 2) r.sa[1] = *reinterpret_cast<const uint16_t*>(lp.sa + so + sfrow128);
-    if (q == 6) r.sb[0] = *reinterpret_cast<const uint16_t*>(lp.sb + so);
-    if (q == 7) r.sb[1] = *reinterpret_cast<const uint16_t*>(lp.sb + so + sfrow128);
+    if (q == 0) r.a[0] = *reinterpret_cast<const u32x4*>(lp.a + o + off_ab);
+    if (q == 1 && AR == 2) r.a[1] = *reinterpret_cast<const u32x4*>(lp.a + (o + row128) + off_ab);
+    if (q == 2) r.b[0] = *reinterpret_cast<const u32x4*>(lp.b + o + off_ab);
+    if (q == 3) r.b[1] = *reinterpret_cast<const u32x4*>(lp.b + (o + row128) + off_ab);
+    if (q == 4) r.sa[0] = *reinterpret_cast<const uint16_t*>(lp.sa + so + off_sf);
+    if (q == 5 && AR == 2) r.sa[1] = *reinterpret_cast<const uint16_t*>(lp.sa + (so + sfrow128) + off_sf);
+    if (q == 6) r.sb[0] = *reinterpret_cast<const uint16_t*>(lp.sb + so + off_sf);
+    if (q == 7) r.sb[1] = *reinterpret_cast<const uint16_t*>(lp.sb + (so + sfrow128) + off_sf);
   };
   auto advance_stream = [&]() {
     const bool wrap = (l_mac + 1 == nmac);
