@@ -814,24 +814,56 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
     // acc[i][j][r] = C[m = li][n = (r/4)*8 + lg*4 + r%4] of its 32x32 sub-tile.
     const Where cw = tile_where(c_tile);
     const float alpha = p.alpha[cw.g];
+    if constexpr (OUT_F32) {
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      const int64_t at = (cw.m0 + wm * (32 * TM) + i * 32 + li) * p.n + cw.n0 + wn * 64 + lg * 4;
-      if (GROUPED && wm * (32 * TM) + i * 32 + li >= cw.valid) continue;
+      for (int i = 0; i < TM; ++i) {
+        const int64_t at = (cw.m0 + wm * (32 * TM) + i * 32 + li) * p.n + cw.n0 + wn * 64 + lg * 4;
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
+        for (int j = 0; j < 2; ++j) {
 #pragma unroll
-        for (int rq = 0; rq < 4; ++rq) {
-          if constexpr (OUT_F32) {
+          for (int rq = 0; rq < 4; ++rq) {
             *reinterpret_cast<f32x4*>(static_cast<float*>(p.out) + at + j * 32 + rq * 8) =
                 f32x4{acc[i][j][rq * 4 + 0] * alpha, acc[i][j][rq * 4 + 1] * alpha, acc[i][j][rq * 4 + 2] * alpha,
                       acc[i][j][rq * 4 + 3] * alpha};
-          } else {
+          }
+        }
+      }
+    } else {
+      // A lane holds 8-byte pieces of 32 different rows; stored like that, a tile is 8192 sixteen-byte write
+      // requests per compute unit, which cost the L2 more time than a K step of MFMAs.  Every 32x32 block of the
+      // wavefront's tile is therefore turned round in a private 2.5 KiB of LDS (32 rows of 64 bytes at a pitch of
+      // 80 bytes) and leaves in 16-byte pieces, 4 lanes to a row's 64 bytes.  This kernel has no register to
+      // spare: one LDS address each for writing and reading (everything else is an immediate offset), one 32-bit
+      // lane offset into the result next to a wave-uniform address; and the lane number passes through an empty
+      // asm statement so that these are worked out here, after the K loop.
+      int elane = lane;
+      asm volatile("" : "+v"(elane));
+      uint8_t* stage = reinterpret_cast<uint8_t*>(lds + 2 * BUF_UNITS) + wave * 2560;
+      uint8_t* wr = stage + (elane & 31) * 80 + (elane >> 5) * 8;
+      const uint8_t* rd = stage + (elane >> 2) * 80 + (elane & 3) * 16;
+      const uint32_t ooff = ((uint32_t)(elane >> 2) * (uint32_t)p.n + (uint32_t)(elane & 3) * 8u) * 2u;
+      uint8_t* obase = reinterpret_cast<uint8_t*>(static_cast<uint16_t*>(p.out) + (cw.m0 + wm * (32 * TM)) * p.n + cw.n0 + wn * 64);
+      const int erow = elane >> 2;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+#pragma unroll
+          for (int rq = 0; rq < 4; ++rq) {
             u32x2 v;
             v[0] = pack2(acc[i][j][rq * 4 + 0] * alpha, acc[i][j][rq * 4 + 1] * alpha, OUT_BF16);
             v[1] = pack2(acc[i][j][rq * 4 + 2] * alpha, acc[i][j][rq * 4 + 3] * alpha, OUT_BF16);
-            *reinterpret_cast<u32x2*>(static_cast<uint16_t*>(p.out) + at + j * 32 + rq * 8) = v;
+            *reinterpret_cast<u32x2*>(wr + rq * 16) = v;
           }
+          asm volatile("" ::: "memory");  // the reads below see the writes above: one wavefront's LDS accesses stay in order
+#pragma unroll
+          for (int t = 0; t < 2; ++t) {
+            const int brow = i * 32 + 16 * t;  // first of the 16 rows of this piece, in the wavefront's tile
+            const u32x4 v = *reinterpret_cast<const u32x4*>(rd + t * 1280);
+            if (!GROUPED || wm * (32 * TM) + brow + erow < cw.valid)
+              *reinterpret_cast<u32x4*>(obase + ((int64_t)brow * p.n + j * 32) * 2 + ooff) = v;
+          }
+          asm volatile("" ::: "memory");
         }
       }
     }
@@ -843,7 +875,7 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
 template <bool OUT_BF16, bool GROUPED, int TM = 4, bool OUT_F32 = false>
 int launch_nvfp4_fast(const Params& p, int cus, hipStream_t stream) {
   auto kern = nvfp4_gemm_256_kernel<OUT_BF16, GROUPED, TM, OUT_F32>;
-  constexpr int lds_bytes = 2 * (64 * TM + 256) * 128;  // 128 KiB / 96 KiB
+  constexpr int lds_bytes = 2 * (64 * TM + 256) * 128 + (OUT_F32 ? 0 : 8 * 2560);  // 128 KiB / 96 KiB of tiles + the epilogue's 20 KiB
   static uint64_t configured = 0;  // one bit per device; a benign race: the attribute call is idempotent
   if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
   const int64_t tiles = (int64_t)(p.m / (64 * TM)) * (p.n / 256);  // grouped: an upper bound
