@@ -1426,22 +1426,42 @@ __global__ __launch_bounds__(256, 1) void grouped16_gemm_256_kernel(const Params
     }
     // ---- epilogue of this tile; the loads of the next tile's first two steps are already in flight.
     // acc[i][j][r] = C[m = li][n = (r/4)*8 + lg*4 + r%4] of its 32x32 sub-tile.
-    uint16_t* out = static_cast<uint16_t*>(p.out);
+    // A lane holds 8-byte pieces of 32 different rows; stored like that, a tile is 8192 sixteen-byte write
+    // requests per compute unit.  Every 32x64 block of the wavefront's tile is therefore turned round in a
+    // private 4.5 KiB of LDS (32 rows of 128 bytes at a pitch of 144 bytes) and leaves in 16-byte pieces, 8 lanes
+    // to a row's 128 bytes.  One LDS address each for writing and reading (the rest are immediate offsets) and
+    // one 32-bit lane offset next to a wave-uniform result address keep the epilogue out of the spill area.
+    int elane = lane;
+    asm volatile("" : "+v"(elane));
+    uint8_t* stage = reinterpret_cast<uint8_t*>(lds + 2 * BUF_UNITS) + wave * 4608;
+    uint8_t* wr = stage + (elane & 31) * 144 + (elane >> 5) * 8;
+    const uint8_t* rd = stage + (elane >> 3) * 144 + (elane & 7) * 16;
+    const uint32_t ooff = ((uint32_t)(elane >> 3) * (uint32_t)p.n + (uint32_t)(elane & 7) * 8u) * 2u;
+    uint8_t* obase = reinterpret_cast<uint8_t*>(static_cast<uint16_t*>(p.out) + (ct.out_row + wm * 128) * (int64_t)p.n + ct.n0 + wn * 128);
+    const int erow = wm * 128 + (elane >> 3);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int mrow = wm * 128 + i * 32 + li;
-      if (mrow < ct.valid) {
-        uint16_t* orow = out + (ct.out_row + mrow) * (int64_t)p.n + ct.n0 + wn * 128 + lg * 4;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+      for (int jh = 0; jh < 2; ++jh) {
+#pragma unroll
+        for (int j2 = 0; j2 < 2; ++j2) {
 #pragma unroll
           for (int rq = 0; rq < 4; ++rq) {
+            const int j = jh * 2 + j2;
             u32x2 v;
             v[0] = pack2(acc[i][j][rq * 4 + 0], acc[i][j][rq * 4 + 1], OUT_BF16);
             v[1] = pack2(acc[i][j][rq * 4 + 2], acc[i][j][rq * 4 + 3], OUT_BF16);
-            *reinterpret_cast<u32x2*>(orow + j * 32 + rq * 8) = v;
+            *reinterpret_cast<u32x2*>(wr + (j2 * 4 + rq) * 16) = v;
           }
         }
+        asm volatile("" ::: "memory");  // the reads below see the writes above: one wavefront's LDS accesses stay in order
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const int brow = i * 32 + 8 * t;  // first of the 8 rows of this piece, in the wavefront's tile
+          const u32x4 v = *reinterpret_cast<const u32x4*>(rd + t * 1152);
+          if (erow + brow < ct.valid) *reinterpret_cast<u32x4*>(obase + ((int64_t)brow * p.n + jh * 64) * 2 + ooff) = v;
+        }
+        asm volatile("" ::: "memory");
       }
     }
     zero_acc();
@@ -1454,7 +1474,7 @@ __global__ __launch_bounds__(256, 1) void grouped16_gemm_256_kernel(const Params
 template <bool BF16_MMA, bool OUT_BF16>
 int launch_grouped16_fast(const Params& p, int cus, hipStream_t stream) {
   auto kern = grouped16_gemm_256_kernel<BF16_MMA, OUT_BF16>;
-  constexpr int lds_bytes = 2 * 2 * 2048 * 16;  // 128 KiB
+  constexpr int lds_bytes = 2 * 2 * 2048 * 16 + 4 * 4608;  // 128 KiB of tiles + the epilogue's 18 KiB
   static uint64_t configured = 0;  // one bit per device; a benign race: the attribute call is idempotent
   if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
   hipLaunchKernelGGL(kern, dim3((unsigned)(cus & ~7)), dim3(256), lds_bytes, stream, p);
