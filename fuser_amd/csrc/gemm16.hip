@@ -1221,7 +1221,7 @@ int launch_nvfp4_skinny(const Params& p0, int cus, hipStream_t stream) {
 //     under the 32 MFMAs of the current one; one barrier per K step.
 // LDS layout as in the NVFP4 fast path: chunk c of row r at chunk position c ^ ((r >> 1) & 7).
 // -------------------------------------------------------------------------------------------------
-template <bool BF16_MMA, bool OUT_BF16>
+template <bool BF16_MMA, bool OUT_BF16, bool STREAM_OUT>
 __global__ __launch_bounds__(256, 1) void grouped16_gemm_256_kernel(const Params p) {
   constexpr int BM = 256, BN = 256;
   constexpr int TILE_UNITS = 2048;           // 16-byte units per operand tile (256 rows x 8 chunks)
@@ -1459,7 +1459,11 @@ __global__ __launch_bounds__(256, 1) void grouped16_gemm_256_kernel(const Params
         for (int t = 0; t < 4; ++t) {
           const int brow = i * 32 + 8 * t;  // first of the 8 rows of this piece, in the wavefront's tile
           const u32x4 v = *reinterpret_cast<const u32x4*>(rd + t * 1152);
-          if (erow + brow < ct.valid) *reinterpret_cast<u32x4*>(obase + ((int64_t)brow * p.n + jh * 64) * 2 + ooff) = v;
+          if (erow + brow < ct.valid) {
+            u32x4* dst = reinterpret_cast<u32x4*>(obase + ((int64_t)brow * p.n + jh * 64) * 2 + ooff);
+            if constexpr (STREAM_OUT) __builtin_nontemporal_store(v, dst);
+            else *dst = v;
+          }
         }
         asm volatile("" ::: "memory");
       }
@@ -1471,14 +1475,24 @@ __global__ __launch_bounds__(256, 1) void grouped16_gemm_256_kernel(const Params
 #undef NVF_PIN_ACC
 }
 
-template <bool BF16_MMA, bool OUT_BF16>
-int launch_grouped16_fast(const Params& p, int cus, hipStream_t stream) {
-  auto kern = grouped16_gemm_256_kernel<BF16_MMA, OUT_BF16>;
+template <bool BF16_MMA, bool OUT_BF16, bool STREAM_OUT>
+int launch_grouped16_fast_cfg(const Params& p, int cus, hipStream_t stream) {
+  auto kern = grouped16_gemm_256_kernel<BF16_MMA, OUT_BF16, STREAM_OUT>;
   constexpr int lds_bytes = 2 * 2 * 2048 * 16 + 4 * 4608;  // 128 KiB of tiles + the epilogue's 18 KiB
   static uint64_t configured = 0;  // one bit per device; a benign race: the attribute call is idempotent
   if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
   hipLaunchKernelGGL(kern, dim3((unsigned)(cus & ~7)), dim3(256), lds_bytes, stream, p);
   return check_launch("grouped16_gemm_256_kernel");
+}
+
+template <bool BF16_MMA, bool OUT_BF16>
+int launch_grouped16_fast(const Params& p, int cus, hipStream_t stream) {
+  // Operands and result together beyond what the 256 MB last-level cache holds: the result leaves with
+  // non-temporal stores, which keeps it from pushing operand panels out (single 8192-row group, 8192^3: +2.6 %,
+  // 16384 x 4096 x 4096: +7 %); smaller problems are better off with plain stores.
+  const int64_t bytes = 2 * ((int64_t)p.m * p.k + (int64_t)p.groups * p.n * p.k + (int64_t)p.m * p.n);
+  return bytes > ((int64_t)224 << 20) ? launch_grouped16_fast_cfg<BF16_MMA, OUT_BF16, true>(p, cus, stream)
+                                       : launch_grouped16_fast_cfg<BF16_MMA, OUT_BF16, false>(p, cus, stream);
 }
 
 template <int BM, int BN, bool BF16_MMA, bool OUT_BF16>
