@@ -450,36 +450,46 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
     // ---- epilogue of this tile; the loads of the next tile's first two steps are already in flight.
     // acc[i][j][r] = C[m = li][n = (r/4)*8 + lg*4 + r%4] of its 32x32 sub-tile.
     // A lane holds 8-byte pieces of 32 different rows; stored like that, a tile is 8192 sixteen-byte write
-    // requests per compute unit and the L2 takes longer over them than over a whole K step of MFMAs.  Each
-    // 32-row block of the wavefront's tile is therefore turned round in a private 8 KiB of LDS (16-byte chunk c
-    // of row r at chunk position c ^ (r & 15)) and leaves in 16-byte pieces, 16 lanes to a 256-byte row segment.
+    // requests per compute unit and the L2 takes longer over them than over a whole K step of MFMAs.  Every
+    // 32x64 block of the wavefront's tile is therefore turned round in a private 4.5 KiB of LDS (32 rows of 128
+    // bytes at a pitch of 144 bytes) and leaves in 16-byte pieces, 8 lanes to a row's 128 bytes.  One LDS address
+    // each for writing and reading (the rest are immediate offsets) and one 32-bit lane offset next to a
+    // wave-uniform result address; the lane number passes through an empty asm statement so that they are worked
+    // out here, after the K loop.
     int m0, n0;
     tile_coords(c_tile, m0, n0);
-    uint16_t* out = static_cast<uint16_t*>(p.out);
-    u32x4* stage = lds + 2 * BUF_UNITS + wave * 512;
-    const int srow = lane >> 4, schunk = lane & 15;
+    int elane = lane;
+    asm volatile("" : "+v"(elane));
+    uint8_t* stage = reinterpret_cast<uint8_t*>(lds + 2 * BUF_UNITS) + wave * 4608;
+    uint8_t* wr = stage + (elane & 31) * 144 + (elane >> 5) * 8;
+    const uint8_t* rd = stage + (elane >> 3) * 144 + (elane & 7) * 16;
+    const uint32_t ooff = ((uint32_t)(elane >> 3) * (uint32_t)p.n + (uint32_t)(elane & 7) * 8u) * 2u;
+    uint8_t* obase = reinterpret_cast<uint8_t*>(static_cast<uint16_t*>(p.out) + (int64_t)(m0 + wm * (32 * TM)) * p.n + n0 + wn * 128);
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+      for (int jh = 0; jh < 2; ++jh) {
 #pragma unroll
-        for (int rq = 0; rq < 4; ++rq) {
-          u32x2 v;
-          v[0] = pack2(acc[i][j][rq * 4 + 0] * alpha, acc[i][j][rq * 4 + 1] * alpha, OUT_BF16);
-          v[1] = pack2(acc[i][j][rq * 4 + 2] * alpha, acc[i][j][rq * 4 + 3] * alpha, OUT_BF16);
-          reinterpret_cast<u32x2*>(stage)[(li * 16 + ((j * 4 + rq) ^ (li & 15))) * 2 + lg] = v;
+        for (int j2 = 0; j2 < 2; ++j2) {
+#pragma unroll
+          for (int rq = 0; rq < 4; ++rq) {
+            const int j = jh * 2 + j2;
+            u32x2 v;
+            v[0] = pack2(acc[i][j][rq * 4 + 0] * alpha, acc[i][j][rq * 4 + 1] * alpha, OUT_BF16);
+            v[1] = pack2(acc[i][j][rq * 4 + 2] * alpha, acc[i][j][rq * 4 + 3] * alpha, OUT_BF16);
+            *reinterpret_cast<u32x2*>(wr + (j2 * 4 + rq) * 16) = v;
+          }
         }
-      }
-      asm volatile("" ::: "memory");  // the reads below see the writes above: one wavefront's LDS accesses stay in order
-      uint16_t* oblk = out + (int64_t)(m0 + wm * (32 * TM) + i * 32) * p.n + n0 + wn * 128 + schunk * 8;
+        asm volatile("" ::: "memory");  // the reads below see the writes above: one wavefront's LDS accesses stay in order
 #pragma unroll
-      for (int t = 0; t < 8; ++t) {
-        const int row = 4 * t + srow;
-        const u32x4 v = stage[row * 16 + (schunk ^ (row & 15))];
-        if constexpr (STREAM_OUT) __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(oblk + (int64_t)row * p.n));
-        else *reinterpret_cast<u32x4*>(oblk + (int64_t)row * p.n) = v;
+        for (int t = 0; t < 4; ++t) {
+          const u32x4 v = *reinterpret_cast<const u32x4*>(rd + t * 1152);
+          u32x4* dst = reinterpret_cast<u32x4*>(obase + ((int64_t)(i * 32 + 8 * t) * p.n + jh * 64) * 2 + ooff);
+          if constexpr (STREAM_OUT) __builtin_nontemporal_store(v, dst);
+          else *dst = v;
+        }
+        asm volatile("" ::: "memory");
       }
-      asm volatile("" ::: "memory");
     }
     zero_acc();
   }
@@ -490,7 +500,7 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
 template <int TM, bool OUT_BF16, bool STREAM_OUT>
 int launch_fast_cfg(const Params& p, hipStream_t stream) {
   auto kern = mxfp8_gemm_256_kernel<TM, OUT_BF16, STREAM_OUT>;
-  constexpr int lds_bytes = 2 * (64 * TM + 256) * 128 + 4 * 8192;  // 128 KiB / 96 KiB of tiles + the epilogue's 32 KiB
+  constexpr int lds_bytes = 2 * (64 * TM + 256) * 128 + 4 * 4608;  // 128 KiB / 96 KiB of tiles + the epilogue's 18 KiB
   static uint64_t configured = 0;  // one bit per device; a benign race: the attribute call is idempotent
   if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
   const int64_t tiles = (int64_t)(p.m / (64 * TM)) * (p.n / 256);
