@@ -30,6 +30,10 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--preheat-ms", type=float, default=300.0,
+                    help="before the warm-up steps of every measurement the same call is repeated for this long: the "
+                         "clocks of an idle GPU take some 100 ms of load to settle (0.43 ms per step right after idle, "
+                         "0.37 ms from then on)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg (profiling runs)")
     ap.add_argument("--no-extra", action="store_true", help="only the headline MXFP8 workload")
     ap.add_argument("--calib", action="store_true", help="profiling aid: also run a plain 1 GiB device copy a few times, "
@@ -57,6 +61,11 @@ def main():
 
     def timed(fn, steps, warmup):
         """Average milliseconds per call: HIP events on the launch stream around `steps` calls."""
+        t_end = time.perf_counter() + args.preheat_ms * 1e-3
+        while time.perf_counter() < t_end:  # steady clocks first; untimed, like the warm-up steps
+            for _ in range(8):
+                fn()
+            torch.cuda.synchronize()
         for _ in range(warmup):
             fn()
         torch.cuda.synchronize()
@@ -346,6 +355,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "preheat_ms": args.preheat_ms,
         "ms_per_step": round(ms, 5),
         "wall_ms_per_step": round(wall_ms, 5),
         "higher_is_better": True,
