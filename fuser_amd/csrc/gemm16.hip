@@ -815,17 +815,32 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
     const Where cw = tile_where(c_tile);
     const float alpha = p.alpha[cw.g];
     if constexpr (OUT_F32) {
+      // as below, with 32x16 blocks of fp32 (64-byte row segments)
+      int elane = lane;
+      asm volatile("" : "+v"(elane));
+      uint8_t* stage = reinterpret_cast<uint8_t*>(lds + 2 * BUF_UNITS) + wave * 2560;
+      uint8_t* wr = stage + (elane & 31) * 80 + (elane >> 5) * 16;
+      const uint8_t* rd = stage + (elane >> 2) * 80 + (elane & 3) * 16;
+      const uint32_t ooff = ((uint32_t)(elane >> 2) * (uint32_t)p.n + (uint32_t)(elane & 3) * 4u) * 4u;
+      uint8_t* obase = reinterpret_cast<uint8_t*>(static_cast<float*>(p.out) + (cw.m0 + wm * (32 * TM)) * p.n + cw.n0 + wn * 64);
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
-        const int64_t at = (cw.m0 + wm * (32 * TM) + i * 32 + li) * p.n + cw.n0 + wn * 64 + lg * 4;
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
+        for (int jh = 0; jh < 4; ++jh) {  // 16 columns: block j = jh / 2, its rq pair jh % 2
+          const int j = jh >> 1;
 #pragma unroll
-          for (int rq = 0; rq < 4; ++rq) {
-            *reinterpret_cast<f32x4*>(static_cast<float*>(p.out) + at + j * 32 + rq * 8) =
-                f32x4{acc[i][j][rq * 4 + 0] * alpha, acc[i][j][rq * 4 + 1] * alpha, acc[i][j][rq * 4 + 2] * alpha,
-                      acc[i][j][rq * 4 + 3] * alpha};
+          for (int r2 = 0; r2 < 2; ++r2) {
+            const int rq = (jh & 1) * 2 + r2;
+            *reinterpret_cast<f32x4*>(wr + r2 * 32) = f32x4{acc[i][j][rq * 4 + 0] * alpha, acc[i][j][rq * 4 + 1] * alpha,
+                                                            acc[i][j][rq * 4 + 2] * alpha, acc[i][j][rq * 4 + 3] * alpha};
           }
+          asm volatile("" ::: "memory");  // one wavefront's LDS accesses stay in order
+#pragma unroll
+          for (int t = 0; t < 2; ++t) {
+            const f32x4 v = *reinterpret_cast<const f32x4*>(rd + t * 1280);
+            *reinterpret_cast<f32x4*>(obase + ((int64_t)(i * 32 + 16 * t) * p.n + jh * 16) * 4 + ooff) = v;
+          }
+          asm volatile("" ::: "memory");
         }
       }
     } else {
@@ -875,7 +890,7 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
 template <bool OUT_BF16, bool GROUPED, int TM = 4, bool OUT_F32 = false>
 int launch_nvfp4_fast(const Params& p, int cus, hipStream_t stream) {
   auto kern = nvfp4_gemm_256_kernel<OUT_BF16, GROUPED, TM, OUT_F32>;
-  constexpr int lds_bytes = 2 * (64 * TM + 256) * 128 + (OUT_F32 ? 0 : 8 * 2560);  // 128 KiB / 96 KiB of tiles + the epilogue's 20 KiB
+  constexpr int lds_bytes = 2 * (64 * TM + 256) * 128 + 8 * 2560;  // 128 KiB / 96 KiB of tiles + the epilogue's 20 KiB
   static uint64_t configured = 0;  // one bit per device; a benign race: the attribute call is idempotent
   if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
   const int64_t tiles = (int64_t)(p.m / (64 * TM)) * (p.n / 256);  // grouped: an upper bound
