@@ -535,7 +535,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
 // TM = 32-row accumulator tiles of a wavefront along M: 4 -> 256x256 workgroup tile, 2 -> 128x256 (dense shapes
 // whose 256x256 tiles would leave compute units idle; 1.5 times the conversion work per MFMA).  The statement
 // order for TM = 4 is the one the 8192^3 measurements were made with.
-template <bool OUT_BF16, bool GROUPED, int TM = 4, bool OUT_F32 = false>
+template <bool OUT_BF16, bool GROUPED, int TM = 4, bool OUT_F32 = false, bool PAIRS = false>
 __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   static_assert(TM == 4 || (TM == 2 && !GROUPED), "tile height");
   constexpr int BM = 64 * TM, BN = 256;
@@ -769,43 +769,87 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
 #pragma unroll
   for (int q = 0; q < NFU; ++q) load_frag_unit(0, 0, q, fr[0]);
 
+  // The two in-flight spans (`cur`: its odd step is converted next, `nxt`: its even step) normally hand over by a
+  // register copy at the end of every span.  With an even number of spans per tile (PAIRS) the loop body is
+  // written for two spans with the names swapped in the second, which saves the 24 register-pair moves per span.
+  auto span_no_copy = [&](Raw& odd_src, Raw& even_src) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        if (kk == 3) {
+          NVF_PIN_ACC();
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+          __builtin_amdgcn_s_barrier();
+          asm volatile("" ::: "memory");
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int q = 0; q < NMK; ++q) {
+          const int i = q >> 1, j = q & 1;
+          const int slot_id = kk * NMK + q;
+          if (q < NFU) load_frag_unit(kk < 3 ? h : (h ^ 1), (kk + 1) & 3, q, fr[(kk + 1) & 1]);
+          if (kk < 3) {
+#pragma unroll
+            for (int part = slot_id * NCU / NMK; part < (slot_id + 1) * NCU / NMK; ++part)
+              convert_phase(h ? even_src : odd_src, h ^ 1, unit_of(part / 3), part % 3, h ^ 1);
+          }
+          if (kk == 3 && h == 1) {  // odd_src is dead: it takes the span after even_src
+#pragma unroll
+            for (int l = q * 8 / NMK; l < (q + 1) * 8 / NMK; ++l) issue_load_unit(odd_src, l);
+            if (q == NMK - 1) advance_stream();
+          }
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, fr[kk & 1].b[j]),
+                                                             __builtin_bit_cast(f16x8, fr[kk & 1].a[i]), acc[i][j], 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    }
+  };
   for (int c_tile = first_tile; c_tile < range_end; c_tile += slots) {
     np = ptrs_or_current(c_tile + tiles_ahead * slots);
-    for (int c_mac = 0; c_mac < nmac; ++c_mac) {
+    if constexpr (PAIRS) {
+      for (int c_mac = 0; c_mac < nmac; c_mac += 2) {
+        span_no_copy(cur, nxt);
+        span_no_copy(nxt, cur);
+      }
+    } else {
+      for (int c_mac = 0; c_mac < nmac; ++c_mac) {
 #pragma unroll
-      for (int h = 0; h < 2; ++h) {  // step g = 2*c_mac + h computes from LDS buffer h
-        // h == 0: the odd step of the current span is converted into buffer 1
-        // h == 1: the even step of the next span is converted into buffer 0; then that span becomes the
-        //         current one and the span after it is requested
+        for (int h = 0; h < 2; ++h) {  // step g = 2*c_mac + h computes from LDS buffer h
+          // h == 0: the odd step of the current span is converted into buffer 1
+          // h == 1: the even step of the next span is converted into buffer 0; then that span becomes the
+          //         current one and the span after it is requested
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
-          if (kk == 3) {
-            // every wave has written its share of step g+1 and read the last fragments of step g
-            NVF_PIN_ACC();
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            __builtin_amdgcn_s_barrier();
-            asm volatile("" ::: "memory");
-            if (h == 1) cur = nxt;
-          }
-          __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-          for (int q = 0; q < NMK; ++q) {
-            const int i = q >> 1, j = q & 1;
-            const int slot_id = kk * NMK + q;  // 3 * NMK slots for the 3 * NCU conversion parts of the step
-            if (q < NFU) load_frag_unit(kk < 3 ? h : (h ^ 1), (kk + 1) & 3, q, fr[(kk + 1) & 1]);
-            if (kk < 3) {
-#pragma unroll
-              for (int part = slot_id * NCU / NMK; part < (slot_id + 1) * NCU / NMK; ++part)
-                convert_phase(h ? nxt : cur, h ^ 1, unit_of(part / 3), part % 3, h ^ 1);
+          for (int kk = 0; kk < 4; ++kk) {
+            if (kk == 3) {
+              // every wave has written its share of step g+1 and read the last fragments of step g
+              NVF_PIN_ACC();
+              asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+              __builtin_amdgcn_s_barrier();
+              asm volatile("" ::: "memory");
+              if (h == 1) cur = nxt;
             }
-            if (kk == 3 && h == 1) {
-#pragma unroll
-              for (int l = q * 8 / NMK; l < (q + 1) * 8 / NMK; ++l) issue_load_unit(nxt, l);
-              if (q == NMK - 1) advance_stream();
-            }
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, fr[kk & 1].b[j]),
-                                                               __builtin_bit_cast(f16x8, fr[kk & 1].a[i]), acc[i][j], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int q = 0; q < NMK; ++q) {
+              const int i = q >> 1, j = q & 1;
+              const int slot_id = kk * NMK + q;  // 3 * NMK slots for the 3 * NCU conversion parts of the step
+              if (q < NFU) load_frag_unit(kk < 3 ? h : (h ^ 1), (kk + 1) & 3, q, fr[(kk + 1) & 1]);
+              if (kk < 3) {
+#pragma unroll
+                for (int part = slot_id * NCU / NMK; part < (slot_id + 1) * NCU / NMK; ++part)
+                  convert_phase(h ? nxt : cur, h ^ 1, unit_of(part / 3), part % 3, h ^ 1);
+              }
+              if (kk == 3 && h == 1) {
+#pragma unroll
+                for (int l = q * 8 / NMK; l < (q + 1) * 8 / NMK; ++l) issue_load_unit(nxt, l);
+                if (q == NMK - 1) advance_stream();
+              }
+              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, fr[kk & 1].b[j]),
+                                                                 __builtin_bit_cast(f16x8, fr[kk & 1].a[i]), acc[i][j], 0, 0, 0);
+              __builtin_amdgcn_sched_barrier(0);
+            }
           }
         }
       }
@@ -887,9 +931,9 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
 #undef NVF_PIN_ACC
 }
 
-template <bool OUT_BF16, bool GROUPED, int TM = 4, bool OUT_F32 = false>
-int launch_nvfp4_fast(const Params& p, int cus, hipStream_t stream) {
-  auto kern = nvfp4_gemm_256_kernel<OUT_BF16, GROUPED, TM, OUT_F32>;
+template <bool OUT_BF16, bool GROUPED, int TM, bool OUT_F32, bool PAIRS>
+int launch_nvfp4_fast_cfg(const Params& p, int cus, hipStream_t stream) {
+  auto kern = nvfp4_gemm_256_kernel<OUT_BF16, GROUPED, TM, OUT_F32, PAIRS>;
   constexpr int lds_bytes = 2 * (64 * TM + 256) * 128 + 8 * 2560;  // 128 KiB / 96 KiB of tiles + the epilogue's 20 KiB
   static uint64_t configured = 0;  // one bit per device; a benign race: the attribute call is idempotent
   if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
@@ -897,6 +941,15 @@ int launch_nvfp4_fast(const Params& p, int cus, hipStream_t stream) {
   const unsigned grid = (unsigned)(tiles >= cus ? (cus & ~7) : ((tiles + 7) / 8) * 8);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds_bytes, stream, p);
   return check_launch("nvfp4_gemm_256_kernel");
+}
+
+template <bool OUT_BF16, bool GROUPED, int TM = 4, bool OUT_F32 = false>
+int launch_nvfp4_fast(const Params& p, int cus, hipStream_t stream) {
+  // an even number of 128-deep spans per tile: the variant whose two in-flight spans swap names instead of being copied
+  if constexpr (TM == 4) {
+    if (((p.k >> 7) & 1) == 0) return launch_nvfp4_fast_cfg<OUT_BF16, GROUPED, TM, OUT_F32, true>(p, cus, stream);
+  }
+  return launch_nvfp4_fast_cfg<OUT_BF16, GROUPED, TM, OUT_F32, false>(p, cus, stream);
 }
 
 // -------------------------------------------------------------------------------------------------
