@@ -946,9 +946,7 @@ int launch_nvfp4_fast_cfg(const Params& p, int cus, hipStream_t stream) {
 template <bool OUT_BF16, bool GROUPED, int TM = 4, bool OUT_F32 = false>
 int launch_nvfp4_fast(const Params& p, int cus, hipStream_t stream) {
   // an even number of 128-deep spans per tile: the variant whose two in-flight spans swap names instead of being copied
-  if constexpr (TM == 4) {
-    if (((p.k >> 7) & 1) == 0) return launch_nvfp4_fast_cfg<OUT_BF16, GROUPED, TM, OUT_F32, true>(p, cus, stream);
-  }
+  if (((p.k >> 7) & 1) == 0) return launch_nvfp4_fast_cfg<OUT_BF16, GROUPED, TM, OUT_F32, true>(p, cus, stream);
   return launch_nvfp4_fast_cfg<OUT_BF16, GROUPED, TM, OUT_F32, false>(p, cus, stream);
 }
 
