@@ -1639,11 +1639,11 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int6
       return launch_nvfp4_skinny<OUT_BF16>(p, cus, stream);
     if (dense && (p.m & 127) == 0 && (p.n & 255) == 0 && (p.k & 127) == 0 && p.k >= 256) {
       // Persistent kernel with 256x256 or 128x256 tiles, or the tile kernel below?  Costs in units of one round
-      // of 256x256 tiles over the compute units = 100: a 128-row tile costs 62 (half the flops at 81 % of the
+      // of 256x256 tiles over the compute units = 100: a 128-row tile costs 58 (half the flops at 86 % of the
       // rate), and the tile kernel, which has no rounds to speak of, runs at about 70 % of the rate (all measured).
       const int64_t t256 = (p.m & 255) == 0 ? tiles(256, 256) : 0, t128 = tiles(128, 256);
       const int64_t cost256 = t256 ? 100 * ceil_div(t256, cus) : INT64_MAX;
-      const int64_t cost128 = 62 * ceil_div(t128, cus);
+      const int64_t cost128 = 58 * ceil_div(t128, cus);
       const int64_t cost_tile = 144 * t128 / (2 * cus);
       if (cost256 <= cost128 && cost256 <= cost_tile) return launch_nvfp4_fast<OUT_BF16, false, 4>(p, cus, stream);
       if (cost128 <= cost_tile) return launch_nvfp4_fast<OUT_BF16, false, 2>(p, cus, stream);
