@@ -447,16 +447,30 @@ __global__ __launch_bounds__(256) void nvfp4_tile_kernel(const Params p) {
     issue_span(cur, span0);
     convert(cur, 0, 0);  // every wave is past the barrier that ended the previous tile's last step
     __syncthreads();
-    for (int sp = span0; sp < span1; ++sp) {
+    // one span: `c` holds it (its even step is in buffer 0 already), `n` takes the span after it; with the larger
+    // tiles the two register sets swap names from span to span, so no span is copied
+    auto one_span = [&](Raw& c, Raw& n, int sp) {
       const bool more = sp + 1 < span1;
-      if (more) issue_span(nxt, sp + 1);
+      if (more) issue_span(n, sp + 1);
       mfma_step(0);
-      convert(cur, 1, 1);
+      convert(c, 1, 1);
       __syncthreads();
       mfma_step(1);
-      if (more) convert(nxt, 0, 0);
+      if (more) convert(n, 0, 0);
       __syncthreads();
-      cur = nxt;
+    };
+    if constexpr (BM >= 128 && !SPLIT_K) {
+      int sp = span0;
+      for (; sp + 1 < span1; sp += 2) {
+        one_span(cur, nxt, sp);
+        one_span(nxt, cur, sp + 1);
+      }
+      if (sp < span1) one_span(cur, nxt, sp);
+    } else {  // (small tiles and short K ranges: measured slower with the doubled loop body)
+      for (int sp = span0; sp < span1; ++sp) {
+        one_span(cur, nxt, sp);
+        cur = nxt;
+      }
     }
 
     // ---- epilogue: acc[i][j][r] = C[m = lane%32][n = (r/4)*8 + (lane/32)*4 + r%4] of its 32x32 tile ----
