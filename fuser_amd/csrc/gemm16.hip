@@ -1246,7 +1246,10 @@ int launch_nvfp4_skinny_ring_cfg(const Params& p, hipStream_t stream) {
 template <int RT, int TT, bool OUT_BF16, bool NSPLIT>
 int launch_nvfp4_skinny_grouped(const Params& p0, int rows_lo, int rows_hi, hipStream_t stream) {
   constexpr int SLOT_KIB = RT + TT + (RT + 1) / 2 + (TT + 1) / 2;
-  constexpr int DEPTH = 8 * 2 * SLOT_KIB <= 160 ? 2 : 1;
+  // One slot per wavefront also where two would fit: measured faster for the groups of up to 32 rows (512 rows
+  // over 256 experts, K=7168: 401 -> 375 us; K=2048: 432 -> 413 us).  Forcing the registers down to two
+  // workgroups per compute unit on top of that costs more than it gains (450 us).
+  constexpr int DEPTH = 1;
   auto kern = nvfp4_skinny_ring_kernel<RT, TT, OUT_BF16, DEPTH, true, NSPLIT>;
   constexpr int red_kib = NSPLIT ? 0 : 8 * (RT * TT <= 8 ? RT * TT : TT);
   constexpr int ring_kib = 8 * DEPTH * SLOT_KIB;
