@@ -1230,7 +1230,8 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
 template <int RT, int TT, bool OUT_BF16>
 int launch_nvfp4_skinny_ring_cfg(const Params& p, hipStream_t stream) {
   constexpr int SLOT_KIB = RT + TT + (RT + 1) / 2 + (TT + 1) / 2;
-  constexpr int DEPTH = 8 * 2 * SLOT_KIB <= 160 ? 2 : 1;
+  // one slot per wavefront also where two would fit (M=16, N=14336, K=4096: 8.0 -> 7.5 us; K=14336: 9.6 -> 9.2 us)
+  constexpr int DEPTH = 1;
   auto kern = nvfp4_skinny_ring_kernel<RT, TT, OUT_BF16, DEPTH>;
   // the ring; the reduction reuses it and needs 8 KiB per partial tile of a round
   constexpr int red_kib = 8 * (RT * TT <= 8 ? RT * TT : TT);
