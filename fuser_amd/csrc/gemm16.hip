@@ -676,16 +676,21 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   int l_mac = 0;
   struct Raw { u32x4 a[2], b[2]; uint32_t sa[2], sb[2]; };
   // load unit q (0..7) of the span the stream is at; advance_stream() after the eighth
+  // Buffer loads: the tile's first row as the resource's base, the span and the second row as the scalar
+  // offset, the thread's fixed offset as the vector offset, so that no address is worked out in vector registers.
+  auto rsrc = [](const uint8_t* base) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(base), 0, 0x7fffffff, 0x00020000);
+  };
   auto issue_load_unit = [&](Raw& r, int q) {
-    const int64_t o = (int64_t)l_mac * 64, so = (int64_t)l_mac * 1024;
-    if (q == 0) r.a[0] = *reinterpret_cast<const u32x4*>(lp.a + o + off_ab);
-    if (q == 1 && AR == 2) r.a[1] = *reinterpret_cast<const u32x4*>(lp.a + (o + row128) + off_ab);
-    if (q == 2) r.b[0] = *reinterpret_cast<const u32x4*>(lp.b + o + off_ab);
-    if (q == 3) r.b[1] = *reinterpret_cast<const u32x4*>(lp.b + (o + row128) + off_ab);
-    if (q == 4) r.sa[0] = *reinterpret_cast<const uint16_t*>(lp.sa + so + off_sf);
-    if (q == 5 && AR == 2) r.sa[1] = *reinterpret_cast<const uint16_t*>(lp.sa + (so + sfrow128) + off_sf);
-    if (q == 6) r.sb[0] = *reinterpret_cast<const uint16_t*>(lp.sb + so + off_sf);
-    if (q == 7) r.sb[1] = *reinterpret_cast<const uint16_t*>(lp.sb + (so + sfrow128) + off_sf);
+    const int o = l_mac * 64, so = l_mac * 1024;
+    if (q == 0) r.a[0] = __builtin_amdgcn_raw_buffer_load_b128(rsrc(lp.a), off_ab, o, 0);
+    if (q == 1 && AR == 2) r.a[1] = __builtin_amdgcn_raw_buffer_load_b128(rsrc(lp.a), off_ab, o + (int)row128, 0);
+    if (q == 2) r.b[0] = __builtin_amdgcn_raw_buffer_load_b128(rsrc(lp.b), off_ab, o, 0);
+    if (q == 3) r.b[1] = __builtin_amdgcn_raw_buffer_load_b128(rsrc(lp.b), off_ab, o + (int)row128, 0);
+    if (q == 4) r.sa[0] = __builtin_amdgcn_raw_buffer_load_b16(rsrc(lp.sa), off_sf, so, 0);
+    if (q == 5 && AR == 2) r.sa[1] = __builtin_amdgcn_raw_buffer_load_b16(rsrc(lp.sa), off_sf, so + (int)sfrow128, 0);
+    if (q == 6) r.sb[0] = __builtin_amdgcn_raw_buffer_load_b16(rsrc(lp.sb), off_sf, so, 0);
+    if (q == 7) r.sb[1] = __builtin_amdgcn_raw_buffer_load_b16(rsrc(lp.sb), off_sf, so + (int)sfrow128, 0);
   };
   auto advance_stream = [&]() {
     const bool wrap = (l_mac + 1 == nmac);
