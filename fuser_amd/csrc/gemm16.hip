@@ -1756,6 +1756,8 @@ int cu_count() {
 int launch_gemm16(int op, const Gemm16Args& a, hipStream_t stream) {
   if (a.groups > kMaxGroups) return fail(NVF_ERR_UNSUPPORTED_SHAPE, "at most %d groups are supported, got %d", kMaxGroups, a.groups);
   if (a.m > INT32_MAX || a.n > INT32_MAX || a.k > INT32_MAX) return fail(NVF_ERR_UNSUPPORTED_SHAPE, "dimension exceeds int32");
+  // (the kernels address a tile's 256 rows with 32-bit byte offsets)
+  if (a.k >= (1 << 22)) return fail(NVF_ERR_UNSUPPORTED_SHAPE, "K = %lld: at most 4194303 is supported", (long long)a.k);
   Params p;
   p.a = static_cast<const uint8_t*>(a.a);
   p.b = static_cast<const uint8_t*>(a.b);
