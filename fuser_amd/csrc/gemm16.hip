@@ -543,8 +543,8 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
 //     in phase and a long run of other instructions in both would idle the matrix pipe.
 //   * One barrier per step, placed before the last quarter of its MFMAs: by then every wave has written
 //     its share of the next step and holds this step's last fragments in registers.
-// LDS: two buffers of (A tile + B tile), each tile 256 rows x 128 bytes with 16-byte chunk c of row r at
-// chunk position c ^ ((r >> 1) & 7): conflict-free for the fragment reads.
+// LDS: two buffers of an A tile and a B tile (stored A0, A1, B0, B1), each tile 256 rows x 128 bytes with 16-byte
+// chunk c of row r at chunk position c ^ ((r >> 1) & 7): conflict-free for the fragment reads.
 // -------------------------------------------------------------------------------------------------
 // TM = 32-row accumulator tiles of a wavefront along M: 4 -> 256x256 workgroup tile, 2 -> 128x256 (dense shapes
 // whose 256x256 tiles would leave compute units idle; 1.5 times the conversion work per MFMA).  The statement
@@ -556,6 +556,10 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   constexpr int A_UNITS = BM * 8;            // 16-byte units of the A tile (fp16, 64 of K per row)
   constexpr int TILE_UNITS = 2048;           // ... of the B tile
   constexpr int BUF_UNITS = A_UNITS + TILE_UNITS;
+  // LDS order: A tile of buffer 0, A tile of buffer 1, B tile of buffer 0, B tile of buffer 1.  The two buffers of an
+  // operand are then less than 64 KiB apart, so that a lane's fragment address for (operand, sub-step) serves both
+  // buffers and all row tiles through the 16-bit immediate offset of the LDS instructions.
+  auto tile_units = [](int buf, int op) { return op ? 2 * A_UNITS + buf * TILE_UNITS : buf * A_UNITS; };
   constexpr int AR = TM / 2;                 // A rows a thread stages per span (rows srow + 128 i)
   constexpr int NMK = 2 * TM;                // MFMAs per 16-deep sub-step
   constexpr int NCU = 2 * AR + 4;            // conversion units per step: operand, row, half scale block
@@ -726,7 +730,7 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
     } else {
       ch[2] = ch[2] * sv[op][i];
       ch[3] = ch[3] * sv[op][i];
-      lds[wbuf * BUF_UNITS + op * A_UNITS + lds_pos2(srow + 128 * i, spiece * 2 + cc)] =
+      lds[tile_units(wbuf, op) + lds_pos2(srow + 128 * i, spiece * 2 + cc)] =
           u32x4{__builtin_bit_cast(uint32_t, ch[0]), __builtin_bit_cast(uint32_t, ch[1]), __builtin_bit_cast(uint32_t, ch[2]),
                 __builtin_bit_cast(uint32_t, ch[3])};
     }
@@ -739,7 +743,7 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
     const int op = (q == 1 || q == 2) ? 1 : 0;
     const int t = op ? q - 1 : (q == 0 ? 0 : q - 2);
     const int row = (op ? wn * 64 : wm * (32 * TM)) + t * 32 + li;
-    const u32x4 v = lds[buf * BUF_UNITS + op * A_UNITS + lds_pos2(row, kk * 2 + lg)];
+    const u32x4 v = lds[tile_units(buf, op) + lds_pos2(row, kk * 2 + lg)];
     if (op) f.b[t] = v; else f.a[t] = v;
   };
 
