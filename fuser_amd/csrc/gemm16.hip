@@ -551,7 +551,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
 // order for TM = 4 is the one the 8192^3 measurements were made with.
 template <bool OUT_BF16, bool GROUPED, int TM = 4, bool OUT_F32 = false, bool PAIRS = false>
 __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
-  static_assert(TM == 4 || (TM == 2 && !GROUPED), "tile height");
+  static_assert(TM == 4 || TM == 2, "tile height");
   constexpr int BM = 64 * TM, BN = 256;
   constexpr int A_UNITS = BM * 8;            // 16-byte units of the A tile (fp16, 64 of K per row)
   constexpr int TILE_UNITS = 2048;           // ... of the B tile
@@ -579,7 +579,8 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   // at a time share 8 A panels and 4 B panels in its L2.
   // GROUPED: the work list holds the 256-row tiles of every group that rows_in_256_tiles() names: the whole
   // ones and a last one of more than 128 rows, whose rows past the group are computed and not stored; what
-  // is left at the end of a group goes to the tile kernel.
+  // is left at the end of a group goes to the tile kernel.  With 128-row tiles (TM == 2) the list is instead one
+  // tile per weight panel for every group of rows_lo..rows_hi (<= 128) rows.
   const int tiles_m = p.m / BM, tiles_n = p.n / BN;
   int total = tiles_m * tiles_n;
   if constexpr (GROUPED) {
@@ -587,7 +588,12 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
       int running = 0;
       for (int base = 0; base < p.groups; base += 64) {
         const int g = base + lane;
-        const int cnt = g < p.groups ? (rows_in_256_tiles(p.problem_sizes[g * 3], p.expert_offsets[g], p.m) / BM) * tiles_n : 0;
+        int cnt = 0;
+        if (g < p.groups) {
+          const int mg = p.problem_sizes[g * 3];
+          if constexpr (TM == 4) cnt = (rows_in_256_tiles(mg, p.expert_offsets[g], p.m) / BM) * tiles_n;
+          else cnt = (mg >= p.rows_lo && mg <= p.rows_hi) ? tiles_n : 0;  // one 128-row tile per group of the class and weight panel
+        }
         int incl = cnt;
 #pragma unroll
         for (int d = 1; d < 64; d <<= 1) {
@@ -619,7 +625,7 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
       w.g = __builtin_amdgcn_readfirstlane(lo);
       const int m_g = __builtin_amdgcn_readfirstlane(p.problem_sizes[w.g * 3]);
       const int64_t row_off = __builtin_amdgcn_readfirstlane(p.expert_offsets[w.g]);
-      const int full_m = rows_in_256_tiles(m_g, row_off, p.m) / BM;
+      const int full_m = TM == 4 ? rows_in_256_tiles(m_g, row_off, p.m) / BM : 1;
       const int local = __builtin_amdgcn_readfirstlane(t - tile_prefix[w.g]);
       // bands of 4 m-tiles, n-major inside a band: 32 consecutive tiles share 4 A and 8 B panels
       const int band = local / (4 * tiles_n), in_band = local - band * 4 * tiles_n;
@@ -661,11 +667,13 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   // fixed 32-bit offsets inside any tile: its row and 16-byte piece, and its scale word (blocks 2*spiece,
   // 2*spiece+1 of the span: 128x4 layout column tile spiece>>1, bytes 2*(spiece&1)..).  A tile's first row is
   // a multiple of 128, so the swizzled scale address splits into the tile's part and the thread's part.
-  struct RowPtrs { const uint8_t *a, *b, *sa, *sb; };
+  struct RowPtrs { const uint8_t *a, *b, *sa, *sb; int a_bytes; };  // a_bytes: bytes of the A rows that exist (buffer range)
   auto tile_ptrs = [&](int t) {
     const Where w = tile_where(t);
     RowPtrs r;
     r.a = p.a + w.m0 * kbytes;
+    // 128-row tiles of the grouped op hold a whole group of fewer rows: the rows past it read as zero
+    r.a_bytes = (GROUPED && TM == 2) ? w.valid * kbytes : 0x7fffffff;
     r.b = p.b + ((int64_t)w.g * p.n + w.n0) * kbytes;
     // (a group's activation scales are a slab of their own, swizzled from its first row)
     const int64_t sa_slab = GROUPED ? (int64_t)__builtin_amdgcn_readfirstlane(p.sf_offsets[w.g]) * sf_padded : 0;
@@ -682,12 +690,12 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   // load unit q (0..7) of the span the stream is at; advance_stream() after the eighth
   // Buffer loads: the tile's first row as the resource's base, the span and the second row as the scalar
   // offset, the thread's fixed offset as the vector offset, so that no address is worked out in vector registers.
-  auto rsrc = [](const uint8_t* base) {
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(base), 0, 0x7fffffff, 0x00020000);
+  auto rsrc = [](const uint8_t* base, int bytes = 0x7fffffff) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(base), 0, bytes, 0x00020000);
   };
   auto issue_load_unit = [&](Raw& r, int q) {
     const int o = l_mac * 64, so = l_mac * 1024;
-    if (q == 0) r.a[0] = __builtin_amdgcn_raw_buffer_load_b128(rsrc(lp.a), off_ab, o, 0);
+    if (q == 0) r.a[0] = __builtin_amdgcn_raw_buffer_load_b128(rsrc(lp.a, lp.a_bytes), off_ab, o, 0);
     if (q == 1 && AR == 2) r.a[1] = __builtin_amdgcn_raw_buffer_load_b128(rsrc(lp.a), off_ab, o + (int)row128, 0);
     if (q == 2) r.b[0] = __builtin_amdgcn_raw_buffer_load_b128(rsrc(lp.b), off_ab, o, 0);
     if (q == 3) r.b[1] = __builtin_amdgcn_raw_buffer_load_b128(rsrc(lp.b), off_ab, o + (int)row128, 0);
@@ -700,6 +708,7 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
     const bool wrap = (l_mac + 1 == nmac);
     l_mac = wrap ? 0 : l_mac + 1;
     lp.a = wrap ? np.a : lp.a;
+    lp.a_bytes = wrap ? np.a_bytes : lp.a_bytes;
     lp.b = wrap ? np.b : lp.b;
     lp.sa = wrap ? np.sa : lp.sa;
     lp.sb = wrap ? np.sb : lp.sb;
@@ -960,7 +969,9 @@ int launch_nvfp4_fast_cfg(const Params& p, int cus, hipStream_t stream) {
   constexpr int lds_bytes = 2 * (64 * TM + 256) * 128 + 8 * 2560;  // 128 KiB / 96 KiB of tiles + the epilogue's 20 KiB
   static uint64_t configured = 0;  // one bit per device; a benign race: the attribute call is idempotent
   if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
-  const int64_t tiles = (int64_t)(p.m / (64 * TM)) * (p.n / 256);  // grouped: an upper bound
+  // grouped: an upper bound (128-row tiles: one per weight panel and group of at least rows_lo rows)
+  const int64_t tiles_m = (GROUPED && TM == 2) ? std::min<int64_t>(p.groups, p.m / std::max(p.rows_lo, 1)) : p.m / (64 * TM);
+  const int64_t tiles = tiles_m * (p.n / 256);
   const unsigned grid = (unsigned)(tiles >= cus ? (cus & ~7) : ((tiles + 7) / 8) * 8);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds_bytes, stream, p);
   return check_launch("nvfp4_gemm_256_kernel");
@@ -1693,8 +1704,18 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int6
       if (p.k < 4096 && (p.n & 255) == 0) rc = launch_nvfp4_skinny_grouped<2, 2, OUT_BF16, true>(p, 1, 32, stream);
       else rc = launch_nvfp4_skinny_grouped<4, 2, OUT_BF16, false>(p, 1, 32, stream);
       if (rc != NVF_OK) return rc;
-      if (p.k < 4096 && (p.n & 255) == 0) rc = launch_nvfp4_skinny_grouped<2, 8, OUT_BF16, true>(p, 33, 128, stream);
-      else rc = launch_nvfp4_skinny_grouped<4, 8, OUT_BF16, false>(p, 33, 128, stream);
+      if (p.k < 4096 && (p.n & 255) == 0 && p.k >= 256) {
+        // shallow K: one 128x256 tile of the persistent kernel per weight panel converts a group's rows once per 256
+        // weight rows; the streaming kernel whose wavefronts own rows converts them once per wavefront
+        Params mid = p;
+        mid.rows_lo = 33;
+        mid.rows_hi = 128;
+        rc = launch_nvfp4_fast<OUT_BF16, true, 2>(mid, cus, stream);
+      } else if (p.k < 4096 && (p.n & 255) == 0) {
+        rc = launch_nvfp4_skinny_grouped<2, 8, OUT_BF16, true>(p, 33, 128, stream);
+      } else {
+        rc = launch_nvfp4_skinny_grouped<4, 8, OUT_BF16, false>(p, 33, 128, stream);
+      }
       if (rc != NVF_OK) return rc;
       Params rest = p;
       rest.min_rows = 129;
