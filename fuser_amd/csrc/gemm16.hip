@@ -257,13 +257,12 @@ __global__ __launch_bounds__(256) void gemm16_kernel(const Params p) {
   }
 }
 
-// Grouped NVFP4: the rows of a group (m_g rows, the first at row row_off of the m_total activation rows) that the
-// 256x256 kernel computes: its whole 256-row tiles, and a last tile of more than 128 rows if the 256 rows that
-// tile loads lie inside the activation tensor (rows past the group are loaded and computed, not stored).  The
-// tile kernel takes the rows from there on; a value >= m_g means none are left.
-__device__ __forceinline__ int rows_in_256_tiles(int m_g, int64_t row_off, int m_total) {
+// Grouped NVFP4: the rows of a group of m_g rows that the 256x256 kernel computes: its whole 256-row tiles, and a
+// last tile of more than 128 rows (its missing rows read as zero through the buffer range and are not stored).
+// The tile kernel takes the rows from there on; a value >= m_g means none are left.
+__device__ __forceinline__ int rows_in_256_tiles(int m_g) {
   const int whole = m_g & ~255;
-  return (m_g - whole > 128 && row_off + whole + 256 <= m_total) ? whole + 256 : whole;
+  return m_g - whole > 128 ? whole + 256 : whole;
 }
 
 // -------------------------------------------------------------------------------------------------
@@ -309,7 +308,7 @@ __global__ __launch_bounds__(256) void nvfp4_tile_kernel(const Params p) {
       int cnt = 0;
       if (g < p.groups) {
         const int mg = p.problem_sizes[g * 3];
-        const int rest = mg < p.min_rows ? 0 : mg - (p.skip_whole_256 ? rows_in_256_tiles(mg, p.expert_offsets[g], p.m) : 0);
+        const int rest = mg < p.min_rows ? 0 : mg - (p.skip_whole_256 ? rows_in_256_tiles(mg) : 0);
         cnt = rest > 0 ? ((rest + BM - 1) / BM) * tiles_n : 0;
       }
       int incl = cnt;
@@ -352,7 +351,7 @@ __global__ __launch_bounds__(256) void nvfp4_tile_kernel(const Params p) {
     }
     const int m_g = dense ? p.m : p.problem_sizes[g * 3];
     const int64_t row_off = dense ? 0 : p.expert_offsets[g];
-    const int skipped = (!dense && p.skip_whole_256) ? rows_in_256_tiles(m_g, row_off, p.m) : 0;
+    const int skipped = (!dense && p.skip_whole_256) ? rows_in_256_tiles(m_g) : 0;
     const int tiles_m = (m_g - skipped + BM - 1) / BM;
     const int local = tile - tile_prefix[g];
     const int mt = local % tiles_m, nt = local / tiles_m;
@@ -578,7 +577,7 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   // range [x*chunk, (x+1)*chunk); with the 8 (m) x 4 (n) blocked numbering the 32 tiles an XCD works on
   // at a time share 8 A panels and 4 B panels in its L2.
   // GROUPED: the work list holds the 256-row tiles of every group that rows_in_256_tiles() names: the whole
-  // ones and a last one of more than 128 rows, whose rows past the group are computed and not stored; what
+  // ones and a last one of more than 128 rows, whose rows past the group read as zero and are not stored; what
   // is left at the end of a group goes to the tile kernel.  With 128-row tiles (TM == 2) the list is instead one
   // tile per weight panel for every group of rows_lo..rows_hi (<= 128) rows.
   const int tiles_m = p.m / BM, tiles_n = p.n / BN;
@@ -591,7 +590,7 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
         int cnt = 0;
         if (g < p.groups) {
           const int mg = p.problem_sizes[g * 3];
-          if constexpr (TM == 4) cnt = (rows_in_256_tiles(mg, p.expert_offsets[g], p.m) / BM) * tiles_n;
+          if constexpr (TM == 4) cnt = (rows_in_256_tiles(mg) / BM) * tiles_n;
           else cnt = (mg >= p.rows_lo && mg <= p.rows_hi) ? tiles_n : 0;  // one 128-row tile per group of the class and weight panel
         }
         int incl = cnt;
@@ -625,7 +624,7 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
       w.g = __builtin_amdgcn_readfirstlane(lo);
       const int m_g = __builtin_amdgcn_readfirstlane(p.problem_sizes[w.g * 3]);
       const int64_t row_off = __builtin_amdgcn_readfirstlane(p.expert_offsets[w.g]);
-      const int full_m = TM == 4 ? rows_in_256_tiles(m_g, row_off, p.m) / BM : 1;
+      const int full_m = TM == 4 ? rows_in_256_tiles(m_g) / BM : 1;
       const int local = __builtin_amdgcn_readfirstlane(t - tile_prefix[w.g]);
       // bands of 4 m-tiles, n-major inside a band: 32 consecutive tiles share 4 A and 8 B panels
       const int band = local / (4 * tiles_n), in_band = local - band * 4 * tiles_n;
@@ -672,8 +671,8 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
     const Where w = tile_where(t);
     RowPtrs r;
     r.a = p.a + w.m0 * kbytes;
-    // 128-row tiles of the grouped op hold a whole group of fewer rows: the rows past it read as zero
-    r.a_bytes = (GROUPED && TM == 2) ? w.valid * kbytes : 0x7fffffff;
+    // the last tile of a group may have fewer rows than the tile: the rows past the group read as zero
+    r.a_bytes = GROUPED ? w.valid * kbytes : 0x7fffffff;
     r.b = p.b + ((int64_t)w.g * p.n + w.n0) * kbytes;
     // (a group's activation scales are a slab of their own, swizzled from its first row)
     const int64_t sa_slab = GROUPED ? (int64_t)__builtin_amdgcn_readfirstlane(p.sf_offsets[w.g]) * sf_padded : 0;
@@ -696,7 +695,7 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   auto issue_load_unit = [&](Raw& r, int q) {
     const int o = l_mac * 64, so = l_mac * 1024;
     if (q == 0) r.a[0] = __builtin_amdgcn_raw_buffer_load_b128(rsrc(lp.a, lp.a_bytes), off_ab, o, 0);
-    if (q == 1 && AR == 2) r.a[1] = __builtin_amdgcn_raw_buffer_load_b128(rsrc(lp.a), off_ab, o + (int)row128, 0);
+    if (q == 1 && AR == 2) r.a[1] = __builtin_amdgcn_raw_buffer_load_b128(rsrc(lp.a, lp.a_bytes), off_ab, o + (int)row128, 0);
     if (q == 2) r.b[0] = __builtin_amdgcn_raw_buffer_load_b128(rsrc(lp.b), off_ab, o, 0);
     if (q == 3) r.b[1] = __builtin_amdgcn_raw_buffer_load_b128(rsrc(lp.b), off_ab, o + (int)row128, 0);
     if (q == 4) r.sa[0] = __builtin_amdgcn_raw_buffer_load_b16(rsrc(lp.sa), off_sf, so, 0);

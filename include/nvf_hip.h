@@ -177,9 +177,7 @@ NVF_API int nvf_grouped_mm(const void* a, const void* b, void* out, const int32_
  *   [sf_offsets[g], sf_offsets[g] + roundUp(m_g,128)) of a [*, k/16] buffer, 128x4-swizzled on its
  *   own; b_scales [groups, n, k/16] e4m3, each [n, k/16] slab 128x4-swizzled; alphas fp32 [groups].
  *   k % 64 == 0, n % 8 == 0 as in the reference; this implementation also needs n % 128 == 0 for
- *   the per-expert b_scales slabs to be whole 128x4 tiles (the reference's pointer rule implies it).
- *   m is the number of rows the a buffer holds: rows of a past a group's end (never past m) may be
- *   read; they reach no output. */
+ *   the per-expert b_scales slabs to be whole 128x4 tiles (the reference's pointer rule implies it). */
 NVF_API int nvf_nvfp4_scaled_grouped_mm(const void* a, const void* b, const void* a_scales,
                                         const void* b_scales, const float* alphas, void* out,
                                         const int32_t* problem_sizes, const int32_t* expert_offsets,

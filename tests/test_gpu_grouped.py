@@ -193,12 +193,12 @@ def test_nvfp4_grouped_mm_empty_and_tiny_groups(dev):
                                        ([40, 64, 2100, 33, 65, 100, 128, 50, 0, 32], 384, 256)])
 def test_nvfp4_grouped_mm_whole_tiles_and_group_ends(dev, sizes, n, k):
     """At least 2048 rows, N % 256 == 0, K % 128 == 0: the whole 256-row tiles of every group, and a last tile of
-    more than 128 rows, run on the persistent 256x256 kernel (which loads and computes the rows past such a
-    group and does not store them: the next group's rows, or the poisoned scale padding), the other group ends
+    more than 128 rows, run on the persistent 256x256 kernel (the rows past such a group read as zero payload
+    with whatever the scale padding holds - it is poisoned here - and are not stored), the other group ends
     on the 128x128 tile kernel.  Groups with no whole tile, only whole tiles, one row past a tile, 255 of 256
     rows, empty groups; two, three and five spans per tile; the third case has more than 320 tiles, i.e. two
-    per workgroup for some; in the last case the final group's 144-row end would load past the activation
-    tensor as a 256-row tile and therefore stays with the tile kernel.  The last two cases add groups of every
+    per workgroup for some; the [2248, 130, 400] case ends with a 144-row tile whose 256 rows would reach past the
+    activation tensor.  The last two cases add groups of every
     weight-streaming class next to a large one (wavefronts owning rows, and wavefronts splitting K).  Every
     output element is compared."""
     from fuser_amd import nvf_cutlass
