@@ -1703,9 +1703,10 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int6
       if (p.k < 4096 && (p.n & 255) == 0) rc = launch_nvfp4_skinny_grouped<2, 2, OUT_BF16, true>(p, 1, 32, stream);
       else rc = launch_nvfp4_skinny_grouped<4, 2, OUT_BF16, false>(p, 1, 32, stream);
       if (rc != NVF_OK) return rc;
-      if (p.k < 4096 && (p.n & 255) == 0 && p.k >= 256) {
+      if ((p.k < 4096 || m_hint < 2048) && (p.n & 255) == 0 && p.k >= 256) {
         // shallow K: one 128x256 tile of the persistent kernel per weight panel converts a group's rows once per 256
-        // weight rows; the streaming kernel whose wavefronts own rows converts them once per wavefront
+        // weight rows; the streaming kernel whose wavefronts own rows converts them once per wavefront.  Few rows
+        // in all (a decode step): such groups are rare and the persistent kernel costs least when it finds none.
         Params mid = p;
         mid.rows_lo = 33;
         mid.rows_hi = 128;
