@@ -56,6 +56,7 @@ struct Params {
   int m_base = 0;
   // grouped skinny kernel: the group sizes it serves; the tile kernel skips groups of fewer than min_rows rows
   int rows_lo = 0, rows_hi = 0, min_rows = 0;
+  int tail_done = 0;  // grouped NVFP4 dispatch: the ends of the large groups have been computed by an earlier launch
 };
 
 __device__ __forceinline__ uint32_t pack2(float a, float b, bool out_bf16) {
@@ -579,7 +580,8 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   // GROUPED: the work list holds the 256-row tiles of every group that rows_in_256_tiles() names: the whole
   // ones and a last one of more than 128 rows, whose rows past the group read as zero and are not stored; what
   // is left at the end of a group goes to the tile kernel.  With 128-row tiles (TM == 2) the list is instead one
-  // tile per weight panel for every group of rows_lo..rows_hi (<= 128) rows.
+  // tile per weight panel for every group of rows_lo..rows_hi (<= 128) rows and, if min_rows is set, for the end
+  // (what rows_in_256_tiles() leaves) of every group of at least min_rows rows.
   const int tiles_m = p.m / BM, tiles_n = p.n / BN;
   int total = tiles_m * tiles_n;
   if constexpr (GROUPED) {
@@ -591,7 +593,8 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
         if (g < p.groups) {
           const int mg = p.problem_sizes[g * 3];
           if constexpr (TM == 4) cnt = (rows_in_256_tiles(mg) / BM) * tiles_n;
-          else cnt = (mg >= p.rows_lo && mg <= p.rows_hi) ? tiles_n : 0;  // one 128-row tile per group of the class and weight panel
+          else  // one 128-row tile per weight panel: a group of the class, or (min_rows set) the end of a larger group
+            cnt = ((mg >= p.rows_lo && mg <= p.rows_hi) || (p.min_rows && mg >= p.min_rows && mg > rows_in_256_tiles(mg))) ? tiles_n : 0;
         }
         int incl = cnt;
 #pragma unroll
@@ -630,7 +633,7 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
       const int band = local / (4 * tiles_n), in_band = local - band * 4 * tiles_n;
       const int band_h = min(4, full_m - 4 * band);
       const int nt = in_band / band_h, mt = 4 * band + (in_band - nt * band_h);
-      w.gm0 = mt * BM;
+      w.gm0 = TM == 4 ? mt * BM : (m_g <= BM ? 0 : rows_in_256_tiles(m_g));
       w.m0 = row_off + w.gm0;
       w.n0 = nt * BN;
       w.valid = min(BM, m_g - w.gm0);
@@ -1699,7 +1702,7 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int6
     if (!dense && p.min_rows == 0 && (p.n & 63) == 0 && (p.k & 127) == 0 && (int64_t)p.k * 64 < (1ll << 31)) {
       // With a shallow K a split of K over the wavefronts leaves each only a chunk or two: they then own
       // different weight rows instead (K=2048, N=7168: 549 -> 464 us for 64 tokens x top-8; deeper K: slower).
-      int rc;
+      int rc, tail_done = 0;
       if (p.k < 4096 && (p.n & 255) == 0) rc = launch_nvfp4_skinny_grouped<2, 2, OUT_BF16, true>(p, 1, 32, stream);
       else rc = launch_nvfp4_skinny_grouped<4, 2, OUT_BF16, false>(p, 1, 32, stream);
       if (rc != NVF_OK) return rc;
@@ -1710,6 +1713,8 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int6
         Params mid = p;
         mid.rows_lo = 33;
         mid.rows_hi = 128;
+        if (m_hint >= 2048) mid.min_rows = 129;  // the 256x256 kernel follows: take the ends of its groups along
+        tail_done = mid.min_rows != 0;
         rc = launch_nvfp4_fast<OUT_BF16, true, 2>(mid, cus, stream);
       } else if (p.k < 4096 && (p.n & 255) == 0) {
         rc = launch_nvfp4_skinny_grouped<2, 8, OUT_BF16, true>(p, 33, 128, stream);
@@ -1719,6 +1724,7 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int6
       if (rc != NVF_OK) return rc;
       Params rest = p;
       rest.min_rows = 129;
+      rest.tail_done = tail_done;
       return launch_sized<NVFP4, BF16_MMA, OUT_BF16>(rest, m_hint, cus, workspace, workspace_bytes, stream);
     }
     // Grouped NVFP4 with room for whole 256-row tiles: those go to the 256x256 kernel (about 1.4 times as
@@ -1726,7 +1732,7 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int6
     // device, so both kernels are always launched; one that finds no work returns at once.
     if (!dense && (p.n & 255) == 0 && (p.k & 127) == 0 && p.k >= 256 && m_hint >= 2048) {
       const int rc = launch_nvfp4_fast<OUT_BF16, true>(p, cus, stream);
-      if (rc != NVF_OK) return rc;
+      if (rc != NVF_OK || p.tail_done) return rc;
       Params rest = p;
       rest.skip_whole_256 = 1;
       const int64_t upper = 2 * (int64_t)p.groups * ceil_div(p.n, 128), cap = 2 * (int64_t)cus;
