@@ -28,7 +28,7 @@ struct Params {
   const float* alpha;
   void* out;
   int m, n, k;
-  int m_base = 0;  // skinny kernel: first of the (at most 128) activation rows this launch computes, a multiple of 128
+  int m_base = 0;  // skinny kernel: first activation row this launch computes, a multiple of 64
 };
 
 __device__ __forceinline__ uint32_t pack2(float a, float b, bool out_bf16) {
@@ -520,9 +520,10 @@ int launch_fast(const Params& p, hipStream_t stream) {
 }
 
 // -------------------------------------------------------------------------------------------------
-// Skinny path: up to 128 activation rows per launch (decode-sized activations; more rows in launches of 128),
-// K % 128 == 0, N % (16*RT) == 0.  A launch streams the weight matrix exactly once, so the op is bound by HBM
-// (by the last-level cache for the launches after the first):
+// Skinny path: slabs of up to 128 activation rows (decode-sized activations; more rows as several slabs, the
+// whole ones side by side in one launch, blockIdx.y = slab), K % 128 == 0, N % (16*RT) == 0.  A slab streams
+// the weight matrix exactly once, so the op is bound by HBM (by the last-level cache for the slabs after the
+// first):
 //   * A workgroup owns 16*RT weight rows for the whole of K and all M activation rows; its 8 wavefronts
 //     split K in interleaved 128-element chunks and their partial sums are added in a fixed order through
 //     LDS (no atomics, no workspace, deterministic).
@@ -556,7 +557,9 @@ __global__ __launch_bounds__(512) void mxfp8_skinny_kernel(const Params p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, g = lane >> 4;
   const int n0 = blockIdx.x * (16 * RT);
-  const int m_loc = min(p.m - p.m_base, 16 * TT);  // activation rows of this launch: [m_base, m_base + m_loc)
+  // activation rows of this workgroup: [m_base, m_base + m_loc); blockIdx.y counts slabs of 16*TT rows
+  const int m_base = p.m_base + (int)blockIdx.y * (16 * TT);
+  const int m_loc = min(p.m - m_base, 16 * TT);
   const int tt_count = (m_loc + 15) >> 4;
   const int chunks = p.k >> 7;
   const int sf_padded = p.k >> 5;  // K % 128 == 0: no padding columns
@@ -578,8 +581,8 @@ __global__ __launch_bounds__(512) void mxfp8_skinny_kernel(const Params p) {
   }
   const int st = lane >> 4;  // tile whose scales this lane fetches
   const uint32_t bsf_off = (uint32_t)((((n0 & 127) + min(st, RT - 1) * 16 + r) & 31) * 16);
-  const uint8_t* a_base = p.a + (int64_t)p.m_base * p.k;
-  const uint8_t* asf_base = p.sfa + (int64_t)(p.m_base >> 7) * ((int64_t)sf_padded << 7);
+  const uint8_t* a_base = p.a + (int64_t)m_base * p.k;
+  const uint8_t* asf_base = p.sfa + (int64_t)(m_base >> 7) * ((int64_t)sf_padded << 7);
   const uint32_t asf_off = (uint32_t)((lane & 31) * 16);  // scale group of rows {lane, lane + 32, ...} of the 128-row tile
   const uint32_t lds_base = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)lds);
   const uint32_t ring_base = lds_base + (uint32_t)wave * (DEPTH * SLOT_BYTES);
@@ -609,7 +612,7 @@ __global__ __launch_bounds__(512) void mxfp8_skinny_kernel(const Params p) {
   for (int rt = 0; rt < RT; ++rt) rd_bsc[rt] = NT * 2048 + rt * 256 + r * 16 + ((((n0 & 127) + rt * 16) >> 5) & 3) * 4;
 #pragma unroll
   for (int tt = 0; tt < TT; ++tt)
-    rd_asc[tt] = NT * 2048 + RT * 256 + ((tt & 1) * 16 + r) * 16 + ((((p.m_base & 127) + tt * 16) >> 5) & 3) * 4;
+    rd_asc[tt] = NT * 2048 + RT * 256 + ((tt & 1) * 16 + r) * 16 + ((((m_base & 127) + tt * 16) >> 5) & 3) * 4;
   const int sc_shift = g * 8;
 
   f32x4 acc[RT][TT];
@@ -684,13 +687,13 @@ __global__ __launch_bounds__(512) void mxfp8_skinny_kernel(const Params p) {
       u32x2 v;
       v[0] = pack2(s[0] * alpha, s[1] * alpha, OUT_BF16);
       v[1] = pack2(s[2] * alpha, s[3] * alpha, OUT_BF16);
-      *reinterpret_cast<u32x2*>(out + (int64_t)(p.m_base + tok) * p.n + n0 + rt * 16 + 4 * (l >> 4)) = v;
+      *reinterpret_cast<u32x2*>(out + (int64_t)(m_base + tok) * p.n + n0 + rt * 16 + 4 * (l >> 4)) = v;
     }
   }
 }
 
 template <int RT, int TT, bool OUT_BF16>
-int launch_skinny_cfg(const Params& p, hipStream_t stream) {
+int launch_skinny_cfg(const Params& p, hipStream_t stream, int slabs = 1) {
   constexpr int SLOT = (RT + TT) * 2048 + RT * 256 + (TT < 2 ? TT : 2) * 256;
   constexpr int DEPTH = 8 * 3 * SLOT <= 160 * 1024 ? 3 : (8 * 2 * SLOT <= 160 * 1024 ? 2 : 1);
   auto kern = mxfp8_skinny_kernel<RT, TT, OUT_BF16, DEPTH>;
@@ -699,7 +702,7 @@ int launch_skinny_cfg(const Params& p, hipStream_t stream) {
   static_assert(lds_bytes <= 160 * 1024, "LDS");
   static uint64_t configured = 0;  // one bit per device; a benign race: the attribute call is idempotent
   if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
-  hipLaunchKernelGGL(kern, dim3((unsigned)(p.n / (16 * RT))), dim3(512), lds_bytes, stream, p);
+  hipLaunchKernelGGL(kern, dim3((unsigned)(p.n / (16 * RT)), (unsigned)slabs), dim3(512), lds_bytes, stream, p);
   return check_launch("mxfp8_skinny_kernel");
 }
 
@@ -720,7 +723,14 @@ int launch_skinny(const Params& p0, hipStream_t stream) {
   const bool wide_n = (p0.n & 63) == 0 && p0.n / 64 >= 256 * 4 / 5;
   const int slab = wide_n ? 64 : 128;
   Params p = p0;
-  for (p.m_base = 0; p.m_base < p.m; p.m_base += slab) {
+  p.m_base = 0;
+  if (!wide_n && p.m >= 256) {
+    // all whole slabs in one launch: a slab alone has N/16 workgroups, too few for the chip when N is small
+    const int whole = p.m / 128;
+    if (const int rc = launch_skinny_cfg<1, 8, OUT_BF16>(p, stream, whole)) return rc;
+    p.m_base = whole * 128;
+  }
+  for (; p.m_base < p.m; p.m_base += slab) {
     const int rows = min(p.m - p.m_base, slab);
     const int rc = rows <= 16 ? launch_skinny_tt<1, OUT_BF16>(p, stream)
                  : rows <= 32 ? launch_skinny_tt<2, OUT_BF16>(p, stream)
@@ -746,8 +756,14 @@ template <bool OUT_BF16>
 int launch_sized(const Params& p, hipStream_t stream) {
   auto tiles = [&](int bm, int bn) { return ceil_div(p.m, bm) * ceil_div(p.n, bn); };
   // up to 256 rows, i.e. four passes over the weights (the later ones out of the last-level cache), this beats
-  // the tile kernels below (measured: 128 x 4096 x 14336 in 35 instead of 117 us, 256 x 14336 x 4096 equal)
-  if (p.m <= 256 && (p.k & 127) == 0 && (p.n & 15) == 0 && (int64_t)p.k * 64 < (1ll << 31))  // 32-bit lane offsets
+  // the tile kernels below (measured: 128 x 4096 x 14336 in 35 instead of 117 us, 256 x 14336 x 4096 equal).
+  // More rows with a deep K and a small N leave the tile kernels too few tiles for the chip: the skinny
+  // kernel's workgroups (one per 128 rows x 16 columns, K split over their wavefronts) then fill it.  A round
+  // of them costs about a quarter of a round of 128x256 tiles, so up to 3 rounds win or tie (measured, K >= 2048:
+  // 512 x 2048 x 7168 in 27 instead of 59 us, 384 x 3072 x 7168 in 39 instead of 62, 384 x 4096 x 4096 27 both).
+  const int64_t skinny_rounds = ceil_div(ceil_div(p.m, 128) * (int64_t)(p.n / 16), 256);
+  if ((p.m <= 256 || (skinny_rounds <= 3 && p.k >= 2048)) && (p.k & 127) == 0 && (p.n & 15) == 0 &&
+      (int64_t)p.k * 64 < (1ll << 31))  // 32-bit lane offsets
     return launch_skinny<OUT_BF16>(p, stream);
   if ((p.k & 127) == 0 && p.k >= 256 && (p.m & 127) == 0 && (p.n & 255) == 0 && (int64_t)p.k * 256 < (1ll << 31)) {
     // Persistent LDS-direct kernel with 256x256 or 128x256 tiles: a 128-row tile costs about 0.61 of a 256-row

@@ -382,6 +382,31 @@ def test_mxfp8_gemm_decode_sized_activations(dev, shape):
         assert torch.equal(out, _run_mxfp8(a, b, sa_p, sb, 0.75, dtype, dev))
 
 
+@pytest.mark.parametrize("shape", [(300, 2048, 2048), (512, 1536, 2304), (384, 3072, 2048), (640, 528, 2176), (1000, 272, 2560),
+                                   (257, 16, 2048), (1024, 768, 2048), (2100, 96, 4096)])
+def test_mxfp8_gemm_many_rows_small_n_deep_k(dev, shape):
+    """More than 256 rows with K >= 2048 and an N small enough that the workgroups of the kernel for decode-sized
+    activations (one per 128 rows x 16 columns) cover the compute units at most three times: all whole 128-row
+    slabs go in one launch (2 to 16 slabs), the remaining rows (44, 104, 1, 52 or none) in a launch of their
+    own with 1 / 4 / 8 activation tiles.  Every output element is compared with the oracle, with poisoned scale
+    padding, both output types and run-to-run determinism."""
+    m, n, k = shape
+    gen = torch.Generator().manual_seed(m * 31 + n)
+    a, sa = _mxfp8_operand(m, k, gen, 1.0)
+    b, sb = _mxfp8_operand(n, k, gen, 1.0)
+    ref = O.ref_mxfp8_scaled_mm(a, b, sa, sb, 0.75)
+    sa_p = sa.clone()  # NaN code in every scale byte of the padding rows / columns
+    sa_p[O.linear_to_swizzled_128_4(torch.ones(m, k // 32, dtype=torch.uint8)) == 0] = 0xFF
+    scale = ref.abs().amax(dim=1, keepdim=True).clamp(min=1e-30)
+    for dtype in (torch.bfloat16, torch.float16):
+        if dtype == torch.float16 and ref.abs().max() > 6e4:
+            continue
+        out = _run_mxfp8(a, b, sa_p, sb, 0.75, dtype, dev)
+        assert out.shape == (m, n)
+        assert ((out.float().cpu() - ref).abs() / scale).max().item() <= GEMM_MAX_REL, (shape, dtype)
+        assert torch.equal(out, _run_mxfp8(a, b, sa_p, sb, 0.75, dtype, dev))
+
+
 @pytest.mark.parametrize("shape", [(4096, 2048, 512), (2560, 3328, 384), (2048, 4096, 256), (8192, 1024, 1152),
                                    (4096, 8192, 256), (8192, 4096, 384), (4352, 4096, 640), (1152, 2048, 384)])
 def test_mxfp8_gemm_persistent_256_tile_kernel_full_compare(dev, shape):
