@@ -1067,7 +1067,10 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
     b_row0 = (int64_t)grp * p.n;
   } else {
     n0 = blockIdx.x * (16 * RT);
-    m_loc = min(p.m - p.m_base, 128);  // activation rows of this launch: [m_base, m_base + m_loc)
+    // activation rows of this workgroup: [m_base, m_base + m_loc); blockIdx.y counts slabs of 128 rows
+    const int m_base = p.m_base + (int)blockIdx.y * 128;
+    a_row0 = asf_row0 = m_base;
+    m_loc = min(p.m - m_base, 128);
   }
   const int tt_count = (m_loc + 15) >> 4;
 
@@ -1250,7 +1253,7 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
 }
 
 template <int RT, int TT, bool OUT_BF16>
-int launch_nvfp4_skinny_ring_cfg(const Params& p, hipStream_t stream) {
+int launch_nvfp4_skinny_ring_cfg(const Params& p, hipStream_t stream, int slabs = 1) {
   constexpr int SLOT_KIB = RT + TT + (RT + 1) / 2 + (TT + 1) / 2;
   // one slot per wavefront also where two would fit (M=16, N=14336, K=4096: 8.0 -> 7.5 us; K=14336: 9.6 -> 9.2 us)
   constexpr int DEPTH = 1;
@@ -1262,7 +1265,7 @@ int launch_nvfp4_skinny_ring_cfg(const Params& p, hipStream_t stream) {
   static_assert(lds_bytes <= 160 * 1024, "LDS");
   static uint64_t configured = 0;  // one bit per device; a benign race: the attribute call is idempotent
   if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
-  hipLaunchKernelGGL(kern, dim3((unsigned)(p.n / (16 * RT))), dim3(512), lds_bytes, stream, p);
+  hipLaunchKernelGGL(kern, dim3((unsigned)(p.n / (16 * RT)), (unsigned)slabs), dim3(512), lds_bytes, stream, p);
   return check_launch("nvfp4_skinny_ring_kernel");
 }
 
@@ -1290,20 +1293,27 @@ int launch_nvfp4_skinny_grouped(const Params& p0, int rows_lo, int rows_hi, hipS
 }
 
 template <int TT, bool OUT_BF16>
-int launch_nvfp4_skinny_tt(const Params& p, int cus, hipStream_t stream) {
+int launch_nvfp4_skinny_tt(const Params& p, int cus, hipStream_t stream, int slabs = 1) {
   // The conversion work bounds this kernel, and every workgroup converts all activation rows it uses:
   // take as many weight rows per workgroup as still leaves about one workgroup per compute unit.
   const int64_t want = (int64_t)cus * 4 / 5;
-  if ((p.n & 63) == 0 && p.n / 64 >= want) return launch_nvfp4_skinny_ring_cfg<4, TT, OUT_BF16>(p, stream);
-  if ((p.n & 31) == 0 && p.n / 32 >= want) return launch_nvfp4_skinny_ring_cfg<2, TT, OUT_BF16>(p, stream);
-  return launch_nvfp4_skinny_ring_cfg<1, TT, OUT_BF16>(p, stream);
+  if ((p.n & 63) == 0 && p.n / 64 >= want) return launch_nvfp4_skinny_ring_cfg<4, TT, OUT_BF16>(p, stream, slabs);
+  if ((p.n & 31) == 0 && p.n / 32 >= want) return launch_nvfp4_skinny_ring_cfg<2, TT, OUT_BF16>(p, stream, slabs);
+  return launch_nvfp4_skinny_ring_cfg<1, TT, OUT_BF16>(p, stream, slabs);
 }
 
 template <bool OUT_BF16>
 int launch_nvfp4_skinny(const Params& p0, int cus, hipStream_t stream) {
-  // more than 128 rows: launches of 128, each streaming the weights (the later ones out of the last-level cache)
+  // more than 128 rows: slabs of 128, each streaming the weights (the later ones out of the last-level cache);
+  // the whole slabs side by side in one launch, because a slab alone may have too few workgroups for the chip
   Params p = p0;
-  for (p.m_base = 0; p.m_base < p.m; p.m_base += 128) {
+  p.m_base = 0;
+  if (p.m >= 256) {
+    const int whole = p.m / 128;
+    if (const int rc = launch_nvfp4_skinny_tt<8, OUT_BF16>(p, cus, stream, whole)) return rc;
+    p.m_base = whole * 128;
+  }
+  for (; p.m_base < p.m; p.m_base += 128) {
     const int rows = p.m - p.m_base;
     const int rc = rows <= 16 ? launch_nvfp4_skinny_tt<1, OUT_BF16>(p, cus, stream)
                  : rows <= 32 ? launch_nvfp4_skinny_tt<2, OUT_BF16>(p, cus, stream)
@@ -1675,7 +1685,14 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int6
     }
     // up to 256 rows (two passes over the weights) this beats the tile kernel (measured: 256 x 14336 x 4096 in
     // 46 instead of 65 us; at 512 rows the tile kernel wins)
-    if (dense && p.m <= 256 && (p.k & 127) == 0 && (p.n & 15) == 0 && (int64_t)p.k * 64 < (1ll << 31))  // 32-bit lane offsets
+    // More rows with a deep K and a small N leave the kernels below too few tiles for the chip (without a
+    // workspace there is no split of K); the skinny kernel splits K over a workgroup's wavefronts, and its
+    // workgroups (one per 128 rows x 16 columns at such N) win or tie while they cover the compute units at most
+    // 3 times, 2 times for K < 4096 (measured: 512 x 2048 x 7168 in 34 instead of 45 us, 384 x 3072 x 7168 in
+    // 49 instead of 59, 1024 x 1536 x 7168 in 50 instead of 59, 300 x 3072 x 2048 in 18 instead of 16).
+    const int64_t skinny_rounds = ceil_div(ceil_div(p.m, 128) * (int64_t)(p.n / 16), cus);
+    if (dense && (p.m <= 256 || (p.k >= 2048 && skinny_rounds <= (p.k >= 4096 ? 3 : 2))) && (p.k & 127) == 0 && (p.n & 15) == 0 &&
+        (int64_t)p.k * 64 < (1ll << 31))  // 32-bit lane offsets
       return launch_nvfp4_skinny<OUT_BF16>(p, cus, stream);
     if (dense && (p.m & 127) == 0 && (p.n & 255) == 0 && (p.k & 127) == 0 && p.k >= 256) {
       // Persistent kernel with 256x256 or 128x256 tiles, or the tile kernel below?  Costs in units of one round

@@ -184,6 +184,28 @@ def test_nvfp4_gemm_decode_sized_activations(dev, shape):
         assert torch.equal(out, _run_nvfp4(a, b, sa_p, sb, alpha, dtype, dev))
 
 
+@pytest.mark.parametrize("shape", [(300, 2048, 2048), (512, 1536, 2304), (384, 3072, 4096), (640, 544, 2176), (1000, 288, 2560),
+                                   (257, 32, 2048), (1024, 768, 2048), (2100, 96, 4096)])
+def test_nvfp4_gemm_many_rows_small_n_deep_k(dev, shape):
+    """More than 256 rows with K >= 2048 and an N small enough that the workgroups of the kernel for decode-sized
+    activations (one per 128 rows x 16 columns) cover the compute units at most two or three times: all whole
+    128-row slabs go in one launch (2 to 16 slabs), the remaining rows (44, 104, 1, 52 or none) in a launch of
+    their own.  Every output element is compared with the oracle, with poisoned scale padding, both output
+    types and run-to-run determinism."""
+    m, n, k = shape
+    gen = torch.Generator().manual_seed(m * 31 + n)
+    a, sa, ga = _nvfp4_operand(m, k, 1.0, gen)
+    b, sb, gb = _nvfp4_operand(n, k, 0.02, gen)
+    alpha = 1.0 / (ga * gb)
+    ref = O.ref_nvfp4_scaled_mm(a, b, sa, sb, alpha)
+    sa_p = sa.clone()  # NaN code in every scale byte of the padding rows
+    sa_p[O.linear_to_swizzled_128_4(torch.ones(m, k // 16, dtype=torch.uint8)) == 0] = 0x7F
+    for dtype in (torch.bfloat16, torch.float16):
+        out = _run_nvfp4(a, b, sa_p, sb, alpha, dtype, dev)
+        assert out.shape == (m, n) and max_rel(out, ref) <= GEMM_MAX_REL, (shape, dtype)
+        assert torch.equal(out, _run_nvfp4(a, b, sa_p, sb, alpha, dtype, dev))
+
+
 @pytest.mark.parametrize("shape", [(128, 1024, 8192), (100, 256, 8224), (200, 512, 10240), (65, 160, 9216), (300, 2048, 14336)])
 def test_nvfp4_gemm_split_k_with_workspace(dev, shape):
     """Few 128x128 output tiles and a deep K: with the scratch memory that
