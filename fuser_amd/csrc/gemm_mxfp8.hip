@@ -762,10 +762,18 @@ int launch_sized(const Params& p, hipStream_t stream) {
   // of them costs about a quarter of a round of 128x256 tiles, so up to 3 rounds win or tie (measured, K >= 2048:
   // 512 x 2048 x 7168 in 27 instead of 59 us, 384 x 3072 x 7168 in 39 instead of 62, 384 x 4096 x 4096 27 both).
   const int64_t skinny_rounds = ceil_div(ceil_div(p.m, 128) * (int64_t)(p.n / 16), 256);
-  if ((p.m <= 256 || (skinny_rounds <= 3 && p.k >= 2048)) && (p.k & 127) == 0 && (p.n & 15) == 0 &&
+  const bool fast_ok = (p.k & 127) == 0 && p.k >= 256 && (p.m & 127) == 0 && (p.n & 255) == 0 && (int64_t)p.k * 256 < (1ll << 31);
+  // Exception: 128 or 256 rows and a wide N.  Per 1024 of K a round of skinny workgroups costs about 1.7 us with
+  // 128-row slabs and 3.4 us with the 64-row slabs of a wide N (which are launches of their own), a round of
+  // 128x256 tiles 6.8 us: where one round of those tiles covers the shape, it wins from about N = 10240 at 256
+  // rows (measured: 256 x 14336 x 4096 in 31 instead of 55 us, 256 x 28672 x 4096 in 34 instead of 104 us).
+  const bool wide_n = (p.n & 63) == 0 && p.n / 64 >= 256 * 4 / 5;
+  const int64_t skinny_cost = wide_n ? 34 * ceil_div(p.m, 64) * ceil_div(p.n / 64, 256) : 17 * skinny_rounds;
+  const bool wide_256 = fast_ok && p.m <= 256 && tiles(128, 256) >= 48 && 68 * ceil_div(tiles(128, 256), 256) < skinny_cost;
+  if (!wide_256 && (p.m <= 256 || (skinny_rounds <= 3 && p.k >= 2048)) && (p.k & 127) == 0 && (p.n & 15) == 0 &&
       (int64_t)p.k * 64 < (1ll << 31))  // 32-bit lane offsets
     return launch_skinny<OUT_BF16>(p, stream);
-  if ((p.k & 127) == 0 && p.k >= 256 && (p.m & 127) == 0 && (p.n & 255) == 0 && (int64_t)p.k * 256 < (1ll << 31)) {
+  if (fast_ok) {
     // Persistent LDS-direct kernel with 256x256 or 128x256 tiles: a 128-row tile costs about 0.61 of a 256-row
     // tile (half the flops at 82 % of the rate, measured), and the time goes with the rounds of tiles over the
     // compute units; below 48 tiles the tile kernels further down do as well.

@@ -430,13 +430,16 @@ def test_mxfp8_gemm_many_rows_small_n_deep_k(dev, shape):
 
 
 @pytest.mark.parametrize("shape", [(4096, 2048, 512), (2560, 3328, 384), (2048, 4096, 256), (8192, 1024, 1152),
-                                   (4096, 8192, 256), (8192, 4096, 384), (4352, 4096, 640), (1152, 2048, 384)])
+                                   (4096, 8192, 256), (8192, 4096, 384), (4352, 4096, 640), (1152, 2048, 384),
+                                   (256, 13312, 256), (128, 28672, 384), (256, 10240, 512)])
 def test_mxfp8_gemm_persistent_256_tile_kernel_full_compare(dev, shape):
     """Shapes with N % 256 == K % 128 == 0 and M % 128 == 0 take the persistent LDS-direct kernel with
     256x256 tiles ((2560, 3328): a tile grid that is not a multiple of the 8 x 4 blocking; the two 512-tile
     shapes: two tiles per workgroup, so that the load stream wraps across tiles) or with 128x256 tiles where
     those fill the compute units better (the 128-tile shapes, 272 tiles, and M = 1152, which is no multiple
-    of 256); two, three, five and nine K steps per tile.  Every output element is compared with the oracle."""
+    of 256); two, three, five and nine K steps per tile; 128 and 256 rows with an N so wide that one round of
+    128x256 tiles beats the kernel for decode-sized activations.  Every output element is compared with the
+    oracle."""
     m, n, k = shape
     gen = torch.Generator().manual_seed(k)
     a, sa = _mxfp8_operand(m, k, gen, 1.0)
