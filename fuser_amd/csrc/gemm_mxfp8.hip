@@ -707,38 +707,55 @@ int launch_skinny_cfg(const Params& p, hipStream_t stream, int slabs = 1) {
 }
 
 template <int TT, bool OUT_BF16>
-int launch_skinny_tt(const Params& p, hipStream_t stream) {
+int launch_skinny_tt(const Params& p, hipStream_t stream, int slabs = 1) {
   // as many weight rows per workgroup as still leaves about one workgroup per compute unit
   const int64_t want = 256 * 4 / 5;
-  if ((p.n & 63) == 0 && p.n / 64 >= want) return launch_skinny_cfg<4, TT, OUT_BF16>(p, stream);
-  if ((p.n & 31) == 0 && p.n / 32 >= want) return launch_skinny_cfg<2, TT, OUT_BF16>(p, stream);
-  return launch_skinny_cfg<1, TT, OUT_BF16>(p, stream);
+  if ((p.n & 63) == 0 && p.n / 64 >= want) return launch_skinny_cfg<4, TT, OUT_BF16>(p, stream, slabs);
+  if ((p.n & 31) == 0 && p.n / 32 >= want) return launch_skinny_cfg<2, TT, OUT_BF16>(p, stream, slabs);
+  return launch_skinny_cfg<1, TT, OUT_BF16>(p, stream, slabs);
 }
 
 template <bool OUT_BF16>
-int launch_skinny(const Params& p0, hipStream_t stream) {
-  // Up to 128 rows per launch.  With 8 activation tiles only one weight-row tile fits the LDS ring, and every
-  // workgroup fetches all activation rows: where N supplies enough workgroups of four weight-row tiles, launches
-  // of 64 rows with those are faster (128 x 14336 x 4096: 30 against 36 us; 128 x 4096 x 4096: 16 against 12).
-  const bool wide_n = (p0.n & 63) == 0 && p0.n / 64 >= 256 * 4 / 5;
-  const int slab = wide_n ? 64 : 128;
-  Params p = p0;
-  p.m_base = 0;
-  if (!wide_n && p.m >= 256) {
-    // all whole slabs in one launch: a slab alone has N/16 workgroups, too few for the chip when N is small
-    const int whole = p.m / 128;
-    if (const int rc = launch_skinny_cfg<1, 8, OUT_BF16>(p, stream, whole)) return rc;
-    p.m_base = whole * 128;
+int launch_skinny(const Params& p, hipStream_t stream) {
+  // Slabs of 128, 64 or 32 rows, all in one launch (blockIdx.y = slab; the last one may be ragged).  With 8
+  // activation tiles only one weight-row tile fits the LDS ring, and every workgroup fetches all activation rows
+  // of its slab: where N supplies enough workgroups of four weight-row tiles, slabs of 64 rows with those are
+  // faster (128 x 14336 x 4096: 30 against 36 us; 128 x 4096 x 4096: 16 against 12).  Otherwise a workgroup
+  // has 16 weight rows, and a small N leaves compute units idle: a round of workgroups costs about 100 / 60 / 47
+  // with slabs of 128 / 64 / 32 rows (measured at K = 2048 and 7168), so lower slabs win where they add no round
+  // (128 x 2048 x 7168: 11.4 -> 8.3 us, 192 x 512 x 7168: 18.2 -> 5.9 us, 512 x 512 x 7168: 13.9 -> 8.8 us).
+  // A ragged last slab either rides along as a whole slab or gets a launch of its own with fewer activation
+  // tiles, whichever the same estimate favours (192 x 8192 x 8192: 58 against 52 us).
+  const bool wide_n = (p.n & 63) == 0 && p.n / 64 >= 256 * 4 / 5;
+  auto single = [&](const Params& q, int rows) {
+    return rows <= 16 ? launch_skinny_tt<1, OUT_BF16>(q, stream)
+         : rows <= 32 ? launch_skinny_tt<2, OUT_BF16>(q, stream)
+         : rows <= 64 ? launch_skinny_tt<4, OUT_BF16>(q, stream)
+                      : launch_skinny_cfg<1, 8, OUT_BF16>(q, stream);
+  };
+  int slab = 64;
+  bool own_launch = false;  // for the ragged last slab
+  if (!wide_n) {
+    auto rounds = [&](int64_t slabs) { return ceil_div(slabs * (int64_t)(p.n / 16), 256); };
+    auto unit = [](int rows) { return rows <= 16 ? 40 : rows <= 32 ? 47 : rows <= 64 ? 60 : 100; };
+    int64_t best = INT64_MAX;
+    for (int s : {128, 64, 32}) {
+      const int whole = p.m / s, rest = p.m % s;
+      const int64_t together = unit(s) * rounds(whole + (rest != 0));
+      const int64_t apart = whole && rest ? unit(s) * rounds(whole) + unit(rest) * rounds(1) : INT64_MAX;
+      if (together < best) best = together, slab = s, own_launch = false;
+      if (apart < best) best = apart, slab = s, own_launch = true;
+    }
   }
-  for (; p.m_base < p.m; p.m_base += slab) {
-    const int rows = min(p.m - p.m_base, slab);
-    const int rc = rows <= 16 ? launch_skinny_tt<1, OUT_BF16>(p, stream)
-                 : rows <= 32 ? launch_skinny_tt<2, OUT_BF16>(p, stream)
-                 : rows <= 64 ? launch_skinny_tt<4, OUT_BF16>(p, stream)
-                              : launch_skinny_cfg<1, 8, OUT_BF16>(p, stream);
-    if (rc != NVF_OK) return rc;
-  }
-  return NVF_OK;
+  if (p.m <= slab) return single(p, p.m);
+  const int slabs = own_launch ? p.m / slab : (int)ceil_div(p.m, slab);
+  const int rc = slab == 128 ? launch_skinny_cfg<1, 8, OUT_BF16>(p, stream, slabs)
+               : slab == 64  ? launch_skinny_tt<4, OUT_BF16>(p, stream, slabs)
+                             : launch_skinny_tt<2, OUT_BF16>(p, stream, slabs);
+  if (rc != NVF_OK || !own_launch) return rc;
+  Params last = p;
+  last.m_base = slabs * slab;
+  return single(last, p.m - last.m_base);
 }
 
 template <int BM, int BN, bool OUT_BF16>

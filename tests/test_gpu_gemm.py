@@ -380,9 +380,11 @@ def test_nvfp4_gemm_persistent_kernel_every_scale_code_is_decoded_exactly(dev, s
 @pytest.mark.parametrize("shape", [(1, 16, 128), (7, 96, 256), (16, 48, 384), (17, 304, 1152), (32, 6560, 128), (33, 160, 2048),
                                    (64, 4096, 512), (5, 6592, 1152), (20, 6560, 640), (50, 6560, 256), (16, 64, 8192),
                                    (9, 288, 3200), (48, 144, 1024), (100, 96, 384), (128, 6560, 256), (200, 64, 1152),
-                                   (256, 160, 512), (129, 32, 128), (100, 13056, 128)])
+                                   (256, 160, 512), (129, 32, 128), (100, 13056, 128), (192, 512, 2048), (100, 1024, 256),
+                                   (250, 2048, 384), (150, 1024, 640), (128, 13120, 256)])
 def test_mxfp8_gemm_decode_sized_activations(dev, shape):
-    """M <= 256 (in launches of 128 rows, or of 64 where N is wide) with K % 128 == 0 and N % 16 == 0 takes the kernel that streams the weights once through
+    """M <= 256 (in one launch of slabs of 128, 64 or 32 rows, the last one ragged: 64 where N is wide, else the height that
+    fills the compute units best) with K % 128 == 0 and N % 16 == 0 takes the kernel that streams the weights once through
     per-wavefront LDS rings into v_mfma_scale_f32_16x16x128_f8f6f4: 1 / 2 / 4 / 8 activation tiles, 1 / 2 / 4
     weight-row tiles per workgroup (rings of 3, 2 and 1 slots), activation rows that do not fill a tile,
     all four scale row groups, 1 to 8 chunks per wavefront (wavefronts without work, ring wrap), scales
