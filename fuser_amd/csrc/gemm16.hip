@@ -1054,7 +1054,7 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
   const int kbytes = p.k >> 1;
   const int chunks = p.k >> 7;
   const int sf_padded = p.k >> 4;  // K % 128 == 0: no padding columns
-  int n0, m_loc, grp = 0;
+  int n0, m_loc, grp = 0, asf_word0 = 0;  // asf_word0: which 32-row group of its 128-row scale tile the slab starts in
   int64_t a_row0 = p.m_base, asf_row0 = p.m_base, b_row0 = 0;  // first activation row, its scale row, first weight row
   if constexpr (GROUPED) {
     const int nblocks = p.n / (16 * RT * (NSPLIT ? W : 1));
@@ -1067,10 +1067,13 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
     b_row0 = (int64_t)grp * p.n;
   } else {
     n0 = blockIdx.x * (16 * RT);
-    // activation rows of this workgroup: [m_base, m_base + m_loc); blockIdx.y counts slabs of 128 rows
-    const int m_base = p.m_base + (int)blockIdx.y * 128;
-    a_row0 = asf_row0 = m_base;
-    m_loc = min(p.m - m_base, 128);
+    // activation rows of this workgroup: [m_base, m_base + m_loc); blockIdx.y counts slabs of 16*TT rows
+    // (TT = 2, 4 or 8 when there is more than one, so that a slab lies inside one 32-row scale group)
+    const int m_base = p.m_base + (int)blockIdx.y * (16 * TT);
+    a_row0 = m_base;
+    asf_row0 = m_base & ~127;
+    asf_word0 = (m_base & 127) >> 5;
+    m_loc = min(p.m - m_base, 16 * TT);
   }
   const int tt_count = (m_loc + 15) >> 4;
 
@@ -1130,7 +1133,7 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
   }
 #pragma unroll
   for (int tt = 0; tt < TT; ++tt)
-    rd_asc[tt] = (NT + B_SC + (tt >> 1)) * 1024 + ((tt & 1) * 2 + (g >> 1)) * 256 + r * 16 + ((tt * 16) >> 5) * 4;
+    rd_asc[tt] = (NT + B_SC + (tt >> 1)) * 1024 + ((tt & 1) * 2 + (g >> 1)) * 256 + r * 16 + (asf_word0 + ((tt * 16) >> 5)) * 4;
   const int sc_shift = (g & 1) * 16;
 
   f32x4 acc[RT][TT];
@@ -1303,25 +1306,29 @@ int launch_nvfp4_skinny_tt(const Params& p, int cus, hipStream_t stream, int sla
 }
 
 template <bool OUT_BF16>
-int launch_nvfp4_skinny(const Params& p0, int cus, hipStream_t stream) {
-  // more than 128 rows: slabs of 128, each streaming the weights (the later ones out of the last-level cache);
-  // the whole slabs side by side in one launch, because a slab alone may have too few workgroups for the chip
-  Params p = p0;
-  p.m_base = 0;
-  if (p.m >= 256) {
-    const int whole = p.m / 128;
-    if (const int rc = launch_nvfp4_skinny_tt<8, OUT_BF16>(p, cus, stream, whole)) return rc;
-    p.m_base = whole * 128;
+int launch_nvfp4_skinny(const Params& p, int cus, hipStream_t stream) {
+  // More than 128 rows: slabs, each streaming the weights (the later ones out of the last-level cache), side by
+  // side in one launch (blockIdx.y = slab; the last one may be ragged).  Where N is so small that a workgroup has
+  // 16 weight rows, the slab height is 128, 64 or 32 rows, whichever fills the chip best: every workgroup
+  // converts all activation rows of its slab, lower slabs need less LDS, so that 2 to 4 workgroups share a
+  // compute unit, and with L workgroups per compute unit a launch takes about 17.5 L / 10.3 + 6.5 (L - 1) /
+  // 6.7 + 3.5 (L - 1) us at K = 7168 (measured: 128 x 1024 x 7168 17.6 -> 6.5 us, 256 x 4096 x 7168 34.9 -> 29.8 us).
+  int slab = 128;
+  if (!((p.n & 31) == 0 && p.n / 32 >= (int64_t)cus * 4 / 5)) {
+    auto load = [&](int rows) { return ceil_div(ceil_div(p.m, rows) * (int64_t)(p.n / 16), cus); };
+    const int64_t c128 = 175 * load(128), c64 = 38 + 65 * load(64), c32 = 32 + 35 * load(32);
+    slab = c128 <= c64 && c128 <= c32 ? 128 : (c64 <= c32 ? 64 : 32);
   }
-  for (; p.m_base < p.m; p.m_base += 128) {
-    const int rows = p.m - p.m_base;
-    const int rc = rows <= 16 ? launch_nvfp4_skinny_tt<1, OUT_BF16>(p, cus, stream)
-                 : rows <= 32 ? launch_nvfp4_skinny_tt<2, OUT_BF16>(p, cus, stream)
-                 : rows <= 64 ? launch_nvfp4_skinny_tt<4, OUT_BF16>(p, cus, stream)
-                              : launch_nvfp4_skinny_tt<8, OUT_BF16>(p, cus, stream);
-    if (rc != NVF_OK) return rc;
+  if (p.m > slab) {
+    const int slabs = (int)ceil_div(p.m, slab);
+    return slab == 128 ? launch_nvfp4_skinny_tt<8, OUT_BF16>(p, cus, stream, slabs)
+         : slab == 64  ? launch_nvfp4_skinny_tt<4, OUT_BF16>(p, cus, stream, slabs)
+                       : launch_nvfp4_skinny_tt<2, OUT_BF16>(p, cus, stream, slabs);
   }
-  return NVF_OK;
+  return p.m <= 16 ? launch_nvfp4_skinny_tt<1, OUT_BF16>(p, cus, stream)
+       : p.m <= 32 ? launch_nvfp4_skinny_tt<2, OUT_BF16>(p, cus, stream)
+       : p.m <= 64 ? launch_nvfp4_skinny_tt<4, OUT_BF16>(p, cus, stream)
+                   : launch_nvfp4_skinny_tt<8, OUT_BF16>(p, cus, stream);
 }
 
 // -------------------------------------------------------------------------------------------------
