@@ -30,6 +30,8 @@ SIGNATURES = {
     "nvf_mxfp8_scaled_mm": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _int, _p]),
     "nvf_grouped_mm": (_int, [_p, _p, _p, _p, _p, _int, _i64, _i64, _i64, _int, _p]),
     "nvf_nvfp4_scaled_grouped_mm": (_int, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _int, _i64, _i64, _i64, _int, _p]),
+    "nvf_selftest_fast_division": (_int, [_p, _p]),
+    "nvf_describe_dispatch": (_int, [ctypes.c_char_p, _i64, _i64, _i64, _int, _int, _i64, ctypes.c_char_p, _i64]),
 }
 
 _lib = None
@@ -46,6 +48,13 @@ def lib():
             fn.argtypes = args
         _lib = handle
     return _lib
+
+
+def describe_dispatch(op, m, n, k, groups=1, dtype=BF16, workspace_bytes=0):
+    """Kernels the GEMM entry point `op` would launch for this shape on a whole MI355X (no GPU needed)."""
+    buf = ctypes.create_string_buffer(2048)
+    check(lib().nvf_describe_dispatch(op.encode(), m, n, k, groups, dtype, workspace_bytes, buf, len(buf)))
+    return buf.value.decode()
 
 
 class NvfError(RuntimeError):

@@ -5,6 +5,7 @@
 #include "nvf_internal.h"
 
 #include <cstring>
+#include <string>
 
 namespace nvf {
 
@@ -16,6 +17,35 @@ int fail(int status, const char* fmt, ...) {
   vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
   va_end(ap);
   return status;
+}
+
+static thread_local bool g_plan = false;
+static thread_local std::string g_plan_text;
+
+bool plan_mode() { return g_plan; }
+
+bool note_launch(const char* fmt, ...) {
+  if (!g_plan) return false;
+  char line[256];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(line, sizeof(line), fmt, ap);
+  va_end(ap);
+  if (!g_plan_text.empty()) g_plan_text += "; ";
+  g_plan_text += line;
+  return true;
+}
+
+int cu_count() {
+  static std::atomic<int> cached{0};
+  int n = cached.load(std::memory_order_relaxed);
+  if (n > 0) return n;
+  if (g_plan) return 256;  // a dry run describes the dispatch on a whole MI355X and touches no device
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+    return 256;
+  cached.store(n, std::memory_order_relaxed);
+  return n;
 }
 
 int check_launch(const char* what) {
@@ -234,6 +264,33 @@ int nvf_nvfp4_scaled_grouped_mm(const void* a, const void* b, const void* a_scal
   NVF_REQUIRE_ALIGNED16(a, b, a_scales, b_scales, out);
   Gemm16Args g{a, b, a_scales, b_scales, alphas, out, problem_sizes, expert_offsets, sf_offsets, groups, m, n, k, out_dtype};
   return launch_gemm16(1, g, static_cast<hipStream_t>(stream));
+}
+
+int nvf_selftest_fast_division(uint32_t* result4, void* stream) {
+  NVF_REQUIRE(result4, NVF_ERR_INVALID_ARGUMENT, "NULL buffer");
+  return launch_division_selftest(result4, static_cast<hipStream_t>(stream));
+}
+
+int nvf_describe_dispatch(const char* op, int64_t m, int64_t n, int64_t k, int groups, int dtype, int64_t workspace_bytes,
+                          char* text, int64_t text_bytes) {
+  NVF_REQUIRE(op && text && text_bytes > 0, NVF_ERR_INVALID_ARGUMENT, "NULL argument");
+  // never dereferenced: in plan mode every launcher returns before it touches the device
+  void* const x = reinterpret_cast<void*>(uintptr_t{256});
+  const float* const f = static_cast<const float*>(x);
+  const int32_t* const i = static_cast<const int32_t*>(x);
+  g_plan = true;
+  g_plan_text.clear();
+  int rc;
+  const std::string name(op);
+  if (name == "nvfp4_scaled_mm") rc = nvf_nvfp4_scaled_mm_ws(x, x, x, x, f, x, m, n, k, dtype, workspace_bytes > 0 ? x : nullptr, workspace_bytes, nullptr);
+  else if (name == "nvfp4_scaled_mm_blockscale") rc = nvf_nvfp4_scaled_mm_blockscale(x, x, x, x, f, f, x, x, static_cast<float*>(x), m, n, k, nullptr);
+  else if (name == "mxfp8_scaled_mm") rc = nvf_mxfp8_scaled_mm(x, x, x, x, f, x, m, n, k, dtype, nullptr);
+  else if (name == "grouped_mm") rc = nvf_grouped_mm(x, x, x, i, i, groups, m, n, k, dtype, nullptr);
+  else if (name == "nvfp4_scaled_grouped_mm") rc = nvf_nvfp4_scaled_grouped_mm(x, x, x, x, f, x, i, i, i, groups, m, n, k, dtype, nullptr);
+  else rc = fail(NVF_ERR_INVALID_ARGUMENT, "unknown op %s", op);
+  g_plan = false;
+  snprintf(text, (size_t)text_bytes, "%s", g_plan_text.c_str());
+  return rc;
 }
 
 }  // extern "C"

@@ -669,13 +669,15 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   // fixed 32-bit offsets inside any tile: its row and 16-byte piece, and its scale word (blocks 2*spiece,
   // 2*spiece+1 of the span: 128x4 layout column tile spiece>>1, bytes 2*(spiece&1)..).  A tile's first row is
   // a multiple of 128, so the swizzled scale address splits into the tile's part and the thread's part.
-  struct RowPtrs { const uint8_t *a, *b, *sa, *sb; int a_bytes; };  // a_bytes: bytes of the A rows that exist (buffer range)
+  // a_bytes / a_bytes2: bytes of the existing A rows among the tile's rows 0..127 / 128..255 (buffer ranges)
+  struct RowPtrs { const uint8_t *a, *b, *sa, *sb; int a_bytes, a_bytes2; };
   auto tile_ptrs = [&](int t) {
     const Where w = tile_where(t);
     RowPtrs r;
     r.a = p.a + w.m0 * kbytes;
     // the last tile of a group may have fewer rows than the tile: the rows past the group read as zero
-    r.a_bytes = GROUPED ? w.valid * kbytes : 0x7fffffff;
+    r.a_bytes = GROUPED ? min(w.valid, 128) * kbytes : 0x7fffffff;
+    r.a_bytes2 = GROUPED ? max(w.valid - 128, 0) * kbytes : 0x7fffffff;
     r.b = p.b + ((int64_t)w.g * p.n + w.n0) * kbytes;
     // (a group's activation scales are a slab of their own, swizzled from its first row)
     const int64_t sa_slab = GROUPED ? (int64_t)__builtin_amdgcn_readfirstlane(p.sf_offsets[w.g]) * sf_padded : 0;
@@ -698,7 +700,9 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   auto issue_load_unit = [&](Raw& r, int q) {
     const int o = l_mac * 64, so = l_mac * 1024;
     if (q == 0) r.a[0] = __builtin_amdgcn_raw_buffer_load_b128(rsrc(lp.a, lp.a_bytes), off_ab, o, 0);
-    if (q == 1 && AR == 2) r.a[1] = __builtin_amdgcn_raw_buffer_load_b128(rsrc(lp.a, lp.a_bytes), off_ab, o + (int)row128, 0);
+    // (rows 128.. of the tile through a resource of their own, so that the range check that zeroes the rows past a
+    // group never depends on whether the hardware counts the scalar offset)
+    if (q == 1 && AR == 2) r.a[1] = __builtin_amdgcn_raw_buffer_load_b128(rsrc(lp.a + row128, lp.a_bytes2), off_ab, o, 0);
     if (q == 2) r.b[0] = __builtin_amdgcn_raw_buffer_load_b128(rsrc(lp.b), off_ab, o, 0);
     if (q == 3) r.b[1] = __builtin_amdgcn_raw_buffer_load_b128(rsrc(lp.b), off_ab, o + (int)row128, 0);
     if (q == 4) r.sa[0] = __builtin_amdgcn_raw_buffer_load_b16(rsrc(lp.sa), off_sf, so, 0);
@@ -711,6 +715,7 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
     l_mac = wrap ? 0 : l_mac + 1;
     lp.a = wrap ? np.a : lp.a;
     lp.a_bytes = wrap ? np.a_bytes : lp.a_bytes;
+    lp.a_bytes2 = wrap ? np.a_bytes2 : lp.a_bytes2;
     lp.b = wrap ? np.b : lp.b;
     lp.sa = wrap ? np.sa : lp.sa;
     lp.sb = wrap ? np.sb : lp.sb;
@@ -969,12 +974,15 @@ template <bool OUT_BF16, bool GROUPED, int TM, bool OUT_F32, bool PAIRS>
 int launch_nvfp4_fast_cfg(const Params& p, int cus, hipStream_t stream) {
   auto kern = nvfp4_gemm_256_kernel<OUT_BF16, GROUPED, TM, OUT_F32, PAIRS>;
   constexpr int lds_bytes = 2 * (64 * TM + 256) * 128 + 8 * 2560;  // 128 KiB / 96 KiB of tiles + the epilogue's 20 KiB
-  static uint64_t configured = 0;  // one bit per device; a benign race: the attribute call is idempotent
-  if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
   // grouped: an upper bound (128-row tiles: one per weight panel and group of at least rows_lo rows)
   const int64_t tiles_m = (GROUPED && TM == 2) ? std::min<int64_t>(p.groups, p.m / std::max(p.rows_lo, 1)) : p.m / (64 * TM);
   const int64_t tiles = tiles_m * (p.n / 256);
   const unsigned grid = (unsigned)(tiles >= cus ? (cus & ~7) : ((tiles + 7) / 8) * 8);
+  if (note_launch("nvfp4_gemm_256_kernel<grouped=%d,TM=%d,f32=%d,pairs=%d> grid=%u rows=%d..%d min_rows=%d", (int)GROUPED, TM, (int)OUT_F32,
+                  (int)PAIRS, grid, p.rows_lo, p.rows_hi, p.min_rows))
+    return NVF_OK;
+  static std::atomic<uint64_t> configured{0};  // one bit per device
+  if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds_bytes, stream, p);
   return check_launch("nvfp4_gemm_256_kernel");
 }
@@ -1011,7 +1019,7 @@ int launch_nvfp4_fast(const Params& p, int cus, hipStream_t stream) {
 // Issued from inline assembly: the compiler neither waits for it nor orders LDS reads against it, the
 // kernels do that with explicit s_waitcnt vmcnt(n).
 __device__ __forceinline__ void lds_dma16(uint32_t lds_byte_addr, const uint8_t* base, uint32_t voff) {
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_byte_addr), "v"(voff), "s"(base) : "memory");
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_byte_addr), "v"(voff), "s"(base) : "memory", "m0");
 }
 
 // 32 packed e2m1 values and their two e4m3 block scales -> four MFMA operands of 8 fp16 values
@@ -1266,7 +1274,8 @@ int launch_nvfp4_skinny_ring_cfg(const Params& p, hipStream_t stream, int slabs 
   constexpr int ring_kib = 8 * DEPTH * SLOT_KIB;
   constexpr int lds_bytes = (ring_kib > red_kib ? ring_kib : red_kib) * 1024;
   static_assert(lds_bytes <= 160 * 1024, "LDS");
-  static uint64_t configured = 0;  // one bit per device; a benign race: the attribute call is idempotent
+  if (note_launch("nvfp4_skinny_ring_kernel<RT=%d,TT=%d> grid=%ux%d", RT, TT, (unsigned)(p.n / (16 * RT)), slabs)) return NVF_OK;
+  static std::atomic<uint64_t> configured{0};  // one bit per device
   if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
   hipLaunchKernelGGL(kern, dim3((unsigned)(p.n / (16 * RT)), (unsigned)slabs), dim3(512), lds_bytes, stream, p);
   return check_launch("nvfp4_skinny_ring_kernel");
@@ -1284,13 +1293,16 @@ int launch_nvfp4_skinny_grouped(const Params& p0, int rows_lo, int rows_hi, hipS
   constexpr int ring_kib = 8 * DEPTH * SLOT_KIB;
   constexpr int lds_bytes = (ring_kib > red_kib ? ring_kib : red_kib) * 1024;
   static_assert(lds_bytes <= 160 * 1024, "LDS");
-  static uint64_t configured = 0;  // one bit per device; a benign race: the attribute call is idempotent
-  if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
   Params p = p0;
   p.rows_lo = rows_lo;
   p.rows_hi = rows_hi;
   const int64_t wgs = (int64_t)p.groups * (p.n / (16 * RT * (NSPLIT ? 8 : 1)));
   if (wgs >= ((int64_t)1 << 31)) return fail(NVF_ERR_UNSUPPORTED_SHAPE, "too many (group, row block) pairs for one launch");
+  if (note_launch("nvfp4_skinny_ring_kernel<RT=%d,TT=%d,grouped,nsplit=%d> grid=%lld rows=%d..%d", RT, TT, (int)NSPLIT, (long long)wgs, rows_lo,
+                  rows_hi))
+    return NVF_OK;
+  static std::atomic<uint64_t> configured{0};  // one bit per device
+  if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
   hipLaunchKernelGGL(kern, dim3((unsigned)wgs), dim3(512), lds_bytes, stream, p);
   return check_launch("nvfp4_skinny_ring_kernel (grouped)");
 }
@@ -1602,7 +1614,8 @@ template <bool BF16_MMA, bool OUT_BF16, bool STREAM_OUT>
 int launch_grouped16_fast_cfg(const Params& p, int cus, hipStream_t stream) {
   auto kern = grouped16_gemm_256_kernel<BF16_MMA, OUT_BF16, STREAM_OUT>;
   constexpr int lds_bytes = 2 * 2 * 2048 * 16 + 4 * 4608;  // 128 KiB of tiles + the epilogue's 18 KiB
-  static uint64_t configured = 0;  // one bit per device; a benign race: the attribute call is idempotent
+  if (note_launch("grouped16_gemm_256_kernel<stream_out=%d> grid=%d", (int)STREAM_OUT, cus & ~7)) return NVF_OK;
+  static std::atomic<uint64_t> configured{0};  // one bit per device
   if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
   hipLaunchKernelGGL(kern, dim3((unsigned)(cus & ~7)), dim3(256), lds_bytes, stream, p);
   return check_launch("grouped16_gemm_256_kernel");
@@ -1622,7 +1635,8 @@ template <int BM, int BN, bool BF16_MMA, bool OUT_BF16>
 int launch_cfg(const Params& p, int grid, hipStream_t stream) {
   auto kern = gemm16_kernel<BM, BN, BF16_MMA, OUT_BF16>;
   constexpr int lds_bytes = 2 * (BM + BN) * 128;
-  static uint64_t configured = 0;  // one bit per device; a benign race: the attribute call is idempotent
+  if (note_launch("gemm16_kernel<%d,%d> grid=%d", BM, BN, grid)) return NVF_OK;
+  static std::atomic<uint64_t> configured{0};  // one bit per device
   if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_bytes, stream, p);
   return check_launch("gemm16_kernel");
@@ -1632,7 +1646,9 @@ template <int BM, int BN, bool OUT_BF16, bool OUT_F32 = false>
 int launch_nvfp4_tile(const Params& p, int grid, hipStream_t stream) {
   auto kern = nvfp4_tile_kernel<BM, BN, OUT_BF16, OUT_F32>;
   constexpr int lds_bytes = 2 * (BM + BN) * 128;
-  static uint64_t configured = 0;  // one bit per device; a benign race: the attribute call is idempotent
+  if (note_launch("nvfp4_tile_kernel<%d,%d,f32=%d> grid=%d skip_whole_256=%d min_rows=%d", BM, BN, (int)OUT_F32, grid, p.skip_whole_256, p.min_rows))
+    return NVF_OK;
+  static std::atomic<uint64_t> configured{0};  // one bit per device
   if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_bytes, stream, p);
   return check_launch("nvfp4_tile_kernel");
@@ -1660,9 +1676,10 @@ int launch_nvfp4_splitk(const Params& p0, int splits, float* workspace, hipStrea
   p.partial = workspace;
   auto kern = nvfp4_tile_kernel<128, 128, OUT_BF16, false, true>;
   constexpr int lds_bytes = 2 * (128 + 128) * 128;
-  static uint64_t configured = 0;  // one bit per device; a benign race: the attribute call is idempotent
-  if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
   const int64_t items = ceil_div(p.m, 128) * ceil_div(p.n, 128) * p.splits;
+  if (note_launch("nvfp4_tile_kernel<128,128,split_k> grid=%lld splits=%d + splitk_reduce_kernel", (long long)items, p.splits)) return NVF_OK;
+  static std::atomic<uint64_t> configured{0};  // one bit per device
+  if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
   hipLaunchKernelGGL(kern, dim3((unsigned)items), dim3(256), lds_bytes, stream, p);
   int rc = check_launch("nvfp4_tile_kernel (split K)");
   if (rc != NVF_OK) return rc;
@@ -1792,18 +1809,6 @@ int launch_nvfp4_f32(const Params& p, int cus, hipStream_t stream) {
   }
   const int64_t t = tiles(64, 64);
   return launch_nvfp4_tile<64, 64, false, true>(p, (int)(t < 4 * cus ? t : 4 * cus), stream);
-}
-
-int cu_count() {
-  static int cached = 0;
-  if (cached == 0) {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
-      cached = n;
-    else
-      return 256;
-  }
-  return cached;
 }
 
 }  // namespace

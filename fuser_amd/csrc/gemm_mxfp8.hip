@@ -28,7 +28,7 @@ struct Params {
   const float* alpha;
   void* out;
   int m, n, k;
-  int m_base = 0;  // skinny kernel: first activation row this launch computes, a multiple of 64
+  int m_base = 0;  // skinny kernel: first activation row this launch computes, a multiple of the slab height (32, 64 or 128)
 };
 
 __device__ __forceinline__ uint32_t pack2(float a, float b, bool out_bf16) {
@@ -227,7 +227,7 @@ __device__ __forceinline__ int lds_pos2(int row, int chunk) { return row * 8 + (
 
 __device__ __forceinline__ void lds_dma16(uint32_t lds_byte_addr, const uint8_t* base, uint32_t voff) {
   // lds_byte_addr and base are wave-uniform; lane L's 16 bytes land at lds_byte_addr + 16 * L
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_byte_addr), "v"(voff), "s"(base) : "memory");
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_byte_addr), "v"(voff), "s"(base) : "memory", "m0");
 }
 
 // TM = 32-row accumulator tiles of a wavefront along M: 4 -> 256x256 workgroup tile, 2 -> 128x256 (for shapes
@@ -501,11 +501,12 @@ template <int TM, bool OUT_BF16, bool STREAM_OUT>
 int launch_fast_cfg(const Params& p, hipStream_t stream) {
   auto kern = mxfp8_gemm_256_kernel<TM, OUT_BF16, STREAM_OUT>;
   constexpr int lds_bytes = 2 * (64 * TM + 256) * 128 + 4 * 4608;  // 128 KiB / 96 KiB of tiles + the epilogue's 18 KiB
-  static uint64_t configured = 0;  // one bit per device; a benign race: the attribute call is idempotent
-  if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
   const int64_t tiles = (int64_t)(p.m / (64 * TM)) * (p.n / 256);
-  const int cus = 256;
+  const int cus = cu_count() & ~7;  // workgroup ids are dealt round-robin to the 8 XCDs
   const unsigned grid = (unsigned)(tiles >= cus ? cus : ((tiles + 7) / 8) * 8);
+  if (note_launch("mxfp8_gemm_256_kernel<TM=%d,stream_out=%d> grid=%u", TM, (int)STREAM_OUT, grid)) return NVF_OK;
+  static std::atomic<uint64_t> configured{0};  // one bit per device
+  if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_bytes, stream, p);
   return check_launch("mxfp8_gemm_256_kernel");
 }
@@ -700,7 +701,8 @@ int launch_skinny_cfg(const Params& p, hipStream_t stream, int slabs = 1) {
   constexpr int ring = 8 * DEPTH * SLOT, red = 8 * RT * TT * 1024;
   constexpr int lds_bytes = ring > red ? ring : red;
   static_assert(lds_bytes <= 160 * 1024, "LDS");
-  static uint64_t configured = 0;  // one bit per device; a benign race: the attribute call is idempotent
+  if (note_launch("mxfp8_skinny_kernel<RT=%d,TT=%d> grid=%ux%d m_base=%d", RT, TT, (unsigned)(p.n / (16 * RT)), slabs, p.m_base)) return NVF_OK;
+  static std::atomic<uint64_t> configured{0};  // one bit per device
   if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
   hipLaunchKernelGGL(kern, dim3((unsigned)(p.n / (16 * RT)), (unsigned)slabs), dim3(512), lds_bytes, stream, p);
   return check_launch("mxfp8_skinny_kernel");
@@ -709,7 +711,7 @@ int launch_skinny_cfg(const Params& p, hipStream_t stream, int slabs = 1) {
 template <int TT, bool OUT_BF16>
 int launch_skinny_tt(const Params& p, hipStream_t stream, int slabs = 1) {
   // as many weight rows per workgroup as still leaves about one workgroup per compute unit
-  const int64_t want = 256 * 4 / 5;
+  const int64_t want = (int64_t)cu_count() * 4 / 5;
   if ((p.n & 63) == 0 && p.n / 64 >= want) return launch_skinny_cfg<4, TT, OUT_BF16>(p, stream, slabs);
   if ((p.n & 31) == 0 && p.n / 32 >= want) return launch_skinny_cfg<2, TT, OUT_BF16>(p, stream, slabs);
   return launch_skinny_cfg<1, TT, OUT_BF16>(p, stream, slabs);
@@ -726,7 +728,8 @@ int launch_skinny(const Params& p, hipStream_t stream) {
   // (128 x 2048 x 7168: 11.4 -> 8.3 us, 192 x 512 x 7168: 18.2 -> 5.9 us, 512 x 512 x 7168: 13.9 -> 8.8 us).
   // A ragged last slab either rides along as a whole slab or gets a launch of its own with fewer activation
   // tiles, whichever the same estimate favours (192 x 8192 x 8192: 58 against 52 us).
-  const bool wide_n = (p.n & 63) == 0 && p.n / 64 >= 256 * 4 / 5;
+  const int64_t cus = cu_count();
+  const bool wide_n = (p.n & 63) == 0 && p.n / 64 >= cus * 4 / 5;
   auto single = [&](const Params& q, int rows) {
     return rows <= 16 ? launch_skinny_tt<1, OUT_BF16>(q, stream)
          : rows <= 32 ? launch_skinny_tt<2, OUT_BF16>(q, stream)
@@ -736,7 +739,7 @@ int launch_skinny(const Params& p, hipStream_t stream) {
   int slab = 64;
   bool own_launch = false;  // for the ragged last slab
   if (!wide_n) {
-    auto rounds = [&](int64_t slabs) { return ceil_div(slabs * (int64_t)(p.n / 16), 256); };
+    auto rounds = [&](int64_t slabs) { return ceil_div(slabs * (int64_t)(p.n / 16), cus); };
     auto unit = [](int rows) { return rows <= 16 ? 40 : rows <= 32 ? 47 : rows <= 64 ? 60 : 100; };
     int64_t best = INT64_MAX;
     for (int s : {128, 64, 32}) {
@@ -762,9 +765,10 @@ template <int BM, int BN, bool OUT_BF16>
 int launch_cfg(const Params& p, hipStream_t stream) {
   auto kern = mxfp8_gemm_kernel<BM, BN, OUT_BF16>;
   constexpr int lds_bytes = 2 * (BM + BN) * 128;
-  static uint64_t configured = 0;  // one bit per device; a benign race: the attribute call is idempotent
-  if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
   const int64_t tiles = ceil_div(p.m, BM) * ceil_div(p.n, BN);
+  if (note_launch("mxfp8_gemm_kernel<%d,%d> grid=%lld", BM, BN, (long long)tiles)) return NVF_OK;
+  static std::atomic<uint64_t> configured{0};  // one bit per device
+  if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
   hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(256), lds_bytes, stream, p);
   return check_launch("mxfp8_gemm_kernel");
 }
@@ -778,15 +782,16 @@ int launch_sized(const Params& p, hipStream_t stream) {
   // kernel's workgroups (one per 128 rows x 16 columns, K split over their wavefronts) then fill it.  A round
   // of them costs about a quarter of a round of 128x256 tiles, so up to 3 rounds win or tie (measured, K >= 2048:
   // 512 x 2048 x 7168 in 27 instead of 59 us, 384 x 3072 x 7168 in 39 instead of 62, 384 x 4096 x 4096 27 both).
-  const int64_t skinny_rounds = ceil_div(ceil_div(p.m, 128) * (int64_t)(p.n / 16), 256);
+  const int64_t cus = cu_count();
+  const int64_t skinny_rounds = ceil_div(ceil_div(p.m, 128) * (int64_t)(p.n / 16), cus);
   const bool fast_ok = (p.k & 127) == 0 && p.k >= 256 && (p.m & 127) == 0 && (p.n & 255) == 0 && (int64_t)p.k * 256 < (1ll << 31);
   // Exception: 128 or 256 rows and a wide N.  Per 1024 of K a round of skinny workgroups costs about 1.7 us with
   // 128-row slabs and 3.4 us with the 64-row slabs of a wide N (which are launches of their own), a round of
   // 128x256 tiles 6.8 us: where one round of those tiles covers the shape, it wins from about N = 10240 at 256
   // rows (measured: 256 x 14336 x 4096 in 31 instead of 55 us, 256 x 28672 x 4096 in 34 instead of 104 us).
-  const bool wide_n = (p.n & 63) == 0 && p.n / 64 >= 256 * 4 / 5;
-  const int64_t skinny_cost = wide_n ? 34 * ceil_div(p.m, 64) * ceil_div(p.n / 64, 256) : 17 * skinny_rounds;
-  const bool wide_256 = fast_ok && p.m <= 256 && tiles(128, 256) >= 48 && 68 * ceil_div(tiles(128, 256), 256) < skinny_cost;
+  const bool wide_n = (p.n & 63) == 0 && p.n / 64 >= cus * 4 / 5;
+  const int64_t skinny_cost = wide_n ? 34 * ceil_div(p.m, 64) * ceil_div(p.n / 64, cus) : 17 * skinny_rounds;
+  const bool wide_256 = fast_ok && p.m <= 256 && tiles(128, 256) >= 48 && 68 * ceil_div(tiles(128, 256), cus) < skinny_cost;
   if (!wide_256 && (p.m <= 256 || (skinny_rounds <= 3 && p.k >= 2048)) && (p.k & 127) == 0 && (p.n & 15) == 0 &&
       (int64_t)p.k * 64 < (1ll << 31))  // 32-bit lane offsets
     return launch_skinny<OUT_BF16>(p, stream);
@@ -794,15 +799,14 @@ int launch_sized(const Params& p, hipStream_t stream) {
     // Persistent LDS-direct kernel with 256x256 or 128x256 tiles: a 128-row tile costs about 0.61 of a 256-row
     // tile (half the flops at 82 % of the rate, measured), and the time goes with the rounds of tiles over the
     // compute units; below 48 tiles the tile kernels further down do as well.
-    const int64_t cus = 256;
     const int64_t t256 = (p.m & 255) == 0 ? tiles(256, 256) : 0, t128 = tiles(128, 256);
     const int64_t cost256 = t256 ? 100 * ceil_div(t256, cus) : INT64_MAX;
     const int64_t cost128 = 61 * ceil_div(t128, cus);
     if (t256 >= 128 && cost256 <= cost128) return launch_fast<4, OUT_BF16>(p, stream);
     if (t128 >= 48) return launch_fast<2, OUT_BF16>(p, stream);
   }
-  if (tiles(256, 256) >= 256) return launch_cfg<256, 256, OUT_BF16>(p, stream);
-  if (tiles(128, 128) >= 256) return launch_cfg<128, 128, OUT_BF16>(p, stream);
+  if (tiles(256, 256) >= cus) return launch_cfg<256, 256, OUT_BF16>(p, stream);
+  if (tiles(128, 128) >= cus) return launch_cfg<128, 128, OUT_BF16>(p, stream);
   return launch_cfg<64, 64, OUT_BF16>(p, stream);
 }
 

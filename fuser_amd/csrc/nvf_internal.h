@@ -2,6 +2,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 
@@ -15,15 +16,24 @@ int fail(int status, const char* fmt, ...) __attribute__((format(printf, 2, 3)))
 // Checks the launch that was just issued on the calling thread.
 int check_launch(const char* what);
 
-// Raises a kernel's dynamic LDS limit on the current device, once per device (`done`: one bit per device id).
-inline int allow_dynamic_lds(const void* kernel, int bytes, uint64_t& done) {
+// Dry run of a dispatch (nvf_describe_dispatch): while the calling thread is in plan mode, launchers
+// record the kernel they would start and return before any HIP call.  note_launch() returns true in that mode.
+bool plan_mode();
+bool note_launch(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
+
+// Compute units of the current device, cached per process (256 when no device can be asked, as in a dry run).
+int cu_count();
+
+// Raises a kernel's dynamic LDS limit on the current device, once per device (`done`: one bit per device id;
+// the attribute call is idempotent, so two threads that both find the bit clear do no harm).
+inline int allow_dynamic_lds(const void* kernel, int bytes, std::atomic<uint64_t>& done) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return fail(NVF_ERR_NO_DEVICE, "hipGetDevice failed");
   const uint64_t bit = 1ull << (dev & 63);
-  if (done & bit) return NVF_OK;
+  if (done.load(std::memory_order_acquire) & bit) return NVF_OK;
   const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
   if (e != hipSuccess) return fail(NVF_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-  done |= bit;
+  done.fetch_or(bit, std::memory_order_release);
   return NVF_OK;
 }
 
@@ -50,6 +60,7 @@ int launch_preprocess_sf(const void* in, int elem_size, int64_t rows, int64_t co
 int launch_mxfp8_quantize(const void* in, int in_dtype, int64_t rows, int64_t cols, int swizzle, void* out_fp8,
                           void* out_sf, hipStream_t stream);
 int launch_cast(int kind, const float* in, int64_t n, uint8_t* out, hipStream_t stream);
+int launch_division_selftest(uint32_t* out4, hipStream_t stream);
 
 // op: 0 dense NVFP4, 1 grouped NVFP4, 2 grouped bf16/f16
 struct Gemm16Args {

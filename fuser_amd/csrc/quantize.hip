@@ -55,8 +55,9 @@ __device__ __forceinline__ int find_group(const int32_t* __restrict__ offsets, i
 //     are merged by the caches before they reach HBM.
 //   * amax/6 and 1/x use a 3-instruction division (reciprocal constant resp. v_rcp_f32, one fused
 //     residual correction); for biased exponents in [2, 250] it returns exactly the IEEE quotient for
-//     every fp32 input (checked exhaustively on the GPU); anything else (zero, denormal, huge, Inf, NaN)
-//     makes the wavefront redo the block scale with true divisions.
+//     every fp32 input (nvf_selftest_fast_division compares every such pattern with true division on the
+//     device), and for a zero operand both forms end in the same result (0 resp. FLT_MAX after the clamp);
+//     anything else (denormal, huge, Inf, NaN) makes the wavefront redo the block scale with true divisions.
 // -------------------------------------------------------------------------------------------------
 // 16 consecutive elements: the raw 16-byte loads are issued first and decoded to fp32 later, so that
 // address-independent work (group lookup, global scale) overlaps the memory latency. Inactive lanes load
@@ -115,8 +116,13 @@ __device__ __forceinline__ void decode16(const Raw16<float>& r, bool active, flo
   }
 }
 
-// true when the 3-instruction divisions below are exact for this operand
-__device__ __forceinline__ bool fast_div_ok(float v) { return ((f32_to_bits(v) >> 23) & 0xffu) - 2u <= 248u; }
+// true when the 3-instruction divisions below give the result of the true division for this operand: biased
+// exponent in [2, 250], or +0 (amax / 6 = 0 exactly; 1 / 0: v_rcp gives +Inf, the correction step NaN, and
+// fminf(NaN, FLT_MAX) = FLT_MAX = fminf(+Inf, FLT_MAX))
+__device__ __forceinline__ bool fast_div_ok(float v) {
+  const uint32_t b = f32_to_bits(v);
+  return ((b >> 23) & 0xffu) - 2u <= 248u || b == 0u;
+}
 __device__ __forceinline__ float fast_div6(float m) {
   const float r6 = 0x1.555556p-3f;  // RN(1/6)
   const float q0 = m * r6;
@@ -273,6 +279,7 @@ int launch_nvfp4_layout(const T* in, const T* in_up, int64_t rows, int64_t cols,
   const int64_t wgs = ceil_div(cover, 4) * segs;
   if (wgs >= ((int64_t)1 << 31)) return fail(NVF_ERR_UNSUPPORTED_SHAPE, "tensor of %lld x %lld is too large for one launch",
                                              (long long)rows, (long long)cols);
+  if (note_launch("nvfp4_quantize_kernel<layout=%d> grid=%lld", LAYOUT, (long long)wgs)) return NVF_OK;
   hipLaunchKernelGGL((nvfp4_quantize_kernel<T, LAYOUT, SILU_MUL>), dim3((unsigned)wgs), dim3(256), 0, stream, in, in_up, rows,
                      cols, gs, in_off, out_off, groups, (uint32_t)segs, out_fp4, out_sf);
   return check_launch("nvfp4_quantize_kernel");
@@ -587,6 +594,33 @@ int launch_preprocess_sf(const void* in, int elem_size, int64_t rows, int64_t co
       return fail(NVF_ERR_INVALID_ARGUMENT, "element size %d is not 1, 2 or 4", elem_size);
   }
   return check_launch("preprocess_sf_kernel");
+}
+
+namespace {
+// Every fp32 pattern with biased exponent in [2, 250] (both signs are the same arithmetic; positive ones are
+// what the quantizer meets): the 3-instruction forms against true division.  out[0] / out[2] count the
+// mismatches of 1/x and x/6, out[1] / out[3] hold the smallest mismatching pattern (0xffffffff: none).
+__global__ __launch_bounds__(256) void division_selftest_kernel(uint32_t* __restrict__ out) {
+  uint32_t bad_rcp = 0, bad_div = 0, first_rcp = 0xffffffffu, first_div = 0xffffffffu;
+  const uint32_t mant = blockIdx.x * 256u + threadIdx.x;  // 2^15 workgroups x 256 = every 23-bit mantissa
+  for (uint32_t e = 2; e <= 250; ++e) {
+    const uint32_t bits = (e << 23) | mant;
+    const float v = bits_to_f32(bits);
+    if (f32_to_bits(fast_rcp(v)) != f32_to_bits(1.0f / v)) { ++bad_rcp; first_rcp = min(first_rcp, bits); }
+    if (f32_to_bits(fast_div6(v)) != f32_to_bits(v / 6.0f)) { ++bad_div; first_div = min(first_div, bits); }
+  }
+  if (bad_rcp) { atomicAdd(out + 0, bad_rcp); atomicMin(out + 1, first_rcp); }
+  if (bad_div) { atomicAdd(out + 2, bad_div); atomicMin(out + 3, first_div); }
+}
+__global__ void division_selftest_init_kernel(uint32_t* out) {
+  out[0] = 0; out[1] = 0xffffffffu; out[2] = 0; out[3] = 0xffffffffu;
+}
+}  // namespace
+
+int launch_division_selftest(uint32_t* out4, hipStream_t stream) {
+  hipLaunchKernelGGL(division_selftest_init_kernel, dim3(1), dim3(1), 0, stream, out4);
+  hipLaunchKernelGGL(division_selftest_kernel, dim3(1u << 15), dim3(256), 0, stream, out4);
+  return check_launch("division_selftest_kernel");
 }
 
 int launch_cast(int kind, const float* in, int64_t n, uint8_t* out, hipStream_t stream) {

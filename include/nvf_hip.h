@@ -184,6 +184,22 @@ NVF_API int nvf_nvfp4_scaled_grouped_mm(const void* a, const void* b, const void
                                         const int32_t* sf_offsets, int groups, int64_t m, int64_t n,
                                         int64_t k, int out_dtype, void* stream);
 
+/* No counterpart in the reference: a self-check of the NVFP4 quantizer's arithmetic on the current device.  The
+ * quantizer evaluates amax / 6 and 1 / x (runtime/block_quantization_kernels.cu:224, :237-239) as a reciprocal
+ * with one fused correction step; this compares both forms with true fp32 division for EVERY fp32 pattern with
+ * biased exponent in [2, 250] (the operands for which the quantizer uses them).  result4: 4 device uint32 =
+ * { mismatches of 1/x, smallest mismatching bit pattern or 0xffffffff, the same two for x/6 }. */
+NVF_API int nvf_selftest_fast_division(uint32_t* result4, void* stream);
+
+/* No counterpart in the reference (its CUTLASS heuristics are not observable either): a dry run of the
+ * dispatch of one GEMM entry point.  Writes into text (text_bytes including the terminator) the kernels the call
+ * would launch on a whole MI355X, in launch order, as "kernel<variant> grid=..; ..", and touches no device -
+ * it works without a GPU.  op: "nvfp4_scaled_mm" (workspace_bytes as given to nvf_nvfp4_scaled_mm_ws),
+ * "nvfp4_scaled_mm_blockscale", "mxfp8_scaled_mm", "grouped_mm", "nvfp4_scaled_grouped_mm" (m = total rows).
+ * Returns the status the real call would return from its argument checks. */
+NVF_API int nvf_describe_dispatch(const char* op, int64_t m, int64_t n, int64_t k, int groups, int dtype,
+                                  int64_t workspace_bytes, char* text, int64_t text_bytes);
+
 #ifdef __cplusplus
 }
 #endif

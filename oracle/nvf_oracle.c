@@ -310,17 +310,6 @@ ORC_API void orc_dequantize_mxfp8(const uint8_t* fp8, const uint8_t* sf_swizzled
     }
 }
 
-/* C[m,n] = sum_k A[m,k] * B[n,k], double accumulation; the textbook contraction
- * the reference tests compare against (torch.matmul(a, b.t())). */
-ORC_API void orc_matmul_nt(const float* a, const float* b, int64_t m, int64_t n, int64_t k, float* c) {
-  for (int64_t i = 0; i < m; ++i)
-    for (int64_t j = 0; j < n; ++j) {
-      double acc = 0.0;
-      for (int64_t p = 0; p < k; ++p) acc += (double)a[i * k + p] * (double)b[j * k + p];
-      c[i * n + j] = (float)acc;
-    }
-}
-
 /* bulk helpers so that tests can sweep whole input spaces without Python loops */
 ORC_API void orc_f32_to_e2m1_n(const float* x, int64_t n, uint8_t* out) {
   for (int64_t i = 0; i < n; ++i) out[i] = orc_f32_to_e2m1(x[i]);

@@ -45,7 +45,6 @@ def _load():
         "orc_block_quantize_mxfp8": (None, [c_p, c_int, c_i64, c_i64, c_p, c_p]),
         "orc_dequantize_nvfp4": (None, [c_p, c_p, c_i64, c_i64, c_f, c_p]),
         "orc_dequantize_mxfp8": (None, [c_p, c_p, c_i64, c_i64, c_p]),
-        "orc_matmul_nt": (None, [c_p, c_p, c_i64, c_i64, c_i64, c_p]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)

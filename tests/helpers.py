@@ -8,8 +8,11 @@ from oracle import nvf_oracle as O
 
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 
-# GEMM tolerance of this build: max |out - ref| <= 1e-2 * max |ref| against the fp32
-# dequantize+matmul oracle.  bf16 rounding of the output alone contributes up to 2^-9 = 2e-3.
+# GEMM tolerance of this build: 1e-2 "max-rel" against the fp32 dequantize+matmul oracle, where max-rel is
+# max |out - ref| / max |ref| -- over the whole output (max_rel) or, stricter, row by row (max_rel_rowwise: an
+# error confined to a row of small magnitude cannot hide behind a large element elsewhere).  It is not an
+# element-wise relative error: elements near zero have none.  bf16 rounding of the output alone contributes
+# up to 2^-9 = 2e-3; observed values are 2-4e-3.
 GEMM_MAX_REL = 1e-2
 
 
@@ -24,6 +27,12 @@ def all_bf16_as_f32():
 def max_rel(out, ref):
     out = out.float().cpu()
     return ((out - ref).abs().max() / ref.abs().max()).item()
+
+
+def max_rel_rowwise(out, ref):
+    out = out.float().cpu()
+    scale = ref.abs().amax(dim=1, keepdim=True).clamp(min=1e-30)
+    return ((out - ref).abs() / scale).max().item()
 
 
 def gs_of(x):

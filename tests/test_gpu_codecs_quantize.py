@@ -230,3 +230,42 @@ def test_quantizer_through_raw_c_abi_on_a_side_stream(dev):
                                                    ctypes.c_void_p(stream.cuda_stream)))
     stream.synchronize()
     assert torch.equal(q.cpu(), rq) and torch.equal(s.cpu(), rs)
+
+
+def test_quantizer_division_shortcuts_equal_true_division_for_every_operand(dev):
+    """amax / 6 and 1 / x inside the NVFP4 quantizer are a reciprocal plus one fused correction step; the library's
+    self-check compares both with true fp32 division on the device for every fp32 pattern with biased exponent in
+    [2, 250] (2.09e9 operands each) -- the range for which the kernel uses them."""
+    from fuser_amd import capi
+
+    res = torch.full((4,), 7, dtype=torch.int32, device=dev)
+    capi.check(capi.lib().nvf_selftest_fast_division(res.data_ptr(), None))
+    torch.cuda.synchronize()
+    bad_rcp, first_rcp, bad_div, first_div = [int(v) & 0xFFFFFFFF for v in res.cpu().tolist()]
+    assert bad_rcp == 0 and first_rcp == 0xFFFFFFFF, f"1/x differs for {bad_rcp} operands, first {first_rcp:#010x}"
+    assert bad_div == 0 and first_div == 0xFFFFFFFF, f"x/6 differs for {bad_div} operands, first {first_div:#010x}"
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_nvfp4_quantizer_zero_and_tiny_blocks_next_to_ordinary_ones(dev, dtype):
+    """All-zero blocks (padded or sparse activations) take the quantizer's ordinary path; blocks whose amax is
+    denormal or whose scale underflows to zero sit in the same wavefronts as N(0,1) blocks: bytes equal the oracle."""
+    from fuser_amd import ops
+
+    gen = torch.Generator().manual_seed(12)
+    x = torch.randn(256, 2048, generator=gen)
+    blocks = x.view(256, 128, 16)
+    blocks[::3, ::2] = 0.0                       # zero blocks interleaved with ordinary ones
+    blocks[1::7, 1::5] *= 1e-30                  # tiny amax: the scale rounds to zero
+    if dtype == torch.float32:
+        blocks[2::11, 3::9] *= 1e-42             # fp32 denormals
+    blocks[5, 7] = 0.0
+    blocks[5, 7, 3] = 2.0 ** -20
+    x = x.to(dtype)
+    for gs in (None, 2688.0 / 4.5, 1e-3):
+        gst = None if gs is None else torch.tensor(gs, device=dev)
+        for swz in (False, True):
+            q, s = ops.nv_block_quantize(x.to(dev), gst, swz, 16)
+            rq, rs = O.block_quantize_nvfp4(x, gs, swz)
+            assert torch.equal(q.view(torch.uint8).cpu(), rq), (gs, swz)
+            assert torch.equal(s.view(torch.uint8).cpu(), rs), (gs, swz)
