@@ -6,6 +6,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libnvf_hip.so")
 
 F32, BF16, F16 = 0, 1, 2
+STATIC_SCRATCH_BYTES = 32 << 20  # NVF_STATIC_SCRATCH_BYTES
 
 _p, _i64, _int = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
 
@@ -26,6 +27,7 @@ SIGNATURES = {
     "nvf_nvfp4_scaled_mm": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _int, _p]),
     "nvf_nvfp4_scaled_mm_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "nvf_nvfp4_scaled_mm_ws": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _int, _p, _i64, _p]),
+    "nvf_nvfp4_scaled_mm_static_ws": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _int, _p]),
     "nvf_nvfp4_scaled_mm_blockscale": (_int, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p]),
     "nvf_mxfp8_scaled_mm": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _int, _p]),
     "nvf_grouped_mm": (_int, [_p, _p, _p, _p, _p, _int, _i64, _i64, _i64, _int, _p]),

@@ -206,6 +206,20 @@ int nvf_nvfp4_scaled_mm(const void* a, const void* b, const void* scales_a, cons
 
 int64_t nvf_nvfp4_scaled_mm_workspace_bytes(int64_t m, int64_t n, int64_t k) { return nvfp4_gemm_workspace_bytes(m, n, k); }
 
+int nvf_nvfp4_scaled_mm_static_ws(const void* a, const void* b, const void* scales_a, const void* scales_b, const float* alpha,
+                                  void* out, int64_t m, int64_t n, int64_t k, int out_dtype, void* stream) {
+  const int64_t need = nvfp4_gemm_workspace_bytes(m, n, k);
+  NVF_REQUIRE(need <= kStaticScratchBytes, NVF_ERR_UNSUPPORTED_SHAPE,
+              "M = %lld, N = %lld, K = %lld needs %lld bytes of scratch memory, the library's static scratch holds %lld: use "
+              "nvf_nvfp4_scaled_mm_ws with a workspace of the caller's, or nvf_nvfp4_scaled_mm",
+              (long long)m, (long long)n, (long long)k, (long long)need, (long long)kStaticScratchBytes);
+  void* ws = nullptr;
+  if (need > 0 && m > 0 && n > 0) {
+    if (const int rc = static_scratch(&ws)) return rc;
+  }
+  return nvf_nvfp4_scaled_mm_ws(a, b, scales_a, scales_b, alpha, out, m, n, k, out_dtype, ws, ws ? need : 0, stream);
+}
+
 int nvf_nvfp4_scaled_mm_blockscale(const void* a, const void* b, const void* scales_a, const void* scales_b,
                                    const float* alpha, const float* global_normconst, void* out_fp4, void* out_scales,
                                    float* workspace, int64_t m, int64_t n, int64_t k, void* stream) {

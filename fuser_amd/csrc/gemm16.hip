@@ -19,6 +19,8 @@
 // accumulator registers hold 4 consecutive N-elements of one output row and are stored as 8 bytes.
 #include "nvf_internal.h"
 
+#include <mutex>
+
 namespace nvf {
 namespace {
 
@@ -1841,6 +1843,33 @@ int launch_gemm16(int op, const Gemm16Args& a, hipStream_t stream) {
   }
   return bf16 ? launch_sized<false, true, true>(p, a.m, cus, nullptr, 0, stream)
               : launch_sized<false, false, false>(p, a.m, cus, nullptr, 0, stream);
+}
+
+// -------------------------------------------------------------------------------------------------
+// Scratch memory that needs no allocation: the fp32 partial tiles of the split of K, for callers that cannot
+// allocate (code under HIP graph capture, tight serving loops).  One array per device, held until the process
+// ends; it keeps the contents of the last call, and the split-K kernels need no clearing because every partial
+// tile the reduction reads has been written by the launch before it.  Calls that overlap on one device race.
+// -------------------------------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+// Device address of this device's copy of the array.  The array's name is only a host-side stand-in; the address
+// comes from hipGetSymbolAddress, asked once per device with that device current.
+int static_scratch(void** ptr) {
+  static std::mutex mu;
+  static void* addr[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return fail(NVF_ERR_NO_DEVICE, "hipGetDevice failed");
+  if (dev < 0 || dev >= 64) return fail(NVF_ERR_NO_DEVICE, "device id %d is out of range", dev);
+  std::lock_guard<std::mutex> lock(mu);
+  if (addr[dev] == nullptr) {
+    void* p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr) return fail(NVF_ERR_LAUNCH, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+    addr[dev] = p;
+  }
+  *ptr = addr[dev];
+  return NVF_OK;
 }
 
 int64_t nvfp4_gemm_workspace_bytes(int64_t m, int64_t n, int64_t k) {

@@ -82,6 +82,9 @@ struct Gemm16Args {
 int launch_gemm16(int op, const Gemm16Args& args, hipStream_t stream);
 // scratch bytes with which the dense NVFP4 GEMM of this shape runs faster (0: none needed)
 int64_t nvfp4_gemm_workspace_bytes(int64_t m, int64_t n, int64_t k);
+// the library's own scratch array (one per device, no allocation): its size and its address on the current device
+constexpr int64_t kStaticScratchBytes = (int64_t)32 << 20;
+int static_scratch(void** ptr);
 int launch_mxfp8_gemm(const void* a, const void* b, const void* sfa, const void* sfb, const float* alpha, void* out,
                       int64_t m, int64_t n, int64_t k, int out_dtype, hipStream_t stream);
 

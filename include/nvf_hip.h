@@ -146,6 +146,19 @@ NVF_API int nvf_nvfp4_scaled_mm_ws(const void* a, const void* b, const void* sca
                                    const float* alpha, void* out, int64_t m, int64_t n, int64_t k, int out_dtype,
                                    void* workspace, int64_t workspace_bytes, void* stream);
 
+/* No counterpart in the reference (its entry point allocates its workspace with torch, cutlass/nvfp4_scaled_mm.cu:241-256).
+ * nvf_nvfp4_scaled_mm_ws for callers that cannot allocate -- code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc: the split of K keeps its fp32 partial tiles in a scratch array inside the
+ * library (NVF_STATIC_SCRATCH_BYTES per device, held until the process ends) and the call allocates nothing.
+ * Results are bit-identical to nvf_nvfp4_scaled_mm_ws with a workspace of nvf_nvfp4_scaled_mm_workspace_bytes.
+ * A shape whose split needs more than NVF_STATIC_SCRATCH_BYTES is rejected with NVF_ERR_UNSUPPORTED_SHAPE.
+ * Every call on a device shares that device's array: calls that may overlap in time on one device (different
+ * streams or threads) race on it and must be serialised by the caller. */
+#define NVF_STATIC_SCRATCH_BYTES (32ll << 20)
+NVF_API int nvf_nvfp4_scaled_mm_static_ws(const void* a, const void* b, const void* scales_a, const void* scales_b,
+                                          const float* alpha, void* out, int64_t m, int64_t n, int64_t k,
+                                          int out_dtype, void* stream);
+
 /* cutlass/nvfp4_scaled_mm_blockscale.cu:332-373 nvfp4_scaled_mm_blockscale (decl cutlass/nvf_cutlass.h:147-154).
  *   Operands as nvf_nvfp4_scaled_mm.  The fp32 product alpha * A * B^T is quantized again along n with
  *   the NVFP4 block quantizer (block 16, global scale *global_normconst): out_fp4 [m, n/2], out_scales

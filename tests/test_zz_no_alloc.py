@@ -1,0 +1,81 @@
+"""nvf_nvfp4_scaled_mm_static_ws: the split-K NVFP4 GEMM with the library's own static scratch array instead of a
+caller-provided workspace, for callers that cannot allocate.  Through the raw C ABI its output must be
+bit-identical to nvf_nvfp4_scaled_mm_ws (same kernels, same fixed-order reduction), on two calls in a row that
+share the array -- the second with a smaller input -- and also after the array has been used by another shape."""
+import pytest
+import torch
+
+from helpers import GEMM_MAX_REL, gs_of, max_rel
+from oracle import nvf_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _operand(rows, k, std, gen):
+    x = (torch.randn(rows, k, generator=gen) * std).bfloat16()
+    gs = gs_of(x)
+    q, s = O.block_quantize_nvfp4(x, gs, True)
+    return q, s, gs
+
+
+def test_static_scratch_entry_point_equals_the_workspace_entry_point(dev):
+    from fuser_amd import capi
+
+    lib = capi.lib()
+    # two split-K shapes, the second smaller in every dimension (ragged M / N / K); then the first again
+    for call, (m, n, k) in enumerate([(128, 1024, 8192), (100, 256, 8224), (128, 1024, 8192)]):
+        gen = torch.Generator().manual_seed(100 + call)
+        a, sa, ga = _operand(m, k, 1.0, gen)
+        b, sb, gb = _operand(n, k, 0.02, gen)
+        alpha = 1.0 / (ga * gb)
+        need = lib.nvf_nvfp4_scaled_mm_workspace_bytes(m, n, k)
+        assert 0 < need <= capi.STATIC_SCRATCH_BYTES
+        ad, bd, sad, sbd = a.to(dev), b.to(dev), sa.to(dev), sb.to(dev)
+        al = torch.tensor(alpha, dtype=torch.float32, device=dev)
+        ws = torch.full((need,), 0xFF, dtype=torch.uint8, device=dev)
+        for dt, code in ((torch.bfloat16, capi.BF16), (torch.float16, capi.F16)):
+            want = torch.full((m, n), 7.0, dtype=dt, device=dev)
+            got = torch.full((m, n), 9.0, dtype=dt, device=dev)
+            capi.check(lib.nvf_nvfp4_scaled_mm_ws(ad.data_ptr(), bd.data_ptr(), sad.data_ptr(), sbd.data_ptr(), al.data_ptr(),
+                                                  want.data_ptr(), m, n, k, code, ws.data_ptr(), need, None))
+            capi.check(lib.nvf_nvfp4_scaled_mm_static_ws(ad.data_ptr(), bd.data_ptr(), sad.data_ptr(), sbd.data_ptr(), al.data_ptr(),
+                                                         got.data_ptr(), m, n, k, code, None))
+            torch.cuda.synchronize()
+            assert torch.equal(got, want), (call, m, n, k, dt)
+            assert max_rel(got, O.ref_nvfp4_scaled_mm(a, b, sa, sb, alpha)) <= GEMM_MAX_REL
+    # a shape that needs no scratch runs as nvf_nvfp4_scaled_mm does
+    m, n, k = 16, 512, 1024
+    gen = torch.Generator().manual_seed(7)
+    a, sa, ga = _operand(m, k, 1.0, gen)
+    b, sb, gb = _operand(n, k, 0.02, gen)
+    al = torch.tensor(1.0 / (ga * gb), dtype=torch.float32, device=dev)
+    ad, bd, sad, sbd = a.to(dev), b.to(dev), sa.to(dev), sb.to(dev)
+    want = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
+    got = torch.empty_like(want)
+    assert lib.nvf_nvfp4_scaled_mm_workspace_bytes(m, n, k) == 0
+    capi.check(lib.nvf_nvfp4_scaled_mm(ad.data_ptr(), bd.data_ptr(), sad.data_ptr(), sbd.data_ptr(), al.data_ptr(), want.data_ptr(), m, n, k,
+                                       capi.BF16, None))
+    capi.check(lib.nvf_nvfp4_scaled_mm_static_ws(ad.data_ptr(), bd.data_ptr(), sad.data_ptr(), sbd.data_ptr(), al.data_ptr(), got.data_ptr(),
+                                                 m, n, k, capi.BF16, None))
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    # The largest scratch any split asks for on 256 compute units is exactly the static array (at most 2 x 256 work
+    # items of 128 x 128 fp32): such a shape is accepted and runs; the size check itself is exercised on the CPU
+    # side of the C ABI only where a device reports more compute units.
+    m, n, k = 256, 8192, 16384
+    assert lib.nvf_nvfp4_scaled_mm_workspace_bytes(m, n, k) == capi.STATIC_SCRATCH_BYTES
+    g = torch.Generator(device=dev).manual_seed(3)
+    ad = torch.randint(0, 256, (m, k // 2), dtype=torch.uint8, device=dev, generator=g)
+    bd = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device=dev, generator=g)
+    sad = torch.randint(0x20, 0x40, (m, k // 16), dtype=torch.uint8, device=dev, generator=g)
+    sbd = torch.randint(0x20, 0x40, (n, k // 16), dtype=torch.uint8, device=dev, generator=g)
+    al = torch.tensor(2.0 ** -6, dtype=torch.float32, device=dev)
+    ws = torch.full((capi.STATIC_SCRATCH_BYTES,), 0xFF, dtype=torch.uint8, device=dev)
+    want = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
+    got = torch.empty_like(want)
+    capi.check(lib.nvf_nvfp4_scaled_mm_ws(ad.data_ptr(), bd.data_ptr(), sad.data_ptr(), sbd.data_ptr(), al.data_ptr(), want.data_ptr(), m, n, k,
+                                          capi.BF16, ws.data_ptr(), capi.STATIC_SCRATCH_BYTES, None))
+    capi.check(lib.nvf_nvfp4_scaled_mm_static_ws(ad.data_ptr(), bd.data_ptr(), sad.data_ptr(), sbd.data_ptr(), al.data_ptr(), got.data_ptr(),
+                                                 m, n, k, capi.BF16, None))
+    torch.cuda.synchronize()
+    assert torch.isfinite(got.float()).all() and torch.equal(got, want)
