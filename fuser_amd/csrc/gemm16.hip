@@ -1373,7 +1373,7 @@ __global__ __launch_bounds__(256, 1) void grouped16_gemm_256_kernel(const Params
   const int li = lane & 31, lg = lane >> 5;
   const int tiles_n = p.n / BN;
 
-  // ---- work list: prefix sums of tiles per group (one wavefront, 64 groups per round)
+  // ---- work list: prefix sums of 256-row tiles per group (one wavefront, 64 groups per round)
   if (wave == 0) {
     int running = 0;
     for (int base = 0; base < p.groups; base += 64) {
@@ -1381,7 +1381,7 @@ __global__ __launch_bounds__(256, 1) void grouped16_gemm_256_kernel(const Params
       int cnt = 0;
       if (g < p.groups) {
         const int mg = p.problem_sizes[g * 3];
-        cnt = mg > 0 ? ((mg + BM - 1) / BM) * tiles_n : 0;
+        cnt = mg > 0 ? (mg + BM - 1) / BM : 0;
       }
       int incl = cnt;
 #pragma unroll
@@ -1395,11 +1395,19 @@ __global__ __launch_bounds__(256, 1) void grouped16_gemm_256_kernel(const Params
     if (lane == 0) tile_prefix[0] = 0;
   }
   __syncthreads();
-  const int total = __builtin_amdgcn_readfirstlane(tile_prefix[p.groups]);
-  const int chunk_tiles = (total + 7) >> 3;
+  // Workgroup ids are dealt round-robin to the 8 XCDs.  The tiles of a group are walked in bands of 4 m-tiles, n-major
+  // inside a band, so that 32 consecutive tiles share 4 A and 8 B panels in an XCD's L2.  DEAL (n-tiles a multiple of
+  // 8): XCD x takes the n-tiles x, x+8, ... of every band, i.e. its own list of (tiles / 8) tiles of the same make-up as
+  // every other XCD's: each expert's weights stream in through all eight XCDs and all of them meet the cheap and
+  // the expensive tiles (small groups are bound by streaming their weights once) at the same rate.  Otherwise XCD
+  // x owns the contiguous eighth [x*chunk, (x+1)*chunk) of the one list.
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, slots = gridDim.x >> 3;
-  const int range_end = min((xcd + 1) * chunk_tiles, total);
-  const int first_tile = xcd * chunk_tiles + slot;
+  const bool deal = (tiles_n & 7) == 0;
+  const int per_m = deal ? tiles_n >> 3 : tiles_n;  // list entries per m-tile
+  const int total = __builtin_amdgcn_readfirstlane(tile_prefix[p.groups]) * per_m;
+  const int chunk_tiles = (total + 7) >> 3;
+  const int range_end = deal ? total : min((xcd + 1) * chunk_tiles, total);
+  const int first_tile = deal ? slot : xcd * chunk_tiles + slot;
   if (first_tile >= range_end) return;
 
   const int kb = p.k * 2;   // bytes per operand row
@@ -1410,18 +1418,18 @@ __global__ __launch_bounds__(256, 1) void grouped16_gemm_256_kernel(const Params
     int lo = 0, hi = p.groups;
     while (hi - lo > 1) {
       const int mid = (lo + hi) >> 1;
-      if (t < tile_prefix[mid]) hi = mid; else lo = mid;
+      if (t < tile_prefix[mid] * per_m) hi = mid; else lo = mid;
     }
     const int g = __builtin_amdgcn_readfirstlane(lo);
     // (loaded through the vector path, which is coherent with this kernel's own stores; made scalar here)
     const int m_g = __builtin_amdgcn_readfirstlane(p.problem_sizes[g * 3]);
     const int64_t row_off = __builtin_amdgcn_readfirstlane(p.expert_offsets[g]);
     const int tiles_m = (m_g + BM - 1) / BM;
-    const int local = __builtin_amdgcn_readfirstlane(t - tile_prefix[g]);
-    // bands of 4 m-tiles, n-major inside a band: 32 consecutive tiles share 4 A and 8 B panels
-    const int band = local / (4 * tiles_n), in_band = local - band * 4 * tiles_n;
+    const int local = __builtin_amdgcn_readfirstlane(t - tile_prefix[g] * per_m);
+    const int band = local / (4 * per_m), in_band = local - band * 4 * per_m;
     const int band_h = min(4, tiles_m - 4 * band);
-    const int nt = in_band / band_h, mt = 4 * band + (in_band - nt * band_h);
+    const int ntl = in_band / band_h, mt = 4 * band + (in_band - ntl * band_h);
+    const int nt = deal ? xcd + 8 * ntl : ntl;
     Tile r;
     r.a = p.a + (row_off + (int64_t)mt * BM) * kb;
     r.b = p.b + ((int64_t)g * p.n + (int64_t)nt * BN) * kb;
