@@ -227,14 +227,16 @@ int nvf_nvfp4_scaled_mm_blockscale(const void* a, const void* b, const void* sca
   NVF_REQUIRE(k % 32 == 0, NVF_ERR_UNSUPPORTED_SHAPE, "The K dimension %lld is not divisible by 32", (long long)k);
   NVF_REQUIRE(n % 32 == 0, NVF_ERR_UNSUPPORTED_SHAPE, "The N dimension %lld is not divisible by 32", (long long)n);
   if (m == 0 || n == 0) return NVF_OK;
-  NVF_REQUIRE(a && b && scales_a && scales_b && alpha && global_normconst && out_fp4 && out_scales && workspace,
-              NVF_ERR_INVALID_ARGUMENT, "NULL buffer");
+  NVF_REQUIRE(a && b && scales_a && scales_b && alpha && global_normconst && out_fp4 && out_scales, NVF_ERR_INVALID_ARGUMENT, "NULL buffer");
   NVF_REQUIRE_ALIGNED16(a, b, scales_a, scales_b, out_fp4, out_scales, workspace);
-  Gemm16Args g{a, b, scales_a, scales_b, alpha, workspace, nullptr, nullptr, nullptr, 1, m, n, k, NVF_F32};
+  Gemm16Args g{a, b, scales_a, scales_b, alpha, out_fp4, nullptr, nullptr, nullptr, 1, m, n, k, kDtypeFp4BlockScaled};
+  g.out_sf = out_scales;
+  g.gnorm = global_normconst;
   const int rc = launch_gemm16(0, g, static_cast<hipStream_t>(stream));
-  if (rc != NVF_OK) return rc;
-  return launch_nvfp4_quantize(workspace, NVF_F32, m, n, global_normconst, /*layout: 128x4*/ 1, nullptr, nullptr, 1, out_fp4,
-                               out_scales, static_cast<hipStream_t>(stream));
+  if (rc != NVF_OK || workspace == nullptr) return rc;
+  // the optional dump of the fp32 product: the same kernel once more, with the accumulators written out as they are
+  Gemm16Args d{a, b, scales_a, scales_b, alpha, workspace, nullptr, nullptr, nullptr, 1, m, n, k, NVF_F32};
+  return launch_gemm16(0, d, static_cast<hipStream_t>(stream));
 }
 
 int nvf_mxfp8_scaled_mm(const void* a, const void* b, const void* scales_a, const void* scales_b, const float* alpha,

@@ -59,6 +59,10 @@ struct Params {
   // grouped skinny kernel: the group sizes it serves; the tile kernel skips groups of fewer than min_rows rows
   int rows_lo = 0, rows_hi = 0, min_rows = 0;
   int tail_done = 0;  // grouped NVFP4 dispatch: the ends of the large groups have been computed by an earlier launch
+  // block-scaled result (nvfp4_scaled_mm_blockscale): out = packed e2m1 [m, n/2], out_sf = e4m3 scales in the 128x4
+  // layout of [roundUp(m,128), roundUp(n/16,4)], gnorm = the result's global (encode) scale on the device
+  uint8_t* out_sf = nullptr;
+  const float* gnorm = nullptr;
 };
 
 __device__ __forceinline__ uint32_t pack2(float a, float b, bool out_bf16) {
@@ -76,6 +80,50 @@ __device__ __forceinline__ uint32_t pack2(float a, float b, bool out_bf16) {
 // consecutive lanes = 16 consecutive rows, one chunk) are conflict-free.
 __device__ __forceinline__ int lds_pos2(int row, int chunk) { return row * 8 + (chunk ^ ((row >> 1) & 7)); }
 __device__ __forceinline__ int lds_pos(int row, int chunk) { return lds_pos2(row, chunk); }
+
+// Block-scaled epilogue (cutlass/nvfp4_scaled_mm_blockscale.cu:87-93: the product is quantized to NVFP4 again along
+// N before it leaves the kernel).  One 32x32 accumulator tile: lane (li, lg) holds row li, columns 8q + 4lg + e in
+// register 4q + e, so each of the row's two 16-column blocks is shared by the lanes (li, 0) and (li, 1): amax over
+// the lane's 8 values, one exchange with lane ^ 32, then the block quantizer's arithmetic
+// (runtime/block_quantization_kernels.cu:224-263) on alpha * acc.  For block b both lanes get the scale code q8[b];
+// h[b] holds this lane's 4 of the block's 8 payload bytes: bits 0..15 = bytes 2lg, 2lg+1, bits 16..31 = bytes
+// 4+2lg, 5+2lg.  Must be called by whole wavefronts.
+__device__ __forceinline__ void quantize_acc_tile(const f32x16& acc, float alpha, float gs, float decode, bool active, uint32_t h[2],
+                                                  uint32_t q8[2]) {
+#pragma unroll
+  for (int b = 0; b < 2; ++b) {
+    float x[8];
+    float m = -INFINITY;
+    bool nonfinite = false;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      x[e] = acc[8 * b + e] * alpha;
+      m = fmaxf(m, fabsf(x[e]));  // NaN ignored, as the quantizer does
+      nonfinite |= !(fabsf(x[e]) < INFINITY);
+    }
+    const int lane = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    m = fmaxf(m, __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ 32) << 2, __builtin_bit_cast(int, m))));
+    float r;
+    q8[b] = nvfp4_block_scale(m, true, gs, decode, active, r);
+    uint32_t w = 0;
+    if (__builtin_amdgcn_ballot_w64(nonfinite) == 0) {
+      w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, x[0] * r, x[1] * r, 1.0f, 0);
+      w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, x[2] * r, x[3] * r, 1.0f, 1);
+      w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, x[4] * r, x[5] * r, 1.0f, 2);
+      w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, x[6] * r, x[7] * r, 1.0f, 3);
+    } else {  // explicit NaN rule of the narrow cast
+#pragma unroll
+      for (int t = 0; t < 4; ++t) w |= f32x2_to_e2m1_byte(x[2 * t] * r, x[2 * t + 1] * r) << (8 * t);
+    }
+    h[b] = w;
+  }
+}
+
+// fills n bytes with zero (the padding of the block-scaled result's scale buffer for ragged shapes)
+__global__ __launch_bounds__(256) void zero_fill_kernel(uint32_t* __restrict__ dst, int64_t words) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < words) dst[i] = 0u;
+}
 
 template <int BM, int BN, bool BF16_MMA, bool OUT_BF16>
 __global__ __launch_bounds__(256) void gemm16_kernel(const Params p) {
@@ -284,7 +332,7 @@ __device__ __forceinline__ int rows_in_256_tiles(int m_g) {
 //     odd step converts its even half: a full step of MFMAs hides the latency.
 // Requires K % 32 == 0 (a piece never straddles the end of a row).
 // -------------------------------------------------------------------------------------------------
-template <int BM, int BN, bool OUT_BF16, bool OUT_F32, bool SPLIT_K = false>
+template <int BM, int BN, bool OUT_BF16, bool OUT_F32, bool SPLIT_K = false, bool OUT_FP4 = false>
 __global__ __launch_bounds__(256) void nvfp4_tile_kernel(const Params p) {
   constexpr int WTM = BM / 2, WTN = BN / 2;  // wave tile
   constexpr int TM = WTM / 32, TN = WTN / 32;
@@ -477,6 +525,35 @@ __global__ __launch_bounds__(256) void nvfp4_tile_kernel(const Params p) {
 
     // ---- epilogue: acc[i][j][r] = C[m = lane%32][n = (r/4)*8 + (lane/32)*4 + r%4] of its 32x32 tile ----
     const float alpha = SPLIT_K ? 1.0f : (dense ? p.alpha[0] : p.alpha[g]);  // split: applied by the reduction
+    if constexpr (OUT_FP4) {
+      // block-scaled result: every 32x32 accumulator tile becomes 32 rows x 16 payload bytes and 32 x 2 scale bytes
+      // (N % 32 == 0: a tile's columns exist or not as a whole)
+      const float gs = p.gnorm[0], decode = 1.0f / gs;
+      const int sf_out_padded = ((p.n >> 4) + 3) & ~3;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const int mrow = m0 + wm * WTM + i * 32 + (lane & 31);
+        const bool row_ok = mrow < m_g;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          const int ncol = n0 + wn * WTN + j * 32;
+          if (ncol >= p.n) continue;  // wave-uniform
+          uint32_t h[2], q8[2];
+          quantize_acc_tile(acc[i][j], alpha, gs, decode, row_ok, h, q8);
+          if (row_ok) {
+            uint8_t* orow = static_cast<uint8_t*>(p.out) + (int64_t)mrow * (p.n >> 1) + (ncol >> 1) + 2 * (lane >> 5);
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+              *reinterpret_cast<uint16_t*>(orow + b * 8) = (uint16_t)(h[b] & 0xffffu);
+              *reinterpret_cast<uint16_t*>(orow + b * 8 + 4) = (uint16_t)(h[b] >> 16);
+            }
+            if ((lane >> 5) == 0)
+              *reinterpret_cast<uint16_t*>(p.out_sf + swizzle_128x4(mrow, ncol >> 4, sf_out_padded)) = (uint16_t)(q8[0] | (q8[1] << 8));
+          }
+        }
+      }
+      continue;
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
       const int mrow = m0 + wm * WTM + i * 32 + (lane & 31);
@@ -551,7 +628,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
 // TM = 32-row accumulator tiles of a wavefront along M: 4 -> 256x256 workgroup tile, 2 -> 128x256 (dense shapes
 // whose 256x256 tiles would leave compute units idle; 1.5 times the conversion work per MFMA).  The statement
 // order for TM = 4 is the one the 8192^3 measurements were made with.
-template <bool OUT_BF16, bool GROUPED, int TM = 4, bool OUT_F32 = false, bool PAIRS = false>
+template <bool OUT_BF16, bool GROUPED, int TM = 4, bool OUT_F32 = false, bool PAIRS = false, bool OUT_FP4 = false>
 __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   static_assert(TM == 4 || TM == 2, "tile height");
   constexpr int BM = 64 * TM, BN = 256;
@@ -899,7 +976,47 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
     // acc[i][j][r] = C[m = li][n = (r/4)*8 + lg*4 + r%4] of its 32x32 sub-tile.
     const Where cw = tile_where(c_tile);
     const float alpha = p.alpha[cw.g];
-    if constexpr (OUT_F32) {
+    if constexpr (OUT_FP4) {
+      // Block-scaled result.  A wavefront's 32 x 64 block i is quantized tile by tile (quantize_acc_tile), its 32 rows
+      // x 32 payload bytes are collected in a private piece of LDS (pitch 48 bytes) and leave as 16 bytes per lane,
+      // two lanes to a row; the four scale codes of a row (its four 16-column blocks are one dword of the 128x4
+      // layout) are kept per i and stored once at the end: 16 bytes per row for the 128 rows of a 256-row tile's
+      // wavefront (they are one whole 128x4 scale tile), 8 bytes for the 64 rows of a 128-row tile's.
+      const float gs = p.gnorm[0], decode = 1.0f / gs;
+      int elane = lane;
+      asm volatile("" : "+v"(elane));
+      uint8_t* stage = reinterpret_cast<uint8_t*>(lds + 2 * BUF_UNITS) + wave * 2560;
+      uint8_t* wr = stage + (elane & 31) * 48 + (elane >> 5) * 2;
+      const uint8_t* rd = stage + (elane >> 1) * 48 + (elane & 1) * 16;
+      const int64_t opitch = p.n >> 1;
+      uint8_t* obase = static_cast<uint8_t*>(p.out) + (cw.m0 + wm * (32 * TM) + (elane >> 1)) * opitch + ((cw.n0 + wn * 64) >> 1) + (elane & 1) * 16;
+      uint32_t sfw[TM];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        sfw[i] = 0;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          uint32_t h[2], q8[2];
+          quantize_acc_tile(acc[i][j], alpha, gs, decode, true, h, q8);
+#pragma unroll
+          for (int b = 0; b < 2; ++b) {
+            *reinterpret_cast<uint16_t*>(wr + j * 16 + b * 8) = (uint16_t)(h[b] & 0xffffu);
+            *reinterpret_cast<uint16_t*>(wr + j * 16 + b * 8 + 4) = (uint16_t)(h[b] >> 16);
+          }
+          sfw[i] |= (q8[0] | (q8[1] << 8)) << (16 * j);
+        }
+        asm volatile("" ::: "memory");  // the read below sees the writes above: one wavefront's LDS accesses stay in order
+        const u32x4 v = *reinterpret_cast<const u32x4*>(rd);
+        *reinterpret_cast<u32x4*>(obase + (int64_t)(i * 32) * opitch) = v;
+        asm volatile("" ::: "memory");
+      }
+      if (lg == 0) {
+        const int sf_cols4 = p.n >> 6;  // 512-byte scale tiles per 128 rows (N % 256 == 0: no padding columns)
+        uint8_t* sfp = p.out_sf + ((cw.m0 >> 7) * (int64_t)sf_cols4 + ((cw.n0 + wn * 64) >> 6)) * 512 + li * 16;
+        if constexpr (TM == 4) *reinterpret_cast<u32x4*>(sfp + (int64_t)wm * sf_cols4 * 512) = u32x4{sfw[0], sfw[1], sfw[2], sfw[3]};
+        else *reinterpret_cast<u32x2*>(sfp + wm * 8) = u32x2{sfw[0], sfw[1]};
+      }
+    } else if constexpr (OUT_F32) {
       // as below, with 32x16 blocks of fp32 (64-byte row segments)
       int elane = lane;
       asm volatile("" : "+v"(elane));
@@ -972,16 +1089,16 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
 #undef NVF_PIN_ACC
 }
 
-template <bool OUT_BF16, bool GROUPED, int TM, bool OUT_F32, bool PAIRS>
+template <bool OUT_BF16, bool GROUPED, int TM, bool OUT_F32, bool PAIRS, bool OUT_FP4 = false>
 int launch_nvfp4_fast_cfg(const Params& p, int cus, hipStream_t stream) {
-  auto kern = nvfp4_gemm_256_kernel<OUT_BF16, GROUPED, TM, OUT_F32, PAIRS>;
+  auto kern = nvfp4_gemm_256_kernel<OUT_BF16, GROUPED, TM, OUT_F32, PAIRS, OUT_FP4>;
   constexpr int lds_bytes = 2 * (64 * TM + 256) * 128 + 8 * 2560;  // 128 KiB / 96 KiB of tiles + the epilogue's 20 KiB
   // grouped: an upper bound (128-row tiles: one per weight panel and group of at least rows_lo rows)
   const int64_t tiles_m = (GROUPED && TM == 2) ? std::min<int64_t>(p.groups, p.m / std::max(p.rows_lo, 1)) : p.m / (64 * TM);
   const int64_t tiles = tiles_m * (p.n / 256);
   const unsigned grid = (unsigned)(tiles >= cus ? (cus & ~7) : ((tiles + 7) / 8) * 8);
-  if (note_launch("nvfp4_gemm_256_kernel<grouped=%d,TM=%d,f32=%d,pairs=%d> grid=%u rows=%d..%d min_rows=%d", (int)GROUPED, TM, (int)OUT_F32,
-                  (int)PAIRS, grid, p.rows_lo, p.rows_hi, p.min_rows))
+  if (note_launch("nvfp4_gemm_256_kernel<grouped=%d,TM=%d,f32=%d,pairs=%d%s> grid=%u rows=%d..%d min_rows=%d", (int)GROUPED, TM, (int)OUT_F32,
+                  (int)PAIRS, OUT_FP4 ? ",fp4_blockscale" : "", grid, p.rows_lo, p.rows_hi, p.min_rows))
     return NVF_OK;
   static std::atomic<uint64_t> configured{0};  // one bit per device
   if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
@@ -989,11 +1106,11 @@ int launch_nvfp4_fast_cfg(const Params& p, int cus, hipStream_t stream) {
   return check_launch("nvfp4_gemm_256_kernel");
 }
 
-template <bool OUT_BF16, bool GROUPED, int TM = 4, bool OUT_F32 = false>
+template <bool OUT_BF16, bool GROUPED, int TM = 4, bool OUT_F32 = false, bool OUT_FP4 = false>
 int launch_nvfp4_fast(const Params& p, int cus, hipStream_t stream) {
   // an even number of 128-deep spans per tile: the variant whose two in-flight spans swap names instead of being copied
-  if (((p.k >> 7) & 1) == 0) return launch_nvfp4_fast_cfg<OUT_BF16, GROUPED, TM, OUT_F32, true>(p, cus, stream);
-  return launch_nvfp4_fast_cfg<OUT_BF16, GROUPED, TM, OUT_F32, false>(p, cus, stream);
+  if (((p.k >> 7) & 1) == 0) return launch_nvfp4_fast_cfg<OUT_BF16, GROUPED, TM, OUT_F32, true, OUT_FP4>(p, cus, stream);
+  return launch_nvfp4_fast_cfg<OUT_BF16, GROUPED, TM, OUT_F32, false, OUT_FP4>(p, cus, stream);
 }
 
 // -------------------------------------------------------------------------------------------------
@@ -1652,11 +1769,12 @@ int launch_cfg(const Params& p, int grid, hipStream_t stream) {
   return check_launch("gemm16_kernel");
 }
 
-template <int BM, int BN, bool OUT_BF16, bool OUT_F32 = false>
+template <int BM, int BN, bool OUT_BF16, bool OUT_F32 = false, bool OUT_FP4 = false>
 int launch_nvfp4_tile(const Params& p, int grid, hipStream_t stream) {
-  auto kern = nvfp4_tile_kernel<BM, BN, OUT_BF16, OUT_F32>;
+  auto kern = nvfp4_tile_kernel<BM, BN, OUT_BF16, OUT_F32, false, OUT_FP4>;
   constexpr int lds_bytes = 2 * (BM + BN) * 128;
-  if (note_launch("nvfp4_tile_kernel<%d,%d,f32=%d> grid=%d skip_whole_256=%d min_rows=%d", BM, BN, (int)OUT_F32, grid, p.skip_whole_256, p.min_rows))
+  if (note_launch("nvfp4_tile_kernel<%d,%d,f32=%d%s> grid=%d skip_whole_256=%d min_rows=%d", BM, BN, (int)OUT_F32, OUT_FP4 ? ",fp4_blockscale" : "", grid,
+                  p.skip_whole_256, p.min_rows))
     return NVF_OK;
   static std::atomic<uint64_t> configured{0};  // one bit per device
   if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
@@ -1805,20 +1923,36 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int6
   return launch_tile<64, 64, NVFP4, BF16_MMA, OUT_BF16>(p, (int)(upper < cap ? upper : cap), stream);
 }
 
-// dense NVFP4 with an fp32 result (the product that the block-scaled epilogue op re-quantizes)
-int launch_nvfp4_f32(const Params& p, int cus, hipStream_t stream) {
+// Dense NVFP4 whose result leaves the kernel re-quantized to NVFP4 (FP4: nvfp4_scaled_mm_blockscale) or as the fp32
+// product itself (that op's optional dump of what it quantized).  Both take the same kernel for a shape, so that
+// the dump holds exactly the accumulators the quantized result was made from.
+template <bool FP4>
+int launch_nvfp4_wide(const Params& p, int cus, hipStream_t stream) {
   auto tiles = [&](int bm, int bn) { return ceil_div(p.m, bm) * ceil_div(p.n, bn); };
-  if ((p.m & 255) == 0 && (p.n & 255) == 0 && (p.k & 127) == 0 && p.k >= 256) {
-    const int64_t t = tiles(256, 256);  // as for the 16-bit results: only if the tiles fill the compute units
-    if (100 * ceil_div(t, cus) <= 144 * t / cus) return launch_nvfp4_fast<false, false, 4, true>(p, cus, stream);
+  if (FP4 && ((p.m & 127) != 0 || ((p.n >> 4) & 3) != 0)) {
+    // ragged: the padding rows / columns of the scale buffer's last 128x4 tiles are written as zero first
+    const int64_t words = round_up(p.m, 128) * round_up(p.n >> 4, 4) / 4;
+    if (!note_launch("zero_fill_kernel grid=%lld", (long long)ceil_div(words, 256))) {
+      hipLaunchKernelGGL(zero_fill_kernel, dim3((unsigned)ceil_div(words, 256)), dim3(256), 0, stream, reinterpret_cast<uint32_t*>(p.out_sf), words);
+      if (const int rc = check_launch("zero_fill_kernel")) return rc;
+    }
   }
-  if (tiles(256, 256) >= cus) return launch_nvfp4_tile<256, 256, false, true>(p, cus, stream);
+  if ((p.n & 255) == 0 && (p.k & 127) == 0 && p.k >= 256) {
+    // as for the 16-bit results: persistent 256x256 or 128x256 tiles where they fill the compute units
+    const int64_t t256 = (p.m & 255) == 0 ? tiles(256, 256) : 0, t128 = (p.m & 127) == 0 ? tiles(128, 256) : 0;
+    const int64_t cost256 = t256 ? 100 * ceil_div(t256, cus) : INT64_MAX;
+    const int64_t cost128 = t128 ? 58 * ceil_div(t128, cus) : INT64_MAX;
+    const int64_t cost_tile = 144 * tiles(128, 256) / (2 * cus);
+    if (t256 && cost256 <= cost128 && cost256 <= cost_tile) return launch_nvfp4_fast<false, false, 4, !FP4, FP4>(p, cus, stream);
+    if (t128 && cost128 <= cost_tile) return launch_nvfp4_fast<false, false, 2, !FP4, FP4>(p, cus, stream);
+  }
+  if (tiles(256, 256) >= cus) return launch_nvfp4_tile<256, 256, false, !FP4, FP4>(p, cus, stream);
   if (tiles(128, 128) >= cus) {
     const int64_t t = tiles(128, 128);
-    return launch_nvfp4_tile<128, 128, false, true>(p, (int)(t < 2 * cus ? t : 2 * cus), stream);
+    return launch_nvfp4_tile<128, 128, false, !FP4, FP4>(p, (int)(t < 2 * cus ? t : 2 * cus), stream);
   }
   const int64_t t = tiles(64, 64);
-  return launch_nvfp4_tile<64, 64, false, true>(p, (int)(t < 4 * cus ? t : 4 * cus), stream);
+  return launch_nvfp4_tile<64, 64, false, !FP4, FP4>(p, (int)(t < 4 * cus ? t : 4 * cus), stream);
 }
 
 }  // namespace
@@ -1844,7 +1978,12 @@ int launch_gemm16(int op, const Gemm16Args& a, hipStream_t stream) {
   p.k = (int)a.k;
   const int cus = cu_count();
   const bool bf16 = a.dtype == NVF_BF16;
-  if (op == 0 && a.dtype == NVF_F32) return launch_nvfp4_f32(p, cus, stream);
+  if (op == 0 && a.dtype == NVF_F32) return launch_nvfp4_wide<false>(p, cus, stream);
+  if (op == 0 && a.dtype == kDtypeFp4BlockScaled) {
+    p.out_sf = static_cast<uint8_t*>(a.out_sf);
+    p.gnorm = a.gnorm;
+    return launch_nvfp4_wide<true>(p, cus, stream);
+  }
   if (op == 0 || op == 1) {
     return bf16 ? launch_sized<true, false, true>(p, a.m, cus, a.workspace, a.workspace_bytes, stream)
                 : launch_sized<true, false, false>(p, a.m, cus, a.workspace, a.workspace_bytes, stream);

@@ -169,12 +169,10 @@ std::pair<torch::Tensor, torch::Tensor> nvfp4_scaled_mm_blockscale(const torch::
   // The 128x4 layout needs whole 128-row tiles; for m % 128 == 0 this is the reference's [m, roundUp(n/16, 4)].
   torch::Tensor output_blockscale =
       at::empty({roundUp(m, 128), roundUp(n / 16, 4)}, at::TensorOptions().dtype(at::ScalarType::Float8_e4m3fn).device(a.device()));
-  torch::Tensor product = at::empty({m, n}, at::TensorOptions().dtype(at::ScalarType::Float).device(a.device()));
   check_status(nvf_nvfp4_scaled_mm_blockscale(a.data_ptr(), b.data_ptr(), scales_a.data_ptr(), scales_b.data_ptr(),
                                               static_cast<const float*>(alpha.data_ptr()),
                                               static_cast<const float*>(global_normconst.data_ptr()), output.data_ptr(),
-                                              output_blockscale.data_ptr(), static_cast<float*>(product.data_ptr()), m, n, k,
-                                              stream),
+                                              output_blockscale.data_ptr(), /*product dump*/ nullptr, m, n, k, stream),
                "nvfp4_scaled_mm_blockscale");
   return {output, output_blockscale};
 }

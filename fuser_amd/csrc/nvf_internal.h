@@ -78,7 +78,12 @@ struct Gemm16Args {
   int dtype;  // out dtype (NVFP4 ops) or in/out dtype (grouped_mm)
   void* workspace = nullptr;  // dense NVFP4: optional scratch for a split of K (nvfp4_gemm_workspace_bytes)
   int64_t workspace_bytes = 0;
+  // dtype == kDtypeFp4BlockScaled (dense NVFP4 only): out = packed e2m1 [m, n/2], out_sf = its e4m3 scales (128x4
+  // layout), gnorm = the result's global scale on the device
+  void* out_sf = nullptr;
+  const float* gnorm = nullptr;
 };
+constexpr int kDtypeFp4BlockScaled = 100;  // internal result type code of launch_gemm16, next to nvf_dtype
 int launch_gemm16(int op, const Gemm16Args& args, hipStream_t stream);
 // scratch bytes with which the dense NVFP4 GEMM of this shape runs faster (0: none needed)
 int64_t nvfp4_gemm_workspace_bytes(int64_t m, int64_t n, int64_t k);
@@ -135,6 +140,48 @@ __device__ __forceinline__ uint32_t f32_to_e8m0_rp(float x) {
   if (e == 0) return m > 0x400000u ? 1u : 0u;  // denormal: 2^-127 is e8m0 code 0
   uint32_t r = e + (m != 0);
   return r > 254u ? 254u : r;
+}
+
+// true when the 3-instruction divisions below give the result of the true division for this operand: biased
+// exponent in [2, 250], or +0 (amax / 6 = 0 exactly; 1 / 0: v_rcp gives +Inf, the correction step NaN, and
+// fminf(NaN, FLT_MAX) = FLT_MAX = fminf(+Inf, FLT_MAX))
+__device__ __forceinline__ bool fast_div_ok(float v) {
+  const uint32_t b = f32_to_bits(v);
+  return ((b >> 23) & 0xffu) - 2u <= 248u || b == 0u;
+}
+__device__ __forceinline__ float fast_div6(float m) {
+  const float r6 = 0x1.555556p-3f;  // RN(1/6)
+  const float q0 = m * r6;
+  return __builtin_fmaf(__builtin_fmaf(-6.0f, q0, m), r6, q0);
+}
+__device__ __forceinline__ float fast_rcp(float v) {
+  const float r0 = __builtin_amdgcn_rcpf(v);
+  return __builtin_fmaf(__builtin_fmaf(-v, r0, 1.0f), r0, r0);
+}
+
+// NVFP4 block scale from the block's amax m (>= 0 or -inf), in the operation order of
+// runtime/block_quantization_kernels.cu:224-239.  Returns the e4m3 code that is stored and sets r, the factor the
+// block's values are multiplied with ahead of the e2m1 cast.  gs: encode scale (use_gs), decode = 1.0f / gs.
+// Must be called by all lanes of the wavefront: if any `active` lane holds an operand outside the range of the
+// 3-instruction divisions, the wavefront redoes the arithmetic with true divisions.
+__device__ __forceinline__ uint32_t nvfp4_block_scale(float m, bool use_gs, float gs, float decode, bool active, float& r) {
+  float s = fast_div6(m);                 // :224  amax / 6
+  if (use_gs) s = s * gs;                 // :226
+  s = fminf(s, 3.402823466e+38f);         // :228
+  uint32_t q8 = f32_to_e4m3_satfinite(s); // :230
+  float sf = e4m3_to_f32(q8);             // :233
+  float den = use_gs ? sf * decode : sf;  // :237 / :239
+  r = fminf(fast_rcp(den), 3.402823466e+38f);
+  if (__builtin_amdgcn_ballot_w64(active && (!fast_div_ok(m) || !fast_div_ok(den))) != 0) {
+    s = m / 6.0f;
+    if (use_gs) s = s * gs;
+    s = fminf(s, 3.402823466e+38f);
+    q8 = f32_to_e4m3_satfinite(s);
+    sf = e4m3_to_f32(q8);
+    den = use_gs ? sf * decode : sf;
+    r = fminf(1.0f / den, 3.402823466e+38f);
+  }
+  return q8;
 }
 
 }  // namespace nvf

@@ -116,23 +116,6 @@ __device__ __forceinline__ void decode16(const Raw16<float>& r, bool active, flo
   }
 }
 
-// true when the 3-instruction divisions below give the result of the true division for this operand: biased
-// exponent in [2, 250], or +0 (amax / 6 = 0 exactly; 1 / 0: v_rcp gives +Inf, the correction step NaN, and
-// fminf(NaN, FLT_MAX) = FLT_MAX = fminf(+Inf, FLT_MAX))
-__device__ __forceinline__ bool fast_div_ok(float v) {
-  const uint32_t b = f32_to_bits(v);
-  return ((b >> 23) & 0xffu) - 2u <= 248u || b == 0u;
-}
-__device__ __forceinline__ float fast_div6(float m) {
-  const float r6 = 0x1.555556p-3f;  // RN(1/6)
-  const float q0 = m * r6;
-  return __builtin_fmaf(__builtin_fmaf(-6.0f, q0, m), r6, q0);
-}
-__device__ __forceinline__ float fast_rcp(float v) {
-  const float r0 = __builtin_amdgcn_rcpf(v);
-  return __builtin_fmaf(__builtin_fmaf(-v, r0, 1.0f), r0, r0);
-}
-
 constexpr int kSegCols = 1024;  // elements per wavefront row segment
 
 // value -> nearest value of the 16-bit type T (round to nearest even), as fp32
@@ -215,22 +198,8 @@ __global__ __launch_bounds__(256) void nvfp4_quantize_kernel(const T* __restrict
   float m = -INFINITY;
 #pragma unroll
   for (int j = 0; j < 16; ++j) m = fmaxf(m, fabsf(x[j]));
-  float s = fast_div6(m);                 // :224  amax / 6
-  if (use_gs) s = s * gs;                 // :226
-  s = fminf(s, FLT_MAX);                  // :228
-  uint32_t q8 = f32_to_e4m3_satfinite(s); // :230
-  float sf = e4m3_to_f32(q8);             // :233
-  float den = use_gs ? sf * decode : sf;  // :237 / :239
-  float r = fminf(fast_rcp(den), FLT_MAX);
-  if (__builtin_amdgcn_ballot_w64(active && (!fast_div_ok(m) || !fast_div_ok(den))) != 0) {
-    s = m / 6.0f;
-    if (use_gs) s = s * gs;
-    s = fminf(s, FLT_MAX);
-    q8 = f32_to_e4m3_satfinite(s);
-    sf = e4m3_to_f32(q8);
-    den = use_gs ? sf * decode : sf;
-    r = fminf(1.0f / den, FLT_MAX);
-  }
+  float r;  // factor of the block's values ahead of the e2m1 cast
+  const uint32_t q8 = nvfp4_block_scale(m, use_gs, gs, decode, active, r);
 
   uint32_t p0 = 0, p1 = 0;
   if (!wave_nonfinite) {

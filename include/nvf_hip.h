@@ -160,10 +160,12 @@ NVF_API int nvf_nvfp4_scaled_mm_static_ws(const void* a, const void* b, const vo
                                           int out_dtype, void* stream);
 
 /* cutlass/nvfp4_scaled_mm_blockscale.cu:332-373 nvfp4_scaled_mm_blockscale (decl cutlass/nvf_cutlass.h:147-154).
- *   Operands as nvf_nvfp4_scaled_mm.  The fp32 product alpha * A * B^T is quantized again along n with
- *   the NVFP4 block quantizer (block 16, global scale *global_normconst): out_fp4 [m, n/2], out_scales
- *   e4m3 in the 128x4 layout of [roundUp(m,128), roundUp(n/16,4)].  workspace: m * n floats of device
- *   memory owned by the caller (the product lives there between the two launches). */
+ *   Operands as nvf_nvfp4_scaled_mm.  The fp32 product alpha * A * B^T is quantized again along n in the GEMM's own
+ *   epilogue (one launch, as the reference's fused epilogue :87-93), with the arithmetic of the NVFP4 block
+ *   quantizer (block 16, global scale *global_normconst): out_fp4 [m, n/2], out_scales e4m3 in the 128x4 layout of
+ *   [roundUp(m,128), roundUp(n/16,4)] (padding bytes of the last tiles written as 0).
+ *   workspace: NULL, or m * n floats of device memory that receive the fp32 product the result was quantized from
+ *   (a verification aid: it costs a second run of the GEMM). */
 NVF_API int nvf_nvfp4_scaled_mm_blockscale(const void* a, const void* b, const void* scales_a, const void* scales_b,
                                            const float* alpha, const float* global_normconst, void* out_fp4,
                                            void* out_scales, float* workspace, int64_t m, int64_t n, int64_t k,

@@ -61,7 +61,7 @@ def test_invalid_arguments_are_rejected_without_a_device():
     assert lib.nvf_nvfp4_scaled_mm(p, p, p, p, p, p, 128, 128, 64, capi.F32, None) == -1  # out dtype
     assert lib.nvf_mxfp8_scaled_mm(p, p, p, p, p, p, 128, 128, 40, capi.BF16, None) == -2
     assert lib.nvf_nvfp4_scaled_mm_blockscale(p, p, p, p, p, p, p, p, p, 128, 128, 48, None) == -2  # k % 32
-    assert lib.nvf_nvfp4_scaled_mm_blockscale(p, p, p, p, p, p, p, p, None, 128, 128, 64, None) == -1  # no workspace
+    assert lib.nvf_nvfp4_scaled_mm_blockscale(p, p, p, p, p, None, p, p, None, 128, 128, 64, None) == -1  # no global scale
     assert lib.nvf_nvfp4_scaled_mm_blockscale(None, None, None, None, None, None, None, None, None, 0, 128, 64, None) == 0
     assert lib.nvf_grouped_mm(p, p, p, p, p, 4, 128, 132, 64, capi.BF16, None) == -2  # n % 8
     assert lib.nvf_grouped_mm(p, p, p, p, p, 4, 128, 128, 64, capi.F32, None) == -1

@@ -82,12 +82,14 @@ def test_nvfp4_gemm_epilogue_reference_shapes(dev, dtype, shape):
     assert (unpack(q) != unpack(eq)).float().mean() < 2e-3 and (sf != esf).float().mean() < 2e-3
 
 
-@pytest.mark.parametrize("shape", [(200, 160, 192), (4096, 3072, 256)])
+@pytest.mark.parametrize("shape", [(200, 160, 192), (4096, 3072, 256), (1920, 4096, 384), (1024, 2048, 384), (300, 544, 608), (64, 96, 64),
+                                   (2176, 2048, 256), (4096, 4128, 128)])
 def test_nvfp4_gemm_epilogue_quantizes_its_own_fp32_product_bit_exactly(dev, shape):
-    """Through the C ABI, where the caller owns the workspace: the fp32 product left there agrees with the
-    oracle product to fp32 summation noise, and payload and scales are bit-identical to the oracle
-    quantizer applied to exactly that product (rows not a multiple of 128 and padded scale columns on the
-    tile kernel; a shape whose fp32 product comes from the persistent 256x256 kernel)."""
+    """Through the C ABI.  The result is quantized in the GEMM's epilogue; with a workspace the call also dumps the
+    fp32 product it quantized: that agrees with the oracle product to fp32 summation noise, and payload and scales
+    are bit-identical to the oracle quantizer applied to exactly that product (rows not a multiple of 128 and
+    padded scale columns on the 64x64, 128x128 and 256x256 tile kernels; shapes on the persistent kernel with
+    256x256 and with 128x256 tiles)."""
     from fuser_amd import capi
 
     m, n, k = shape
@@ -107,8 +109,14 @@ def test_nvfp4_gemm_epilogue_quantizes_its_own_fp32_product_bit_exactly(dev, sha
     assert max_rel(ws, prod) <= 1e-5
     eq, esf = O.block_quantize_nvfp4(ws.cpu(), norm, True)
     assert torch.equal(q.cpu(), eq)
-    valid = O.linear_to_swizzled_128_4(torch.ones(m, n // 16, dtype=torch.uint8)) != 0
-    assert torch.equal(sf.cpu()[valid], esf[valid])
+    assert torch.equal(sf.cpu(), esf)  # the padding bytes of the last 128x4 tiles are zero as well
+    # without the dump (what the at::Tensor layer calls): the same bytes from the one fused launch
+    q2 = torch.zeros_like(q)
+    sf2 = torch.full_like(sf, 0x55)
+    capi.check(capi.lib().nvf_nvfp4_scaled_mm_blockscale(d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), d[3].data_ptr(), al.data_ptr(),
+                                                         nc.data_ptr(), q2.data_ptr(), sf2.data_ptr(), None, m, n, k, None))
+    torch.cuda.synchronize()
+    assert torch.equal(q2, q) and torch.equal(sf2, sf)
 
 
 def test_config1_quantize_then_gemm(dev):
