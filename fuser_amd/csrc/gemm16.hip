@@ -1478,6 +1478,7 @@ int launch_nvfp4_skinny(const Params& p, int cus, hipStream_t stream) {
 template <bool BF16_MMA, bool OUT_BF16, bool STREAM_OUT>
 __global__ __launch_bounds__(256, 1) void grouped16_gemm_256_kernel(const Params p) {
   constexpr int BM = 256, BN = 256;
+  constexpr int kBand = 4;  // m-tiles that share a weight panel while it is in an XCD's L2 (8: measured no better)
   constexpr int TILE_UNITS = 2048;           // 16-byte units per operand tile (256 rows x 8 chunks)
   constexpr int BUF_UNITS = 2 * TILE_UNITS;  // A + B
   extern __shared__ u32x4 lds[];
@@ -1512,8 +1513,9 @@ __global__ __launch_bounds__(256, 1) void grouped16_gemm_256_kernel(const Params
     if (lane == 0) tile_prefix[0] = 0;
   }
   __syncthreads();
-  // Workgroup ids are dealt round-robin to the 8 XCDs.  The tiles of a group are walked in bands of 4 m-tiles, n-major
-  // inside a band, so that 32 consecutive tiles share 4 A and 8 B panels in an XCD's L2.  DEAL (n-tiles a multiple of
+  // Workgroup ids are dealt round-robin to the 8 XCDs.  The tiles of a group are walked in bands of up to 4 m-tiles,
+  // n-major inside a band, so that 32 consecutive tiles share 4 A and 8 B panels in an XCD's L2 and a weight panel
+  // comes in from memory once per band.  DEAL (n-tiles a multiple of
   // 8): XCD x takes the n-tiles x, x+8, ... of every band, i.e. its own list of (tiles / 8) tiles of the same make-up as
   // every other XCD's: each expert's weights stream in through all eight XCDs and all of them meet the cheap and
   // the expensive tiles (small groups are bound by streaming their weights once) at the same rate.  Otherwise XCD
@@ -1543,9 +1545,15 @@ __global__ __launch_bounds__(256, 1) void grouped16_gemm_256_kernel(const Params
     const int64_t row_off = __builtin_amdgcn_readfirstlane(p.expert_offsets[g]);
     const int tiles_m = (m_g + BM - 1) / BM;
     const int local = __builtin_amdgcn_readfirstlane(t - tile_prefix[g] * per_m);
-    const int band = local / (4 * per_m), in_band = local - band * 4 * per_m;
-    const int band_h = min(4, tiles_m - 4 * band);
-    const int ntl = in_band / band_h, mt = 4 * band + (in_band - ntl * band_h);
+    // bands of up to kBand m-tiles of near-equal height (9 m-tiles: 5 + 4), n-major inside a band
+    const int nb = (tiles_m + kBand - 1) / kBand, base_h = tiles_m / nb, taller = tiles_m - base_h * nb;  // the first `taller` bands have base_h + 1
+    const int mrow = local / per_m;  // m-tiles of the group that lie in earlier bands, plus a remainder
+    const int split = taller * (base_h + 1);
+    const int band = mrow < split ? mrow / (base_h + 1) : taller + (mrow - split) / base_h;
+    const int band_h = band < taller ? base_h + 1 : base_h;
+    const int band_m0 = band < taller ? band * (base_h + 1) : split + (band - taller) * base_h;
+    const int in_band = local - band_m0 * per_m;
+    const int ntl = in_band / band_h, mt = band_m0 + (in_band - ntl * band_h);
     const int nt = deal ? xcd + 8 * ntl : ntl;
     Tile r;
     r.a = p.a + (row_off + (int64_t)mt * BM) * kb;
