@@ -54,7 +54,7 @@ struct Params {
   // NVFP4 tile kernel, grouped: 1 = rows [0, rows & ~255) of every group are computed by the 256x256 kernel,
   // take only the rows after them
   int skip_whole_256 = 0;
-  // skinny kernel: first of the (at most 128) activation rows this launch computes, a multiple of 128
+  // skinny kernel: first activation row this launch computes (its slabs of 16*TT rows follow in blockIdx.y order)
   int m_base = 0;
   // grouped skinny kernel: the group sizes it serves; the tile kernel skips groups of fewer than min_rows rows
   int rows_lo = 0, rows_hi = 0, min_rows = 0;

@@ -199,9 +199,9 @@ def test_nvfp4_gemm_decode_sized_activations(dev, shape):
                                    (257, 32, 2048), (1024, 768, 2048), (2100, 96, 4096)])
 def test_nvfp4_gemm_many_rows_small_n_deep_k(dev, shape):
     """More than 256 rows with K >= 2048 and an N small enough that the workgroups of the kernel for decode-sized
-    activations (one per 128 rows x 16 columns) cover the compute units at most two or three times: all whole
-    128-row slabs go in one launch (2 to 16 slabs), the remaining rows (44, 104, 1, 52 or none) in a launch of
-    their own.  Every output element is compared with the oracle, with poisoned scale padding, both output
+    activations (one per 128 rows x 16 columns) cover the compute units at most two or three times: all slabs
+    (of 128, 64 or 32 rows, 3 to 33 of them, the last one ragged: 44, 104, 1, 52 rows or whole) go side by side in
+    one launch.  Every output element is compared with the oracle, with poisoned scale padding, both output
     types and run-to-run determinism."""
     m, n, k = shape
     gen = torch.Generator().manual_seed(m * 31 + n)

@@ -1,6 +1,6 @@
 """The entry points under HIP graph capture: no allocation of their own, no host synchronisation, no
 memset nodes.  A chain quantize -> global scale -> GEMMs (dense, decode-sized, split-K with torch-allocated
-scratch, grouped) is captured once and replayed several times with other work on the stream in between;
+scratch, grouped, block-scaled result) is captured once and replayed several times with other work on the stream in between;
 every replay must reproduce the eager results bit for bit, also after the inputs have been overwritten in
 place."""
 import pytest
@@ -51,7 +51,13 @@ def test_chain_replays_bit_exactly(dev):
         f8a, e8a = ops.nv_block_quantize(x, None, True, 32, torch.float8_e4m3fn)
         f8b, e8b = ops.nv_block_quantize(w, None, True, 32, torch.float8_e4m3fn)
         mx = nvf_cutlass.mxfp8_scaled_mm(f8a, f8b, e8a, e8b, one, torch.bfloat16)
-        return [gs, dense, decode, split, grouped[: sum(sizes)], bf[: sum(sizes)], mx]
+        # block-scaled result: fused epilogue on the persistent kernel, and a ragged shape whose scale padding is
+        # cleared by a fill kernel (no memset node)
+        bq, bsf = nvf_cutlass.nvfp4_scaled_mm_blockscale(xq, wq, xsf, wsf, one, one)
+        rq, rsf = nvf_cutlass.nvfp4_scaled_mm_blockscale(xq[:200].contiguous(), wq[:160].contiguous(), xsf[:256].contiguous(),
+                                                         wsf[:256].contiguous(), one, one)
+        return [gs, dense, decode, split, grouped[: sum(sizes)], bf[: sum(sizes)], mx, bq.view(torch.uint8), bsf.view(torch.uint8),
+                rq.view(torch.uint8), rsf.view(torch.uint8)]
 
     eager = [t.clone() for t in chain()]  # also the warm-up: function attributes are set outside the capture
     torch.cuda.synchronize()
