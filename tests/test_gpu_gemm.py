@@ -119,6 +119,48 @@ def test_nvfp4_gemm_epilogue_quantizes_its_own_fp32_product_bit_exactly(dev, sha
     assert torch.equal(q2, q) and torch.equal(sf2, sf)
 
 
+def test_nvfp4_gemm_epilogue_random_shapes_and_codes(dev):
+    """Sixty seeded cases over every tile kernel: arbitrary payload bytes (all sixteen e2m1 codes, both signs),
+    scale codes over 2^-10..2^1, all-zero rows, several alpha and norm constants.  Payload and scales equal the
+    oracle quantizer applied to the dumped fp32 product, byte for byte, padding of the scale layout included."""
+    import random
+
+    from fuser_amd import capi
+
+    rnd = random.Random(5)
+    lib = capi.lib()
+    for case in range(60):
+        kind = ("persistent", "half_tiles", "ragged", "tiny")[case % 4]
+        if kind == "persistent":
+            m, n, k = 256 * rnd.randint(1, 8), 256 * rnd.randint(1, 8), 128 * rnd.randint(2, 6)
+        elif kind == "half_tiles":
+            m, n, k = 128 * rnd.randint(1, 16), 256 * rnd.randint(1, 8), 128 * rnd.randint(2, 5)
+        elif kind == "ragged":
+            m, n, k = rnd.randint(1, 700), 32 * rnd.randint(1, 40), 32 * rnd.randint(1, 20)
+        else:
+            m, n, k = rnd.randint(1, 64), 32 * rnd.randint(1, 6), 32 * rnd.randint(1, 8)
+        g = torch.Generator(device=dev).manual_seed(case)
+        a = torch.randint(0, 256, (m, k // 2), dtype=torch.uint8, device=dev, generator=g)
+        b = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device=dev, generator=g)
+        sa = torch.randint(0x28, 0x48, (O.round_up(m, 128), O.round_up(k // 16, 4)), dtype=torch.uint8, device=dev, generator=g)
+        sb = torch.randint(0x28, 0x48, (O.round_up(n, 128), O.round_up(k // 16, 4)), dtype=torch.uint8, device=dev, generator=g)
+        if case % 5 == 0:
+            a[rnd.randrange(m)] = 0  # a row of zero blocks
+        alpha, norm = rnd.choice([1.0, 0.37, 2.0**-8]), rnd.choice([1.0, 2.0, 26.88, 1e-3])
+        al, nc = torch.tensor(alpha, dtype=torch.float32, device=dev), torch.tensor(norm, dtype=torch.float32, device=dev)
+        q = torch.zeros(m, n // 2, dtype=torch.uint8, device=dev)
+        sf = torch.full((O.round_up(m, 128), O.round_up(n // 16, 4)), 0x55, dtype=torch.uint8, device=dev)
+        ws = torch.zeros(m, n, dtype=torch.float32, device=dev)
+        capi.check(lib.nvf_nvfp4_scaled_mm_blockscale(a.data_ptr(), b.data_ptr(), sa.data_ptr(), sb.data_ptr(), al.data_ptr(), nc.data_ptr(),
+                                                      q.data_ptr(), sf.data_ptr(), ws.data_ptr(), m, n, k, None))
+        torch.cuda.synchronize()
+        eq, esf = O.block_quantize_nvfp4(ws.cpu(), norm, True)
+        assert torch.equal(q.cpu(), eq) and torch.equal(sf.cpu(), esf), (kind, m, n, k, alpha, norm)
+        if case % 6 == 0:  # the dumped product itself, against the oracle GEMM
+            ref = O.ref_nvfp4_scaled_mm(a.cpu(), b.cpu(), sa.cpu(), sb.cpu(), alpha)
+            assert max_rel(ws, ref) <= 1e-5, (kind, m, n, k)
+
+
 def test_config1_quantize_then_gemm(dev):
     """BASELINE config 1: A [256,1024], B [1024,1024] N(0,1) bf16, quantized on the GPU, C = A B^T bf16."""
     from fuser_amd import nvf_cutlass, ops
