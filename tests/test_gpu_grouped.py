@@ -90,6 +90,32 @@ def test_grouped_mm_persistent_256_tile_kernel_full_compare(dev, tensor_dtype, k
     assert ((out[:rows].float().cpu() - ref[:rows]).abs() / scale).max().item() <= GEMM_MAX_REL
 
 
+@pytest.mark.parametrize("n,k", [(2048, 192), (2304, 128), (4096, 320), (2304, 1024)])
+def test_grouped_mm_group_ends_inside_tiles(dev, n, k):
+    """Persistent 256-row-tile kernel: groups that end 128, 129, 1, 100 and 127 rows into a tile, groups smaller than
+    half a tile, N with 8 | N/256 (n-tiles dealt to the XCDs) and without, two to 16 K steps.  Every element
+    compared, rows after the last group untouched."""
+    from fuser_amd import capi
+
+    sizes = [384, 128, 129, 895, 100, 2048 + 127, 256, 0, 257]
+    m = sum(sizes) + 5
+    gen = torch.Generator().manual_seed(n + k)
+    a = torch.randn(m, k, generator=gen).bfloat16()
+    b = (torch.randn(len(sizes), n, k, generator=gen) * 0.05).bfloat16()
+    ps, eo, _, _ = _grouped_args(sizes, n, k, dev)
+    ad, bd, psd, eod = a.to(dev), b.to(dev), ps.to(dev), eo.to(dev)
+    assert capi.describe_dispatch("grouped_mm", m, n, k, groups=len(sizes)).startswith("grouped16_gemm_256_kernel")
+    out = torch.full((m, n), 7.0, dtype=torch.bfloat16, device=dev)
+    capi.check(capi.lib().nvf_grouped_mm(ad.data_ptr(), bd.data_ptr(), out.data_ptr(), psd.data_ptr(), eod.data_ptr(), len(sizes),
+                                         m, n, k, capi.BF16, None))
+    torch.cuda.synchronize()
+    ref = O.ref_grouped_mm(a, b, ps, eo)
+    rows = sum(sizes)
+    assert (out[rows:] == 7.0).all()
+    scale = ref[:rows].abs().amax(dim=1, keepdim=True).clamp(min=1e-30)
+    assert ((out[:rows].float().cpu() - ref[:rows]).abs() / scale).max().item() <= GEMM_MAX_REL
+
+
 def _moe_sizes_top2(tokens, experts, seed):
     gen = torch.Generator().manual_seed(seed)
     logits = torch.randn(tokens, experts, generator=gen) + torch.linspace(-1.5, 1.5, experts)
