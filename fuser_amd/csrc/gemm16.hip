@@ -1263,58 +1263,137 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
     rd_asc[tt] = (NT + B_SC + (tt >> 1)) * 1024 + ((tt & 1) * 2 + (g >> 1)) * 256 + r * 16 + (asf_word0 + ((tt * 16) >> 5)) * 4;
   const int sc_shift = (g & 1) * 16;
 
-  f32x4 acc[RT][TT];
+  const float alpha = p.alpha[grp];
+  uint16_t* out = static_cast<uint16_t*>(p.out);
+  // Accumulators acc[RT][TTC] of the TTC activation tiles this workgroup was compiled for (tt_count <= TTC of them
+  // hold rows) -> result: stored directly (NSPLIT) or summed over the wavefronts through LDS.
+  auto finish = [&](auto ttc_c, auto& acc) {
+    constexpr int TTC = decltype(ttc_c)::value;
+    if constexpr (NSPLIT) {
+      // every wavefront holds finished sums: element e of lane l = weight row 4*(l/16) + e, activation row l%16
 #pragma unroll
-  for (int rt = 0; rt < RT; ++rt)
+      for (int tt = 0; tt < TTC; ++tt) {
+        const int tok = tt * 16 + r;
+        if (tok < m_loc) {
 #pragma unroll
-    for (int tt = 0; tt < TT; ++tt) acc[rt][tt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+          for (int rt = 0; rt < RT; ++rt) {
+            u32x2 v;
+            v[0] = pack2(acc[rt][tt][0] * alpha, acc[rt][tt][1] * alpha, OUT_BF16);
+            v[1] = pack2(acc[rt][tt][2] * alpha, acc[rt][tt][3] * alpha, OUT_BF16);
+            *reinterpret_cast<u32x2*>(out + (a_row0 + tok) * p.n + n0 + rt * 16 + 4 * g) = v;
+          }
+        }
+      }
+      return;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no LDS-direct load may be pending when the ring is reused
+    __syncthreads();
+
+    // ---- sum the wavefronts' partial tiles in wave order and store: all tiles in one round if they fit the
+    // ring's memory (RT * TT <= 8), else one round per weight-row tile
+    constexpr int ROUNDS = RT * TT <= 8 ? 1 : RT;
+    constexpr int RPR = RT / ROUNDS;  // weight-row tiles per round
+    const int tiles = RPR * tt_count;   // tile index inside a round: rt * tt_count + tt
+    const int units = tiles * 64;
+#pragma unroll
+    for (int round = 0; round < ROUNDS; ++round) {
+      if (round > 0) __syncthreads();
+#pragma unroll
+      for (int r2 = 0; r2 < RPR; ++r2)
+#pragma unroll
+        for (int tt = 0; tt < TTC; ++tt)
+          if (tt < tt_count) red[(wave * tiles + r2 * tt_count + tt) * 64 + lane] = acc[round * RPR + r2][tt];
+      __syncthreads();
+      for (int u = tid; u < units; u += 512) {
+        const int l = u & 63, tile = u >> 6;
+        const int r2 = tile / tt_count, tt = tile - r2 * tt_count;
+        f32x4 s = red[u];
+#pragma unroll
+        for (int w = 1; w < W; ++w) s += red[w * units + u];
+        const int tok = tt * 16 + (l & 15);
+        if (tok < m_loc) {
+          u32x2 v;
+          v[0] = pack2(s[0] * alpha, s[1] * alpha, OUT_BF16);
+          v[1] = pack2(s[2] * alpha, s[3] * alpha, OUT_BF16);
+          *reinterpret_cast<u32x2*>(out + (a_row0 + tok) * p.n + n0 + (round * RPR + r2) * 16 + 4 * (l >> 4)) = v;
+        }
+      }
+    }
+  };
 
   constexpr int CSTEP = NSPLIT ? 1 : W;  // distance of a wavefront's consecutive chunks
   const int c_first = NSPLIT ? 0 : wave;
+  // Many activation tiles (TT > 2): the slot is refilled tile by tile.  A chunk's loads are issued in a fixed order -
+  // the weight tiles and their scale blocks, then activation tile 0, 1, scale block 0, tile 2, 3, scale block 1, ... -
+  // each as soon as its place in LDS has been read out, so every load has a whole chunk's conversion and MFMA time
+  // to land, and the waits are for counts that follow from that order (loads complete in the order of issue).
+  constexpr bool kFineRing = TT > 2 && DEPTH == 1;
+  if constexpr (kFineRing) {
+    constexpr int LB = RT + B_SC;  // loads of the weight part
+    auto load_b_part = [&](uint32_t c) {
 #pragma unroll
-  for (int d = 0; d < DEPTH; ++d) issue_chunk(c_first + d * CSTEP, d);
-  int slot = 0;
-  for (int c = c_first; c < chunks; c += CSTEP) {
-    // the oldest chunk in flight has landed when only the loads of the next one (if there is one) are pending
-    if (DEPTH == 2 && c + CSTEP < chunks)
-      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NDMA) : "memory");
-    else
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    const char* sp = reinterpret_cast<const char*>(red) + (wave * DEPTH + slot) * SLOT_BYTES;
-    // the activation tiles are read out of LDS together with the weight tiles (few of them) or one at a time
-    // right before their conversion (many: their registers would not fit)
-    constexpr bool kLazyA = TT > 2;
-    constexpr int NQ = kLazyA ? RT : NT;
-    u32x4 q[NQ];
-    uint32_t sc[NQ];
+      for (int rt = 0; rt < RT; ++rt) lds_dma16(ring_base + rt * 1024, b_base, b_off[rt] + c * 64u);
 #pragma unroll
-    for (int t = 0; t < NQ; ++t) q[t] = *reinterpret_cast<const u32x4*>(sp + t * 1024 + rd_payload);
+      for (int j = 0; j < B_SC; ++j) lds_dma16(ring_base + (NT + j) * 1024, bsf_base, bsf_off[j] + c * 1024u);
+    };
+    int fine_lrow = lrow;  // re-derived per use: eight row offsets kept in registers would not fit
+    auto load_a_tile = [&](uint32_t c, int tt) {
+      asm volatile("" : "+v"(fine_lrow));
+      lds_dma16(ring_base + (RT + tt) * 1024, a_base, (uint32_t)min(tt * 16 + fine_lrow, m_loc - 1) * (uint32_t)kbytes + lpiece * 16 + c * 64u);
+    };
+    auto load_a_scales = [&](uint32_t c, int j) { lds_dma16(ring_base + (NT + B_SC + j) * 1024, asf_base, asf_off[j] + c * 1024u); };
+    const char* sp = reinterpret_cast<const char*>(red) + wave * SLOT_BYTES;
+    auto read_a_tile = [&](int tt, u32x4& aq, uint32_t& as) {
+      aq = *reinterpret_cast<const u32x4*>(sp + (RT + tt) * 1024 + rd_payload);
+      as = *reinterpret_cast<const uint32_t*>(sp + rd_asc[tt]) >> sc_shift;
+    };
+    // one chunk with TTC activation tiles; REFILL: this wavefront has another chunk after it
+    auto chunk = [&](auto ttc_c, auto refill_c, uint32_t c, auto& acc) {
+      constexpr int TTC = decltype(ttc_c)::value;
+      constexpr bool REFILL = decltype(refill_c)::value;
+      constexpr int JC = (TTC + 1) / 2, LA = TTC + JC;  // activation scale blocks, loads of the activation part
+      const uint32_t cn = c + CSTEP;
+      // the weight part was issued first: only the activation part of this chunk may still be on its way
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LA) : "memory");
+      u32x4 q[RT];
+      uint32_t sc[RT];
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt) sc[rt] = *reinterpret_cast<const uint32_t*>(sp + rd_bsc[rt]) >> sc_shift;
-    if constexpr (!kLazyA) {
+      for (int rt = 0; rt < RT; ++rt) q[rt] = *reinterpret_cast<const u32x4*>(sp + rt * 1024 + rd_payload);
 #pragma unroll
-      for (int tt = 0; tt < TT; ++tt) sc[RT + tt] = *reinterpret_cast<const uint32_t*>(sp + rd_asc[tt]) >> sc_shift;
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // read out: the slot may be refilled
-      issue_chunk(c + DEPTH * CSTEP, slot);
-    }
-    u32x4 fb[RT][4];
+      for (int rt = 0; rt < RT; ++rt) sc[rt] = *reinterpret_cast<const uint32_t*>(sp + rd_bsc[rt]) >> sc_shift;
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // read out: may be refilled
+      if constexpr (REFILL) load_b_part(cn);
+      // Scale block j follows tiles 2j and 2j+1 in the order of issue (position 3j+2 of the activation part; 3j+1
+      // behind a last tile without a partner).  Behind it, when it is needed: the rest of this chunk's activation
+      // part and, with REFILL, what has been issued for the next chunk by then (weight part and 3j loads).
+      u32x4 fb[RT][4];
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt) dequant_frags(q[rt], sc[rt], fb[rt]);
+      for (int rt = 0; rt < RT; ++rt) dequant_frags(q[rt], sc[rt], fb[rt]);
 #pragma unroll
-    for (int tt = 0; tt < TT; ++tt) {
-      if (tt < tt_count) {
+      for (int tt = 0; tt < TTC; ++tt) {
+        __builtin_amdgcn_sched_barrier(0);  // tile by tile: scheduled across tiles, the block would not fit the registers
+        if ((tt & 1) == 0) {
+          const int j = tt >> 1;
+          const int pos = 3 * j + (2 * j + 1 < TTC ? 2 : 1);
+          const int behind = LA - 1 - pos + (REFILL ? LB + 3 * j : 0);
+          // (one s_waitcnt per possible count: the operand is an immediate)
+          switch (behind) {
+#define NVF_VMCNT_CASE(n) case n: asm volatile("s_waitcnt vmcnt(" #n ")" ::: "memory"); break;
+            NVF_VMCNT_CASE(0) NVF_VMCNT_CASE(1) NVF_VMCNT_CASE(2) NVF_VMCNT_CASE(3) NVF_VMCNT_CASE(4) NVF_VMCNT_CASE(5)
+            NVF_VMCNT_CASE(6) NVF_VMCNT_CASE(7) NVF_VMCNT_CASE(8) NVF_VMCNT_CASE(9) NVF_VMCNT_CASE(10) NVF_VMCNT_CASE(11)
+            NVF_VMCNT_CASE(12) NVF_VMCNT_CASE(13) NVF_VMCNT_CASE(14) NVF_VMCNT_CASE(15) NVF_VMCNT_CASE(16) NVF_VMCNT_CASE(17)
+            NVF_VMCNT_CASE(18) NVF_VMCNT_CASE(19) NVF_VMCNT_CASE(20)
+#undef NVF_VMCNT_CASE
+            default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+          }
+        }
         u32x4 aq;
         uint32_t as;
-        if constexpr (kLazyA) {
-          aq = *reinterpret_cast<const u32x4*>(sp + (RT + tt) * 1024 + rd_payload);
-          as = *reinterpret_cast<const uint32_t*>(sp + rd_asc[tt]) >> sc_shift;
-          if (tt + 1 == tt_count) {
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the last read of the slot is complete
-            issue_chunk(c + DEPTH * CSTEP, slot);
-          }
-        } else {
-          aq = q[kLazyA ? 0 : RT + tt];
-          as = sc[kLazyA ? 0 : RT + tt];
+        read_a_tile(tt, aq, as);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // tile tt has been read out
+        if constexpr (REFILL) {
+          load_a_tile(cn, tt);
+          if ((tt & 1) || tt + 1 == TTC) load_a_scales(cn, tt >> 1);
         }
         u32x4 fa[4];
         dequant_frags(aq, as, fa);
@@ -1325,60 +1404,146 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
             acc[rt][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, fb[rt][t]),
                                                                  __builtin_bit_cast(f16x8, fa[t]), acc[rt][tt], 0, 0, 0);
       }
-    }
-    if constexpr (DEPTH == 2) slot ^= 1;
-  }
-  const float alpha = p.alpha[grp];
-  uint16_t* out = static_cast<uint16_t*>(p.out);
-  if constexpr (NSPLIT) {
-    // every wavefront holds finished sums: element e of lane l = weight row 4*(l/16) + e, activation row l%16
+    };
+    // One whole-slot refill per chunk, as in the kernels with few activation tiles: for tile counts whose
+    // accumulators leave no registers for the finer scheme.
+    auto chunk_coarse = [&](auto ttc_c, uint32_t c, auto& acc) {
+      constexpr int TTC = decltype(ttc_c)::value;
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      u32x4 q[RT];
+      uint32_t sc[RT];
 #pragma unroll
-    for (int tt = 0; tt < TT; ++tt) {
-      const int tok = tt * 16 + r;
-      if (tok < m_loc) {
+      for (int rt = 0; rt < RT; ++rt) q[rt] = *reinterpret_cast<const u32x4*>(sp + rt * 1024 + rd_payload);
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt) {
-          u32x2 v;
-          v[0] = pack2(acc[rt][tt][0] * alpha, acc[rt][tt][1] * alpha, OUT_BF16);
-          v[1] = pack2(acc[rt][tt][2] * alpha, acc[rt][tt][3] * alpha, OUT_BF16);
-          *reinterpret_cast<u32x2*>(out + (a_row0 + tok) * p.n + n0 + rt * 16 + 4 * g) = v;
+      for (int rt = 0; rt < RT; ++rt) sc[rt] = *reinterpret_cast<const uint32_t*>(sp + rd_bsc[rt]) >> sc_shift;
+      u32x4 fb[RT][4];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) dequant_frags(q[rt], sc[rt], fb[rt]);
+#pragma unroll
+      for (int tt = 0; tt < TTC; ++tt) {
+        __builtin_amdgcn_sched_barrier(0);
+        u32x4 aq;
+        uint32_t as;
+        read_a_tile(tt, aq, as);
+        if (tt + 1 == TTC) {
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the last read of the slot is complete
+          if (c + CSTEP < (uint32_t)chunks) {
+            load_b_part(c + CSTEP);
+#pragma unroll
+            for (int t2 = 0; t2 < TTC; ++t2) {
+              load_a_tile(c + CSTEP, t2);
+              if ((t2 & 1) || t2 + 1 == TTC) load_a_scales(c + CSTEP, t2 >> 1);
+            }
+          }
+        }
+        u32x4 fa[4];
+        dequant_frags(aq, as, fa);
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt)
+            acc[rt][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, fb[rt][t]),
+                                                                 __builtin_bit_cast(f16x8, fa[t]), acc[rt][tt], 0, 0, 0);
+      }
+    };
+    auto run = [&](auto ttc_c) {
+      constexpr int TTC = decltype(ttc_c)::value;
+      constexpr bool kFits = RT * TTC <= 20;  // accumulator registers that leave room for the finer scheme
+      f32x4 acc[RT][TTC];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int tt = 0; tt < TTC; ++tt) acc[rt][tt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+      if (c_first < chunks) {
+        load_b_part((uint32_t)c_first);
+#pragma unroll
+        for (int tt = 0; tt < TTC; ++tt) {
+          load_a_tile((uint32_t)c_first, tt);
+          if ((tt & 1) || tt + 1 == TTC) load_a_scales((uint32_t)c_first, tt >> 1);
         }
       }
-    }
-    return;
-  }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no LDS-direct load may be pending when the ring is reused
-  __syncthreads();
-
-  // ---- sum the wavefronts' partial tiles in wave order and store: all tiles in one round if they fit the
-  // ring's memory (RT * TT <= 8), else one round per weight-row tile
-  constexpr int ROUNDS = RT * TT <= 8 ? 1 : RT;
-  constexpr int RPR = RT / ROUNDS;  // weight-row tiles per round
-  const int tiles = RPR * tt_count;   // tile index inside a round: rt * tt_count + tt
-  const int units = tiles * 64;
-#pragma unroll
-  for (int round = 0; round < ROUNDS; ++round) {
-    if (round > 0) __syncthreads();
-#pragma unroll
-    for (int r2 = 0; r2 < RPR; ++r2)
-#pragma unroll
-      for (int tt = 0; tt < TT; ++tt)
-        if (tt < tt_count) red[(wave * tiles + r2 * tt_count + tt) * 64 + lane] = acc[round * RPR + r2][tt];
-    __syncthreads();
-    for (int u = tid; u < units; u += 512) {
-      const int l = u & 63, tile = u >> 6;
-      const int r2 = tile / tt_count, tt = tile - r2 * tt_count;
-      f32x4 s = red[u];
-#pragma unroll
-      for (int w = 1; w < W; ++w) s += red[w * units + u];
-      const int tok = tt * 16 + (l & 15);
-      if (tok < m_loc) {
-        u32x2 v;
-        v[0] = pack2(s[0] * alpha, s[1] * alpha, OUT_BF16);
-        v[1] = pack2(s[2] * alpha, s[3] * alpha, OUT_BF16);
-        *reinterpret_cast<u32x2*>(out + (a_row0 + tok) * p.n + n0 + (round * RPR + r2) * 16 + 4 * (l >> 4)) = v;
+      for (int c = c_first; c < chunks; c += CSTEP) {
+        if constexpr (!kFits) chunk_coarse(ttc_c, (uint32_t)c, acc);
+        else if (c + CSTEP < chunks) chunk(ttc_c, std::true_type{}, (uint32_t)c, acc);
+        else chunk(ttc_c, std::false_type{}, (uint32_t)c, acc);
       }
+      finish(ttc_c, acc);
+    };
+    switch (tt_count) {
+      case 1: run(std::integral_constant<int, 1>{}); break;
+      case 2: run(std::integral_constant<int, 2>{}); break;
+      case 3: run(std::integral_constant<int, 3>{}); break;
+      case 4: run(std::integral_constant<int, (TT >= 4 ? 4 : 1)>{}); break;
+      case 5: run(std::integral_constant<int, (TT >= 5 ? 5 : 1)>{}); break;
+      case 6: run(std::integral_constant<int, (TT >= 6 ? 6 : 1)>{}); break;
+      case 7: run(std::integral_constant<int, (TT >= 7 ? 7 : 1)>{}); break;
+      case 8: run(std::integral_constant<int, (TT >= 8 ? 8 : 1)>{}); break;
+      default: break;
     }
+  } else {
+    f32x4 acc[RT][TT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int tt = 0; tt < TT; ++tt) acc[rt][tt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) issue_chunk(c_first + d * CSTEP, d);
+    int slot = 0;
+    for (int c = c_first; c < chunks; c += CSTEP) {
+      // the oldest chunk in flight has landed when only the loads of the next one (if there is one) are pending
+      if (DEPTH == 2 && c + CSTEP < chunks)
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NDMA) : "memory");
+      else
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      const char* sp = reinterpret_cast<const char*>(red) + (wave * DEPTH + slot) * SLOT_BYTES;
+      // the activation tiles are read out of LDS together with the weight tiles (few of them) or one at a time
+      // right before their conversion (many: their registers would not fit)
+      constexpr bool kLazyA = TT > 2;
+      constexpr int NQ = kLazyA ? RT : NT;
+      u32x4 q[NQ];
+      uint32_t sc[NQ];
+#pragma unroll
+      for (int t = 0; t < NQ; ++t) q[t] = *reinterpret_cast<const u32x4*>(sp + t * 1024 + rd_payload);
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) sc[rt] = *reinterpret_cast<const uint32_t*>(sp + rd_bsc[rt]) >> sc_shift;
+      if constexpr (!kLazyA) {
+#pragma unroll
+        for (int tt = 0; tt < TT; ++tt) sc[RT + tt] = *reinterpret_cast<const uint32_t*>(sp + rd_asc[tt]) >> sc_shift;
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // read out: the slot may be refilled
+        issue_chunk(c + DEPTH * CSTEP, slot);
+      }
+      u32x4 fb[RT][4];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) dequant_frags(q[rt], sc[rt], fb[rt]);
+#pragma unroll
+      for (int tt = 0; tt < TT; ++tt) {
+        if (tt < tt_count) {
+          u32x4 aq;
+          uint32_t as;
+          if constexpr (kLazyA) {
+            aq = *reinterpret_cast<const u32x4*>(sp + (RT + tt) * 1024 + rd_payload);
+            as = *reinterpret_cast<const uint32_t*>(sp + rd_asc[tt]) >> sc_shift;
+            if (tt + 1 == tt_count) {
+              asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the last read of the slot is complete
+              issue_chunk(c + DEPTH * CSTEP, slot);
+            }
+          } else {
+            aq = q[kLazyA ? 0 : RT + tt];
+            as = sc[kLazyA ? 0 : RT + tt];
+          }
+          u32x4 fa[4];
+          dequant_frags(aq, as, fa);
+#pragma unroll
+          for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+              acc[rt][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, fb[rt][t]),
+                                                                   __builtin_bit_cast(f16x8, fa[t]), acc[rt][tt], 0, 0, 0);
+        }
+      }
+      if constexpr (DEPTH == 2) slot ^= 1;
+    }
+    finish(std::integral_constant<int, TT>{}, acc);
   }
 }
 
