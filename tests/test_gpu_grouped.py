@@ -303,6 +303,50 @@ def test_nvfp4_grouped_mm_small_groups_stream_their_weights(dev, n, k):
         assert torch.equal(out[:rows], nvf_cutlass.nvfp4_scaled_grouped_mm(*args, dtype)[:rows])
 
 
+@pytest.mark.parametrize("n,k", [(512, 4096), (1024, 4224)])
+def test_nvfp4_grouped_mm_mid_sized_groups_of_a_prefill(dev, n, k):
+    """A prefill-sized call (2048 rows or more) with K >= 4096 and N % 512 == 0: groups of 33..80 rows run on the kernel
+    that converts a group's activation rows once per 512 weight rows (work items found from the device-resident
+    sizes; three, four and five row tiles, sizes on both sides of its borders), their neighbours of 81..128 rows on
+    the streaming kernel, larger ones on the tile kernels.  33 K chunks: the odd and the even LDS slot both end a
+    walk.  A different alpha per group, poisoned padding of the activation scale slabs; every element compared, rows
+    after the last group untouched, run-to-run bit equality."""
+    from fuser_amd import capi, nvf_cutlass
+
+    sizes = [33, 80, 48, 49, 64, 65, 81, 32, 0, 128, 34, 47, 79, 300, 66, 50, 40, 72, 1, 129] + [56, 77, 35, 63] * 6
+    g, m = len(sizes), sum(sizes) + 3
+    assert sum(sizes) >= 2048
+    assert "nvfp4_group_panel_kernel" in capi.describe_dispatch("nvfp4_scaled_grouped_mm", m, n, k, groups=g)
+    gen = torch.Generator().manual_seed(n + k)
+    x = torch.randn(m, k, generator=gen).bfloat16()
+    w = (torch.randn(g, n, k, generator=gen) * 0.05).bfloat16()
+    ps, eo, st, ct = _grouped_args(sizes, n, k, dev)
+    so = start_offsets([O.round_up(t, 128) for t in sizes])
+    aq, valid = O.grouped_block_quantize_nvfp4(x, eo, so, None)
+    lin = torch.zeros_like(valid, dtype=torch.bool)
+    for e, t in enumerate(sizes):
+        if t:
+            ones = O.linear_to_swizzled_128_4(torch.ones(t, k // 16, dtype=torch.uint8))
+            lin[int(so[e]) : int(so[e]) + ones.shape[0]] |= ones.bool()
+    asf = torch.where(lin, valid, torch.full_like(valid, 0x7F))  # NaN code wherever no row owns the byte
+    bq = torch.empty(g, n, k // 2, dtype=torch.uint8)
+    bsf = torch.empty(g, n, k // 16, dtype=torch.uint8)
+    alphas = torch.empty(g)
+    for e in range(g):
+        gs = gs_of(w[e])
+        bq[e], bsf[e] = O.block_quantize_nvfp4(w[e], gs, True)
+        alphas[e] = (e % 7 + 1) / gs
+    ref = O.ref_nvfp4_scaled_grouped_mm(aq, bq, valid, bsf, alphas, ps, eo, so)
+    rows = sum(sizes)
+    args = (fp4(aq.to(dev)), fp4(bq.to(dev)), e4m3(asf.to(dev)), e4m3(bsf.to(dev)), alphas.to(dev), st, ct, ps.to(dev), eo.to(dev), so.to(dev))
+    for dtype in (torch.bfloat16, torch.float16):
+        out = nvf_cutlass.nvfp4_scaled_grouped_mm(*args, dtype)
+        torch.cuda.synchronize()
+        scale = ref[:rows].abs().amax(dim=1, keepdim=True).clamp(min=1e-30)
+        assert ((out[:rows].float().cpu() - ref[:rows]).abs() / scale).max().item() <= GEMM_MAX_REL, (n, k, dtype)
+        assert torch.equal(out[:rows], nvf_cutlass.nvfp4_scaled_grouped_mm(*args, dtype)[:rows])
+
+
 def _zipf_sizes(tokens, topk, experts, s, seed):
     gen = torch.Generator().manual_seed(seed)
     p = 1.0 / torch.arange(1, experts + 1).float() ** s
