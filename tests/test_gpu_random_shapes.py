@@ -98,7 +98,9 @@ def test_grouped_mm_random_groups(dev, case):
     assert _rowwise_rel(out, ref) <= GEMM_MAX_REL
 
 
-@pytest.mark.parametrize("case", [(4, 600, 128, 128), (7, 1500, 256, 192), (3, 2048, 512, 320), (12, 900, 384, 64)])
+@pytest.mark.parametrize("case", [(4, 600, 128, 128), (7, 1500, 256, 192), (3, 2048, 512, 320), (12, 900, 384, 64),
+                                  # prefill-sized with many small experts and a deep K: every kernel of the grouped op in one call
+                                  (40, 2600, 512, 4096), (33, 2200, 1024, 4224), (64, 4200, 512, 4352)])
 def test_nvfp4_scaled_grouped_mm_random_groups(dev, case):
     from fuser_amd import nvf_cutlass, ops
 
