@@ -2439,12 +2439,11 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int6
         rc = launch_nvfp4_skinny_grouped<2, 8, OUT_BF16, true>(p, 33, 128, stream);
       } else if ((p.n & 511) == 0) {
         rc = launch_nvfp4_group_panel<4, 5, 2, OUT_BF16>(p, 33, 80, stream);
-        if (rc == NVF_OK) rc = launch_nvfp4_skinny_grouped<4, 8, OUT_BF16, false>(p, 81, 128, stream);
         if (rc == NVF_OK) {
-          // the ends of the groups that the 256x256 kernel takes: 128x256 tiles of the persistent kernel (no whole
-          // group falls into the empty range 129..128), at 1.2 times the rate of the 128x128 tile kernel
+          // groups of 81..128 rows and the ends of the groups that the 256x256 kernel takes: 128x256 tiles of the
+          // persistent kernel, at 1.2 times the rate of the 128x128 tile kernel
           Params ends = p;
-          ends.rows_lo = 129;
+          ends.rows_lo = 81;
           ends.rows_hi = 128;
           ends.min_rows = 129;
           tail_done = 1;

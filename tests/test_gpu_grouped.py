@@ -307,8 +307,8 @@ def test_nvfp4_grouped_mm_small_groups_stream_their_weights(dev, n, k):
 def test_nvfp4_grouped_mm_mid_sized_groups_of_a_prefill(dev, n, k):
     """A prefill-sized call (2048 rows or more) with K >= 4096 and N % 512 == 0: groups of 33..80 rows run on the kernel
     that converts a group's activation rows once per 512 weight rows (work items found from the device-resident
-    sizes; three, four and five row tiles, sizes on both sides of its borders), their neighbours of 81..128 rows on
-    the streaming kernel, larger ones on the tile kernels.  33 K chunks: the odd and the even LDS slot both end a
+    sizes; three, four and five row tiles, sizes on both sides of its borders), their neighbours of 81..128 rows and
+    the ends of the larger ones on 128x256 tiles of the persistent kernel, the rest of those on its 256x256 tiles.  33 K chunks: the odd and the even LDS slot both end a
     walk.  A different alpha per group, poisoned padding of the activation scale slabs; every element compared, rows
     after the last group untouched, run-to-run bit equality."""
     from fuser_amd import capi, nvf_cutlass
