@@ -2434,6 +2434,13 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int6
         mid.rows_hi = 128;
         if (m_hint >= 2048) mid.min_rows = 129;  // the 256x256 kernel follows: take the ends of its groups along
         tail_done = mid.min_rows != 0;
+        if (m_hint >= 2048 && (p.n & 511) == 0 && p.k >= 1024) {
+          // a prefill: the groups of up to 80 rows on the panel kernel, which multiplies row tiles of 16 (config 5,
+          // K=2048: 5376 tiles of 128x256 in 680 us -> 325 us + 1792 tiles in 227 us)
+          rc = launch_nvfp4_group_panel<4, 5, 2, OUT_BF16>(p, 33, 80, stream);
+          if (rc != NVF_OK) return rc;
+          mid.rows_lo = 81;
+        }
         rc = launch_nvfp4_fast<OUT_BF16, true, 2>(mid, cus, stream);
       } else if (p.k < 4096 && (p.n & 255) == 0) {
         rc = launch_nvfp4_skinny_grouped<2, 8, OUT_BF16, true>(p, 33, 128, stream);

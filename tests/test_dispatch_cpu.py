@@ -58,15 +58,11 @@ def test_config5_nvfp4_grouped(n, k):
     got = plan("nvfp4_scaled_grouped_mm", 65536, n, k, groups=256)
     kernels = [g.split(" ")[0] for g in got.split("; ")]
     assert any(kk.startswith("nvfp4_gemm_256_kernel<grouped=1,TM=4") for kk in kernels), got  # the 256-row tiles of the large experts
-    # the mid-sized experts: with the deep K the kernel that converts their rows once per 512 weight rows (33-80 rows)
-    # and 128x256 tiles of the persistent kernel (81-128 rows and the ends of the large experts: no tile kernel);
-    # with the shallow K those tiles for all of them
-    if k >= 4096:
-        assert "nvfp4_group_panel_kernel<RT=4,TT=5,slots=2>" in got and "rows=33..80" in got, got
-        assert any(kk.startswith("nvfp4_gemm_256_kernel<grouped=1,TM=2") for kk in kernels) and "rows=81..128 min_rows=129" in got, got
-        assert "nvfp4_tile_kernel" not in got, got
-    else:
-        assert any(kk.startswith("nvfp4_gemm_256_kernel<grouped=1,TM=2") for kk in kernels) and "panel" not in got, got
+    # the mid-sized experts: the kernel that converts their rows once per 512 weight rows (33-80 rows) and 128x256
+    # tiles of the persistent kernel (81-128 rows and the ends of the large experts: no tile kernel)
+    assert "nvfp4_group_panel_kernel<RT=4,TT=5,slots=2>" in got and "rows=33..80" in got, got
+    assert any(kk.startswith("nvfp4_gemm_256_kernel<grouped=1,TM=2") for kk in kernels) and "rows=81..128 min_rows=129" in got, got
+    assert "nvfp4_tile_kernel" not in got, got
 
 
 def test_dry_run_reports_argument_errors_and_touches_no_device():

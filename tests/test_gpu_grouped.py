@@ -303,14 +303,15 @@ def test_nvfp4_grouped_mm_small_groups_stream_their_weights(dev, n, k):
         assert torch.equal(out[:rows], nvf_cutlass.nvfp4_scaled_grouped_mm(*args, dtype)[:rows])
 
 
-@pytest.mark.parametrize("n,k", [(512, 4096), (1024, 4224)])
+@pytest.mark.parametrize("n,k", [(512, 4096), (1024, 4224), (512, 2048), (1024, 1024), (512, 1152)])
 def test_nvfp4_grouped_mm_mid_sized_groups_of_a_prefill(dev, n, k):
-    """A prefill-sized call (2048 rows or more) with K >= 4096 and N % 512 == 0: groups of 33..80 rows run on the kernel
+    """A prefill-sized call (2048 rows or more) with K >= 1024 and N % 512 == 0: groups of 33..80 rows run on the kernel
     that converts a group's activation rows once per 512 weight rows (work items found from the device-resident
     sizes; three, four and five row tiles, sizes on both sides of its borders), their neighbours of 81..128 rows and
-    the ends of the larger ones on 128x256 tiles of the persistent kernel, the rest of those on its 256x256 tiles.  33 K chunks: the odd and the even LDS slot both end a
-    walk.  A different alpha per group, poisoned padding of the activation scale slabs; every element compared, rows
-    after the last group untouched, run-to-run bit equality."""
+    the ends of the larger ones on 128x256 tiles of the persistent kernel, the rest of those on its 256x256 tiles.  8, 9,
+    16, 32 and 33 K chunks: the odd and the even LDS slot both end a walk.  A different alpha per group, poisoned
+    padding of the activation scale slabs; every element compared, rows after the last group untouched, run-to-run
+    bit equality."""
     from fuser_amd import capi, nvf_cutlass
 
     sizes = [33, 80, 48, 49, 64, 65, 81, 32, 0, 128, 34, 47, 79, 300, 66, 50, 40, 72, 1, 129] + [56, 77, 35, 63] * 6
