@@ -180,9 +180,10 @@ int nvf_cast_f32_to_e2m1(const float* in, int64_t n, uint8_t* out, void* stream)
 int nvf_cast_f32_to_e4m3(const float* in, int64_t n, uint8_t* out, void* stream) { return cast_common(1, in, n, out, stream); }
 int nvf_cast_f32_to_e8m0(const float* in, int64_t n, uint8_t* out, void* stream) { return cast_common(2, in, n, out, stream); }
 
-int nvf_nvfp4_scaled_mm_ws(const void* a, const void* b, const void* scales_a, const void* scales_b, const float* alpha,
-                           void* out, int64_t m, int64_t n, int64_t k, int out_dtype, void* workspace,
-                           int64_t workspace_bytes, void* stream) {
+// argument checks of nvfp4_scaled_mm shared by its three entry points; *empty is set for a call without output
+static int check_nvfp4_scaled_mm(const void* a, const void* b, const void* scales_a, const void* scales_b, const float* alpha, void* out,
+                                 int64_t m, int64_t n, int64_t k, int out_dtype, int64_t workspace_bytes, bool* empty) {
+  *empty = true;
   NVF_REQUIRE(dtype16(out_dtype), NVF_ERR_INVALID_ARGUMENT, "output dtype must be bf16 or f16, got %d", out_dtype);
   NVF_REQUIRE(m >= 0 && n >= 0 && k >= 0, NVF_ERR_INVALID_ARGUMENT, "negative size");
   NVF_REQUIRE(k % 32 == 0, NVF_ERR_UNSUPPORTED_SHAPE, "The K dimension %lld is not divisible by 32", (long long)k);
@@ -191,6 +192,16 @@ int nvf_nvfp4_scaled_mm_ws(const void* a, const void* b, const void* scales_a, c
   if (m == 0 || n == 0) return NVF_OK;
   NVF_REQUIRE(a && b && scales_a && scales_b && alpha && out, NVF_ERR_INVALID_ARGUMENT, "NULL buffer");
   NVF_REQUIRE_ALIGNED16(a, b, scales_a, scales_b, out);
+  *empty = false;
+  return NVF_OK;
+}
+
+int nvf_nvfp4_scaled_mm_ws(const void* a, const void* b, const void* scales_a, const void* scales_b, const float* alpha,
+                           void* out, int64_t m, int64_t n, int64_t k, int out_dtype, void* workspace,
+                           int64_t workspace_bytes, void* stream) {
+  bool empty;
+  if (const int rc = check_nvfp4_scaled_mm(a, b, scales_a, scales_b, alpha, out, m, n, k, out_dtype, workspace_bytes, &empty)) return rc;
+  if (empty) return NVF_OK;
   Gemm16Args g{a, b, scales_a, scales_b, alpha, out, nullptr, nullptr, nullptr, 1, m, n, k, out_dtype};
   if (workspace != nullptr && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0) {  // fp32x4 accesses
     g.workspace = workspace;
@@ -208,13 +219,17 @@ int64_t nvf_nvfp4_scaled_mm_workspace_bytes(int64_t m, int64_t n, int64_t k) { r
 
 int nvf_nvfp4_scaled_mm_static_ws(const void* a, const void* b, const void* scales_a, const void* scales_b, const float* alpha,
                                   void* out, int64_t m, int64_t n, int64_t k, int out_dtype, void* stream) {
+  // the arguments first: an invalid call must not touch the device
+  bool empty;
+  if (const int rc = check_nvfp4_scaled_mm(a, b, scales_a, scales_b, alpha, out, m, n, k, out_dtype, 0, &empty)) return rc;
+  if (empty) return NVF_OK;
   const int64_t need = nvfp4_gemm_workspace_bytes(m, n, k);
   NVF_REQUIRE(need <= kStaticScratchBytes, NVF_ERR_UNSUPPORTED_SHAPE,
               "M = %lld, N = %lld, K = %lld needs %lld bytes of scratch memory, the library's static scratch holds %lld: use "
               "nvf_nvfp4_scaled_mm_ws with a workspace of the caller's, or nvf_nvfp4_scaled_mm",
               (long long)m, (long long)n, (long long)k, (long long)need, (long long)kStaticScratchBytes);
   void* ws = nullptr;
-  if (need > 0 && m > 0 && n > 0) {
+  if (need > 0) {
     if (const int rc = static_scratch(&ws)) return rc;
   }
   return nvf_nvfp4_scaled_mm_ws(a, b, scales_a, scales_b, alpha, out, m, n, k, out_dtype, ws, ws ? need : 0, stream);
@@ -299,7 +314,7 @@ int nvf_describe_dispatch(const char* op, int64_t m, int64_t n, int64_t k, int g
   int rc;
   const std::string name(op);
   if (name == "nvfp4_scaled_mm") rc = nvf_nvfp4_scaled_mm_ws(x, x, x, x, f, x, m, n, k, dtype, workspace_bytes > 0 ? x : nullptr, workspace_bytes, nullptr);
-  else if (name == "nvfp4_scaled_mm_blockscale") rc = nvf_nvfp4_scaled_mm_blockscale(x, x, x, x, f, f, x, x, static_cast<float*>(x), m, n, k, nullptr);
+  else if (name == "nvfp4_scaled_mm_blockscale") rc = nvf_nvfp4_scaled_mm_blockscale(x, x, x, x, f, f, x, x, workspace_bytes > 0 ? static_cast<float*>(x) : nullptr, m, n, k, nullptr);
   else if (name == "mxfp8_scaled_mm") rc = nvf_mxfp8_scaled_mm(x, x, x, x, f, x, m, n, k, dtype, nullptr);
   else if (name == "grouped_mm") rc = nvf_grouped_mm(x, x, x, i, i, groups, m, n, k, dtype, nullptr);
   else if (name == "nvfp4_scaled_grouped_mm") rc = nvf_nvfp4_scaled_grouped_mm(x, x, x, x, f, x, i, i, i, groups, m, n, k, dtype, nullptr);

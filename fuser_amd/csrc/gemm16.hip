@@ -1097,6 +1097,7 @@ int launch_nvfp4_fast_cfg(const Params& p, int cus, hipStream_t stream) {
   const int64_t tiles_m = (GROUPED && TM == 2) ? std::min<int64_t>(p.groups, p.m / std::max(p.rows_lo, 1)) : p.m / (64 * TM);
   const int64_t tiles = tiles_m * (p.n / 256);
   const unsigned grid = (unsigned)(tiles >= cus ? (cus & ~7) : ((tiles + 7) / 8) * 8);
+  if (grid == 0) return NVF_OK;  // fewer rows in the whole call than the smallest group this launch serves: no work
   if (note_launch("nvfp4_gemm_256_kernel<grouped=%d,TM=%d,f32=%d,pairs=%d%s> grid=%u rows=%d..%d min_rows=%d", (int)GROUPED, TM, (int)OUT_F32,
                   (int)PAIRS, OUT_FP4 ? ",fp4_blockscale" : "", grid, p.rows_lo, p.rows_hi, p.min_rows))
     return NVF_OK;
@@ -1955,9 +1956,9 @@ int launch_nvfp4_group_panel(const Params& p0, int rows_lo, int rows_hi, hipStre
   Params p = p0;
   p.rows_lo = rows_lo;
   p.rows_hi = rows_hi;
-  // an upper bound of the items: the groups of the row range have at least rows_lo rows each
-  const int64_t groups_max = std::min<int64_t>(p.groups, p.m / std::max(rows_lo, 1));
-  const int64_t wgs = groups_max * (p.n / (128 * RT));
+  // one workgroup per (group, block) of all groups: the group sizes live on the device and need not add up to the
+  // rows of `a`, so no tighter bound is safe; workgroups past the last item return right after the prefix scan
+  const int64_t wgs = (p.m < rows_lo ? 0 : (int64_t)p.groups) * (p.n / (128 * RT));
   if (wgs >= ((int64_t)1 << 31)) return fail(NVF_ERR_UNSUPPORTED_SHAPE, "too many (group, row block) pairs for one launch");
   if (note_launch("nvfp4_group_panel_kernel<RT=%d,TT=%d,slots=%d> grid=%lld rows=%d..%d", RT, TT, BSLOTS, (long long)wgs, rows_lo, rows_hi))
     return NVF_OK;

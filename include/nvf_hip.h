@@ -153,7 +153,9 @@ NVF_API int nvf_nvfp4_scaled_mm_ws(const void* a, const void* b, const void* sca
  * Results are bit-identical to nvf_nvfp4_scaled_mm_ws with a workspace of nvf_nvfp4_scaled_mm_workspace_bytes.
  * A shape whose split needs more than NVF_STATIC_SCRATCH_BYTES is rejected with NVF_ERR_UNSUPPORTED_SHAPE.
  * Every call on a device shares that device's array: calls that may overlap in time on one device (different
- * streams or threads) race on it and must be serialised by the caller. */
+ * streams or threads) race on it and must be serialised by the caller.
+ * The first call on a device looks up the array's address and sets kernel attributes (a mutex, hipGetSymbolAddress,
+ * hipFuncSetAttribute): make it outside any stream capture; every later call only launches kernels. */
 #define NVF_STATIC_SCRATCH_BYTES (32ll << 20)
 NVF_API int nvf_nvfp4_scaled_mm_static_ws(const void* a, const void* b, const void* scales_a, const void* scales_b,
                                           const float* alpha, void* out, int64_t m, int64_t n, int64_t k,

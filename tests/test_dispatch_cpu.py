@@ -70,3 +70,53 @@ def test_dry_run_reports_argument_errors_and_touches_no_device():
     assert capi.lib().nvf_describe_dispatch(b"mxfp8_scaled_mm", 128, 128, 40, 1, BF16, 0, buf, 64) == -2
     assert capi.lib().nvf_describe_dispatch(b"no_such_op", 128, 128, 64, 1, BF16, 0, buf, 64) == -1
     assert capi.lib().nvf_describe_dispatch(b"mxfp8_scaled_mm", 128, 128, 64, 1, BF16, 0, None, 64) == -1
+
+
+@pytest.mark.parametrize("m", [1, 8, 32])
+@pytest.mark.parametrize("n,k", [(2048, 7168), (7168, 2048), (256, 256), (512, 4096)])
+def test_grouped_nvfp4_with_few_rows_in_all_launches_no_empty_grid(m, n, k):
+    # a decode step of a few tokens x top-8: fewer rows in the whole call than the smallest group some launches serve
+    got = plan("nvfp4_scaled_grouped_mm", m, n, k, groups=8)
+    assert got and "grid=0" not in got, got
+
+
+def test_blockscale_is_one_launch_and_ragged_shapes_add_only_the_fill_kernel():
+    got = plan("nvfp4_scaled_mm_blockscale", 8192, 8192, 8192)
+    assert got.startswith("nvfp4_gemm_256_kernel<") and "fp4_blockscale" in got and ";" not in got, got
+    ragged = plan("nvfp4_scaled_mm_blockscale", 200, 160, 512).split("; ")
+    assert len(ragged) == 2 and ragged[0].startswith("zero_fill_kernel") and ragged[1].startswith("nvfp4_tile_kernel<"), ragged
+    # the optional dump of the fp32 product is a second run of the same kernel
+    dump = plan("nvfp4_scaled_mm_blockscale", 8192, 8192, 8192, ws=4 * 8192 * 8192).split("; ")
+    assert len(dump) == 2 and "fp4_blockscale" in dump[0] and "f32=1" in dump[1], dump
+
+
+KNOWN_KERNELS = ("nvfp4_skinny_ring_kernel<", "nvfp4_gemm_256_kernel<", "nvfp4_tile_kernel<", "nvfp4_group_panel_kernel<",
+                 "gemm16_kernel<", "grouped16_gemm_256_kernel<", "mxfp8_gemm_256_kernel<", "mxfp8_skinny_kernel<", "mxfp8_gemm_kernel<",
+                 "zero_fill_kernel", "nvfp4_act_convert_kernel", "nvfp4_skinny_f16a_kernel<", "splitk_reduce_kernel")
+
+
+def _assert_known(got):
+    assert got, "empty plan"
+    assert "grid=0" not in got, got
+    for part in got.split("; "):
+        assert any(k in part for k in KNOWN_KERNELS), got
+
+
+def test_sweep_of_other_shapes_reaches_a_kernel_on_every_branch():
+    """Shapes off the benchmark's list: the dry run must return NVF_OK and name known kernels with non-empty grids,
+    whatever the tuning constants of the dispatch are (catches dead or broken branches after a constant changes)."""
+    ms = [1, 16, 17, 48, 100, 128, 129, 256, 300, 512, 1000, 2048, 4096, 8192]
+    nks = [(32, 32), (64, 128), (128, 512), (256, 256), (512, 1024), (1024, 8192), (1536, 7168), (2048, 2048), (3072, 2048),
+           (4096, 4096), (4128, 4096), (6144, 512), (7168, 2048), (14336, 4096), (28672, 4096), (4096, 14336), (256, 16384)]
+    for m in ms:
+        for n, k in nks:
+            for ws in (0, 64 << 20):
+                _assert_known(plan("nvfp4_scaled_mm", m, n, k, ws=ws))
+            _assert_known(plan("nvfp4_scaled_mm_blockscale", m, n, k))
+            _assert_known(plan("mxfp8_scaled_mm", m, n, k))
+            _assert_known(plan("mxfp8_scaled_mm", m, n, k, dtype=F16))
+            _assert_known(plan("grouped_mm", m, n, k, groups=1))
+            for groups in (3, 8, 64, 256):
+                _assert_known(plan("grouped_mm", m, n, k, groups=groups))
+                if n % 128 == 0 and k % 64 == 0:
+                    _assert_known(plan("nvfp4_scaled_grouped_mm", m, n, k, groups=groups))

@@ -13,7 +13,7 @@ pytestmark = pytest.mark.gpu
 
 
 def test_chain_replays_bit_exactly(dev):
-    from fuser_amd import nvf_cutlass, ops
+    from fuser_amd import capi, nvf_cutlass, ops
 
     gen = torch.Generator(device=dev).manual_seed(5)
     m, n, k = 512, 1024, 512
@@ -42,6 +42,12 @@ def test_chain_replays_bit_exactly(dev):
         dq, dsf = ops.nv_block_quantize(xd, None, True, 16)
         wdq, wdsf = ops.nv_block_quantize(wd, None, True, 16)
         split = nvf_cutlass.nvfp4_scaled_mm(dq, wdq, dsf, wdsf, one, torch.float16)
+        # the same split with the library's static scratch array (the entry point for callers that cannot allocate;
+        # its first call per device, which looks the array's address up, is the eager run below, outside the capture)
+        static = torch.empty_like(split)
+        capi.check(capi.lib().nvf_nvfp4_scaled_mm_static_ws(dq.data_ptr(), wdq.data_ptr(), dsf.data_ptr(), wdsf.data_ptr(), one.data_ptr(),
+                                                            static.data_ptr(), 128, 256, 8192, capi.F16,
+                                                            torch.cuda.current_stream().cuda_stream))
         gq, gsf = ops.nv_grouped_block_quantize(x, eo, so, None, 16)
         wgq = torch.stack([ops.nv_block_quantize(wg[e], None, True, 16)[0].view(torch.uint8) for e in range(len(sizes))])
         wgs = torch.stack([ops.nv_block_quantize(wg[e], None, True, 16)[1].view(torch.uint8) for e in range(len(sizes))])
@@ -56,10 +62,11 @@ def test_chain_replays_bit_exactly(dev):
         bq, bsf = nvf_cutlass.nvfp4_scaled_mm_blockscale(xq, wq, xsf, wsf, one, one)
         rq, rsf = nvf_cutlass.nvfp4_scaled_mm_blockscale(xq[:200].contiguous(), wq[:160].contiguous(), xsf[:256].contiguous(),
                                                          wsf[:256].contiguous(), one, one)
-        return [gs, dense, decode, split, grouped[: sum(sizes)], bf[: sum(sizes)], mx, bq.view(torch.uint8), bsf.view(torch.uint8),
+        return [gs, dense, decode, split, static, grouped[: sum(sizes)], bf[: sum(sizes)], mx, bq.view(torch.uint8), bsf.view(torch.uint8),
                 rq.view(torch.uint8), rsf.view(torch.uint8)]
 
     eager = [t.clone() for t in chain()]  # also the warm-up: function attributes are set outside the capture
+    assert capi.lib().nvf_nvfp4_scaled_mm_workspace_bytes(128, 256, 8192) > 0 and torch.equal(eager[3], eager[4])
     torch.cuda.synchronize()
     side = torch.cuda.Stream()
     with torch.cuda.stream(side):

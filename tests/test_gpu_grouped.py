@@ -4,7 +4,7 @@ test_cutlass_nvfp4_gemm.py:178-281 verbatim, then BASELINE configs 4 and 5."""
 import pytest
 import torch
 
-from helpers import GEMM_MAX_REL, e4m3, fp4, gs_of, max_rel, start_offsets
+from helpers import GEMM_MAX_REL, e4m3, fp4, gs_of, max_rel, max_rel_rowwise, start_offsets
 from oracle import nvf_oracle as O
 
 pytestmark = pytest.mark.gpu
@@ -39,6 +39,7 @@ def test_grouped_mm_reference_configs(dev, config, tokens_per_expert_neg_one, te
     ref = O.ref_grouped_mm(mat1, mat2, ps, eo)
     assert not ref.isnan().any()
     assert max_rel(out, ref) <= GEMM_MAX_REL
+    assert max_rel_rowwise(out, ref) <= GEMM_MAX_REL
     torch.testing.assert_close(out.float().cpu(), ref.to(tensor_dtype).float(), atol=1e-2 * ref.abs().max().item(), rtol=1e-2)
 
 
@@ -58,7 +59,7 @@ def test_grouped_mm_empty_groups_and_untouched_rows(dev):
     torch.cuda.synchronize()
     ref = O.ref_grouped_mm(a, b, ps, eo)
     assert ref[200:].isnan().all() and (out[200:] == 7.0).all()
-    assert max_rel(out[:200], ref[:200]) <= GEMM_MAX_REL
+    assert max_rel_rowwise(out[:200], ref[:200]) <= GEMM_MAX_REL
 
 
 @pytest.mark.parametrize("tensor_dtype,k,n", [(torch.bfloat16, 192, 2048), (torch.float16, 128, 2048), (torch.bfloat16, 1088, 2048),
@@ -122,14 +123,19 @@ def _moe_sizes_top2(tokens, experts, seed):
     return torch.bincount(logits.topk(2, dim=1).indices.flatten(), minlength=experts).tolist()
 
 
-def test_config4_bf16_grouped_moe(dev):
-    """BASELINE config 4: 8 experts, K=4096, N=14336, 4096 tokens top-2 (8192 rows), uneven groups."""
+@pytest.mark.parametrize("near_empty", [False, True])
+def test_config4_bf16_grouped_moe(dev, near_empty):
+    """BASELINE config 4: 8 experts, K=4096, N=14336, 4096 tokens top-2 (8192 rows), uneven groups: exactly the
+    group sizes bench.py times ([40, 90, 220, 427, 872, 1413, 2211, 2919]), and the same with one expert
+    emptied down to 3 rows."""
     from fuser_amd import nvf_cutlass
 
     g, k, n = 8, 4096, 14336
     sizes = _moe_sizes_top2(4096, g, seed=0)
-    sizes[3] += sizes[5] - 3
-    sizes[5] = 3  # a near-empty expert
+    assert sizes == [40, 90, 220, 427, 872, 1413, 2211, 2919]
+    if near_empty:
+        sizes[3] += sizes[5] - 3
+        sizes[5] = 3
     m = sum(sizes)
     assert m == 8192
     gen = torch.Generator(device=dev).manual_seed(1)
@@ -138,15 +144,17 @@ def test_config4_bf16_grouped_moe(dev):
     ps, eo, st, ct = _grouped_args(sizes, n, k, dev)
     out = nvf_cutlass.grouped_mm(a, b, st, ct, ps.to(dev), eo.to(dev))
     torch.cuda.synchronize()
-    # oracle on a sample of rows (every expert, first/last row of each) and of columns
-    cols = torch.randint(0, n, (256,), generator=torch.Generator().manual_seed(2))
+    # oracle on a sample of rows (every expert: first and last row, the rows either side of every 128-row border, random
+    # ones) and of columns (first, last, random)
+    cols = torch.unique(torch.cat([torch.tensor([0, n - 1]), torch.randint(0, n, (254,), generator=torch.Generator().manual_seed(2))]))
     worst = 0.0
     for e in range(g):
         lo, hi = int(eo[e]), int(eo[e]) + sizes[e]
-        rows = torch.unique(torch.cat([torch.tensor([lo, hi - 1]), torch.randint(lo, hi, (24,), generator=torch.Generator().manual_seed(e))]))
+        borders = torch.tensor([r for b128 in range(128, sizes[e], 128) for r in (lo + b128 - 1, lo + b128)], dtype=torch.long)
+        rows = torch.unique(torch.cat([torch.tensor([lo, hi - 1]), borders, torch.randint(lo, hi, (24,), generator=torch.Generator().manual_seed(e))]))
         ref = a[rows.to(dev)].float().cpu() @ b[e][cols.to(dev)].float().cpu().t()
         got = out[rows.to(dev)][:, cols.to(dev)]
-        worst = max(worst, max_rel(got, ref))
+        worst = max(worst, max_rel_rowwise(got, ref))
     assert worst <= GEMM_MAX_REL
 
 
@@ -183,6 +191,7 @@ def test_nvfp4_grouped_mm_reference_config(dev, config, tokens_per_expert_neg_on
     assert out.dtype == out_dtype and out.shape == (m, n)
     ref = O.ref_nvfp4_scaled_grouped_mm(raq, bq, rasf, bsf, alphas, ps, eo, so)
     assert max_rel(out, ref) <= GEMM_MAX_REL
+    assert max_rel_rowwise(out, ref) <= GEMM_MAX_REL
     torch.testing.assert_close(out.float().cpu(), ref, atol=1e-2 * ref.abs().max().item(), rtol=1e-2)
 
 
@@ -209,7 +218,38 @@ def test_nvfp4_grouped_mm_empty_and_tiny_groups(dev):
     out = nvf_cutlass.nvfp4_scaled_grouped_mm(fp4(aq.to(dev)), fp4(bq.to(dev)), e4m3(asf.to(dev)), e4m3(bsf.to(dev)), alphas.to(dev), st, ct,
                                               ps.to(dev), eo.to(dev), so.to(dev), torch.bfloat16)
     torch.cuda.synchronize()
-    assert max_rel(out, ref) <= GEMM_MAX_REL
+    assert max_rel_rowwise(out, ref) <= GEMM_MAX_REL
+
+
+@pytest.mark.parametrize("m_total,n,k", [(1, 256, 256), (8, 2048, 7168), (32, 7168, 2048), (31, 384, 4096), (20, 512, 1024)])
+def test_nvfp4_grouped_mm_fewer_rows_in_all_than_the_smallest_mid_sized_group(dev, m_total, n, k):
+    """A decode step of a few tokens: at most 32 rows in the whole call, so the launches that serve groups of 33 rows and
+    more have nothing to do (and must not be launched with an empty grid).  Every element compared."""
+    from fuser_amd import capi, nvf_cutlass
+
+    g = 8
+    gen = torch.Generator().manual_seed(m_total + n)
+    cuts = sorted(torch.randint(0, m_total + 1, (g - 1,), generator=gen).tolist())
+    sizes = [b - a for a, b in zip([0] + cuts, cuts + [m_total])]
+    assert sum(sizes) == m_total
+    assert "grid=0" not in capi.describe_dispatch("nvfp4_scaled_grouped_mm", m_total, n, k, groups=g)
+    x = torch.randn(m_total, k, generator=gen).bfloat16()
+    w = (torch.randn(g, n, k, generator=gen) * 0.05).bfloat16()
+    ps, eo, st, ct = _grouped_args(sizes, n, k, dev)
+    so = start_offsets([O.round_up(t, 128) for t in sizes])
+    aq, asf = O.grouped_block_quantize_nvfp4(x, eo, so, None)
+    bq = torch.empty(g, n, k // 2, dtype=torch.uint8)
+    bsf = torch.empty(g, n, k // 16, dtype=torch.uint8)
+    alphas = torch.empty(g)
+    for e in range(g):
+        gs = gs_of(w[e])
+        bq[e], bsf[e] = O.block_quantize_nvfp4(w[e], gs, True)
+        alphas[e] = (e + 1) / gs
+    ref = O.ref_nvfp4_scaled_grouped_mm(aq, bq, asf, bsf, alphas, ps, eo, so)
+    out = nvf_cutlass.nvfp4_scaled_grouped_mm(fp4(aq.to(dev)), fp4(bq.to(dev)), e4m3(asf.to(dev)), e4m3(bsf.to(dev)), alphas.to(dev), st, ct,
+                                              ps.to(dev), eo.to(dev), so.to(dev), torch.bfloat16)
+    torch.cuda.synchronize()
+    assert max_rel_rowwise(out[:m_total], ref[:m_total]) <= GEMM_MAX_REL
 
 
 @pytest.mark.parametrize("sizes,n,k", [([600, 0, 256, 255, 1, 1030, 512], 512, 384), ([300, 2100, 0, 257], 256, 256),
@@ -383,24 +423,32 @@ def test_config5_nvfp4_grouped_large_moe(dev, kn):
         bq[e], bsf[e], alphas[e] = q.view(torch.uint8), s.view(torch.uint8), 1.0 / gs
     out = nvf_cutlass.nvfp4_scaled_grouped_mm(aq, fp4(bq), asf, e4m3(bsf), alphas, st, ct, ps.to(dev), eo.to(dev), so.to(dev), torch.bfloat16)
     torch.cuda.synchronize()
-    order = sorted(range(g), key=lambda e: sizes[e])
-    picked = order[:3] + order[g // 2 : g // 2 + 2] + order[-2:]
-    cols = torch.randint(0, n, (128,), generator=torch.Generator().manual_seed(6))
+    # two experts of every class of the dispatch (they run on different kernels): 1-32 rows, 33-80, 81-128, 129-255, and
+    # 256 and more with a last partial tile of at most 128 rows / of more than 128 rows (or none); plus the largest
+    classes = {"1-32": lambda t: 1 <= t <= 32, "33-80": lambda t: 33 <= t <= 80, "81-128": lambda t: 81 <= t <= 128,
+               "129-255": lambda t: 129 <= t <= 255, "256+, short end": lambda t: t >= 256 and 1 <= t % 256 <= 128,
+               "256+, long end": lambda t: t >= 256 and (t % 256 == 0 or t % 256 > 128)}
+    picked = [max(range(g), key=lambda e: sizes[e])]
+    for name, member in classes.items():
+        of_class = [e for e in range(g) if member(sizes[e])]
+        assert len(of_class) >= 2, name
+        picked += [of_class[0], of_class[-1]]
+    cols = torch.unique(torch.cat([torch.tensor([0, n - 1]), torch.randint(0, n, (126,), generator=torch.Generator().manual_seed(6))]))
     worst = 0.0
     aq8, asf8 = aq.view(torch.uint8), asf.view(torch.uint8)
     for e in picked:
         t = sizes[e]
-        if t == 0:
-            continue
         lo, slo = int(eo[e]), int(so[e])
-        local = torch.unique(torch.cat([torch.tensor([0, t - 1]), torch.randint(0, t, (14,), generator=torch.Generator().manual_seed(e))]))
+        # first and last row, the rows either side of the last 256-row and 128-row borders, random ones: 32 at most
+        edge = [0, t - 1] + [r for b in ((t - 1) // 256 * 256, (t - 1) // 128 * 128) for r in (b - 1, b) if 0 <= r < t]
+        local = torch.unique(torch.cat([torch.tensor(edge), torch.randint(0, t, (26,), generator=torch.Generator().manual_seed(e))]))
         a_rows = aq8[(lo + local).to(dev)].cpu()
         sf_lin = O.swizzled_to_linear_128_4(asf8[slo : slo + O.round_up(t, 128)].cpu(), t, k // 16)[local]
         b_rows = bq[e][cols.to(dev)].cpu()
         sb_lin = O.swizzled_to_linear_128_4(bsf[e].cpu(), n, k // 16)[cols]
         ref = O.ref_nvfp4_scaled_mm(a_rows, b_rows, O.linear_to_swizzled_128_4(sf_lin), O.linear_to_swizzled_128_4(sb_lin), float(alphas[e]))
         got = out[(lo + local).to(dev)][:, cols.to(dev)]
-        worst = max(worst, max_rel(got, ref))
+        worst = max(worst, max_rel_rowwise(got, ref))
     assert worst <= GEMM_MAX_REL
 
 
