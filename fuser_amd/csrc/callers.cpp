@@ -1,5 +1,7 @@
 #include "callers.h"
 
+#include "nvf_checks.h"
+
 namespace nvfuser {
 namespace callers {
 
@@ -23,7 +25,7 @@ torch::Tensor scaled_mma(const torch::Tensor& mat1, const torch::Tensor& mat2, c
 }
 
 GroupedMmaArguments grouped_mma_arguments(const torch::Tensor& offsets, int64_t n, int64_t k) {
-  if (offsets.dim() != 1) throw nvfError("grouped_mma_arguments: offsets must be a 1D tensor of group end rows");
+  NVF_CHECK(offsets.dim() == 1, "grouped_mma_arguments: offsets must be a 1D tensor of group end rows");
   const auto i32 = offsets.options().dtype(at::kInt);
   const auto i64 = offsets.options().dtype(at::kLong);
   const int64_t groups = offsets.size(0);
@@ -54,12 +56,10 @@ torch::Tensor cutlass_nvfp4_grouped_mma(const torch::Tensor& mat1, const torch::
                                         const torch::Tensor& scale2, const torch::Tensor& alpha,
                                         const torch::Tensor& problem_sizes, const torch::Tensor& expert_offsets,
                                         const torch::Tensor& sf_offsets, at::ScalarType out_dtype) {
-  if (mat1.scalar_type() != at::ScalarType::Float4_e2m1fn_x2 || mat2.scalar_type() != at::ScalarType::Float4_e2m1fn_x2)
-    throw nvfError("Expected mat1.scalar_type() == Float4_e2m1fn_x2 && mat2.scalar_type() == Float4_e2m1fn_x2 . ");
-  if (problem_sizes.dim() != 2) throw nvfError("Expected problem_sizes.dim() == 2 . problem_sizes must be a 2D tensor");
-  if (problem_sizes.size(1) != 3)
-    throw nvfError("Expected problem_sizes.size(1) == 3 . problem_sizes must have shape (num_experts, 3)");
-  if (mat1.dim() != 2 || mat2.dim() != 3) throw nvfError("cutlass_nvfp4_grouped_mma: mat1 must be 2D and mat2 3D");
+  NVF_CHECK(mat1.scalar_type() == at::ScalarType::Float4_e2m1fn_x2 && mat2.scalar_type() == at::ScalarType::Float4_e2m1fn_x2);
+  NVF_CHECK(problem_sizes.dim() == 2, "problem_sizes must be a 2D tensor");
+  NVF_CHECK(problem_sizes.size(1) == 3, "problem_sizes must have shape (num_experts, 3)");
+  NVF_CHECK(mat1.dim() == 2 && mat2.dim() == 3, "cutlass_nvfp4_grouped_mma: mat1 must be 2D and mat2 3D");
   const int64_t groups = problem_sizes.size(0);
   const int64_t k = mat1.size(1) * 2;  // mat1 is packed, two values per byte
   const int64_t n = mat2.size(2);

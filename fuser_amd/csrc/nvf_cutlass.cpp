@@ -5,31 +5,11 @@
 #include <c10/core/DeviceGuard.h>
 #include <c10/hip/HIPStream.h>
 
-#include <sstream>
-
+#include "nvf_checks.h"
 #include "nvf_hip.h"
 
 namespace nvfuser {
 namespace {
-
-template <typename... Args>
-std::string concat(const Args&... args) {
-  std::ostringstream os;
-  (void)std::initializer_list<int>{((os << args), 0)...};
-  return os.str();
-}
-
-// Same message shape as NVF_CHECK (csrc/exceptions.h:200-245): "Expected <cond> . <message>".
-#define NVF_CHECK(cond, ...)                                                        \
-  do {                                                                              \
-    if (!(cond)) throw ::nvfuser::nvfError(concat("Expected " #cond " . ", ##__VA_ARGS__)); \
-  } while (0)
-#define NVF_CHECK_EQ(lhs, rhs, ...)                                                                            \
-  do {                                                                                                         \
-    if (!((lhs) == (rhs)))                                                                                     \
-      throw ::nvfuser::nvfError(concat("Expected " #lhs " == " #rhs " . Found ", (lhs), " vs ", (rhs), ". ", ##__VA_ARGS__)); \
-  } while (0)
-#define NVF_THROW(...) throw ::nvfuser::nvfError(concat(__VA_ARGS__))
 
 void* current_stream(const torch::Tensor& t) {
   return static_cast<void*>(c10::hip::getCurrentHIPStream(t.device().index()).stream());

@@ -13,17 +13,31 @@
 
 #define NVF_HOST_API __attribute__((visibility("default")))
 
+// Built inside the reference's tree (its csrc/ on the include path), the failed checks throw the reference's own
+// nvfuser::nvfError through its own NVF_CHECK / NVF_THROW (csrc/exceptions.h:136-245), so that the program holds one
+// definition of the class and catch sites may use msg(), context(), what_without_backtrace().  Built on its own,
+// a stand-in with the same name, base class and what() takes its place.
+#if defined(__has_include)
+#if __has_include(<exceptions.h>) && __has_include(<visibility.h>)
+#include <exceptions.h>
+#define NVF_HIP_REFERENCE_EXCEPTIONS 1
+#endif
+#endif
+
 namespace nvfuser {
 
-// Counterpart of nvfuser::nvfError (csrc/exceptions.h:136-245): what every failed check throws.
+#ifndef NVF_HIP_REFERENCE_EXCEPTIONS
 class NVF_HOST_API nvfError : public std::exception {
  public:
   explicit nvfError(std::string msg) : msg_(std::move(msg)) {}
   const char* what() const noexcept override { return msg_.c_str(); }
+  const std::string& msg() const { return msg_; }
+  const char* what_without_backtrace() const noexcept { return msg_.c_str(); }
 
  private:
   std::string msg_;
 };
+#endif
 
 namespace cutlass_kernels {
 
