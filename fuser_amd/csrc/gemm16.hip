@@ -1180,8 +1180,14 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, g = lane >> 4;
   const int kbytes = p.k >> 1;
-  const int chunks = p.k >> 7;
+  int chunks = p.k >> 7;
   const int sf_padded = p.k >> 4;  // K % 128 == 0: no padding columns
+  // dense with a workspace: blockIdx.z owns the chunks [c_lo, c_lo + chunks) of K and leaves an fp32 partial result
+  int c_lo = 0;
+  if (!GROUPED && p.partial != nullptr) {
+    c_lo = (int)blockIdx.z * p.spans_per_split;
+    chunks = min(chunks - c_lo, p.spans_per_split);
+  }
   int n0, m_loc, grp = 0, asf_word0 = 0;  // asf_word0: which 32-row group of its 128-row scale tile the slab starts in
   int64_t a_row0 = p.m_base, asf_row0 = p.m_base, b_row0 = 0;  // first activation row, its scale row, first weight row
   if constexpr (GROUPED) {
@@ -1207,10 +1213,10 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
 
   // ---- load side (memory order): lane L fetches row L/4, piece (L%4) ^ ((L/16)&3) of a payload tile
   const int lrow = lane >> 2, lpiece = (lane & 3) ^ ((lane >> 4) & 3);
-  const uint8_t* b_base = p.b + (b_row0 + n0) * kbytes;
-  const uint8_t* bsf_base = p.sfb + b_row0 * sf_padded + swizzle_128x4(n0 & ~127, 0, sf_padded);
-  const uint8_t* a_base = p.a + a_row0 * kbytes;
-  const uint8_t* asf_base = p.sfa + asf_row0 * sf_padded;  // the 128-row scale tile of these rows (row0 % 128 == 0)
+  const uint8_t* b_base = p.b + (b_row0 + n0) * kbytes + c_lo * 64;
+  const uint8_t* bsf_base = p.sfb + b_row0 * sf_padded + swizzle_128x4(n0 & ~127, 0, sf_padded) + (int64_t)c_lo * 1024;
+  const uint8_t* a_base = p.a + a_row0 * kbytes + c_lo * 64;
+  const uint8_t* asf_base = p.sfa + asf_row0 * sf_padded + (int64_t)c_lo * 1024;  // the 128-row scale tile of these rows (row0 % 128 == 0)
   uint32_t b_off[RT], a_off[TT], bsf_off[B_SC], asf_off[A_SC];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) b_off[rt] = (uint32_t)(rt * 16 + lrow) * (uint32_t)kbytes + lpiece * 16;
@@ -1313,10 +1319,15 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
         for (int w = 1; w < W; ++w) s += red[w * units + u];
         const int tok = tt * 16 + (l & 15);
         if (tok < m_loc) {
-          u32x2 v;
-          v[0] = pack2(s[0] * alpha, s[1] * alpha, OUT_BF16);
-          v[1] = pack2(s[2] * alpha, s[3] * alpha, OUT_BF16);
-          *reinterpret_cast<u32x2*>(out + (a_row0 + tok) * p.n + n0 + (round * RPR + r2) * 16 + 4 * (l >> 4)) = v;
+          const int64_t at = (a_row0 + tok) * p.n + n0 + (round * RPR + r2) * 16 + 4 * (l >> 4);
+          if (!GROUPED && p.partial != nullptr) {  // this K range's sums as they are; the reduction applies alpha
+            *reinterpret_cast<f32x4*>(p.partial + (int64_t)blockIdx.z * p.m * p.n + at) = s;
+          } else {
+            u32x2 v;
+            v[0] = pack2(s[0] * alpha, s[1] * alpha, OUT_BF16);
+            v[1] = pack2(s[2] * alpha, s[3] * alpha, OUT_BF16);
+            *reinterpret_cast<u32x2*>(out + at) = v;
+          }
         }
       }
     }
@@ -1462,6 +1473,119 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
                                                                  __builtin_bit_cast(f16x8, fa[t]), acc[rt][tt], 0, 0, 0);
       }
     };
+    // s_waitcnt vmcnt(n) for a wave-uniform n (the operand is an immediate)
+    auto wait_loads = [&](int n) {
+      switch (n) {
+#define NVF_VMCNT_CASE(n) case n: asm volatile("s_waitcnt vmcnt(" #n ")" ::: "memory"); break;
+        NVF_VMCNT_CASE(1) NVF_VMCNT_CASE(2) NVF_VMCNT_CASE(3) NVF_VMCNT_CASE(4) NVF_VMCNT_CASE(5) NVF_VMCNT_CASE(6)
+        NVF_VMCNT_CASE(7) NVF_VMCNT_CASE(8) NVF_VMCNT_CASE(9) NVF_VMCNT_CASE(10) NVF_VMCNT_CASE(11) NVF_VMCNT_CASE(12)
+        NVF_VMCNT_CASE(13) NVF_VMCNT_CASE(14) NVF_VMCNT_CASE(15) NVF_VMCNT_CASE(16) NVF_VMCNT_CASE(17) NVF_VMCNT_CASE(18)
+        NVF_VMCNT_CASE(19) NVF_VMCNT_CASE(20) NVF_VMCNT_CASE(21) NVF_VMCNT_CASE(22) NVF_VMCNT_CASE(23) NVF_VMCNT_CASE(24)
+        NVF_VMCNT_CASE(25) NVF_VMCNT_CASE(26) NVF_VMCNT_CASE(27) NVF_VMCNT_CASE(28) NVF_VMCNT_CASE(29) NVF_VMCNT_CASE(30)
+#undef NVF_VMCNT_CASE
+        default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      }
+    };
+    // one dword of an MFMA operand: two of a raw dword's eight values (byte `sel`), times their block's scale
+    auto dequant_pair = [&](uint32_t qw, int sel, f16x2 sv) {
+      const f16x2 h = (sel == 0   ? __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(qw, 1.0f, 0)
+                       : sel == 1 ? __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(qw, 1.0f, 1)
+                       : sel == 2 ? __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(qw, 1.0f, 2)
+                                  : __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(qw, 1.0f, 3)) * sv;
+      return __builtin_bit_cast(uint32_t, h);
+    };
+    // One chunk for tile counts whose accumulators leave no registers for the scheme above (RT * TTC > 20).  A
+    // wavefront issues one conversion instruction per 8 cycles at best and an MFMA of this shape per 16, so a chunk
+    // that converts a tile and then multiplies it takes the sum of both; here the two instructions that make one
+    // dword of an activation operand follow every MFMA, so that they issue while the matrix pipe works: the 8 MFMAs
+    // on the first half of a tile's K range (2 steps x RT weight tiles) carry the conversion of its second half, the 8
+    // on the second half that of the next tile's first half.  Only the weight operands of the whole chunk are
+    // converted up front.  A tile's raw bytes are read out of LDS one tile ahead and its slot is refilled with the
+    // wavefront's next chunk at once, the weight part right at the start of the chunk: every load has most of a
+    // chunk's time to land.  Loads complete in the order of issue, and that order is fixed - weight part, then per
+    // tile its bytes and, after every second tile and the last, the scale block of the pair - so the waits are for
+    // counts that follow from it.
+    auto chunk_pipe = [&](auto ttc_c, uint32_t c, auto& acc) {
+      constexpr int TTC = decltype(ttc_c)::value;
+      constexpr int NS = (TTC + 1) / 2, NA = TTC + NS, LB = RT + B_SC;
+      const bool has_next = c + CSTEP < (uint32_t)chunks;
+      // loads of this chunk still pending once tile tt and the scale block of its pair have landed
+      auto after_tile = [&](int tt) {
+        const int last_of_pair = (tt | 1) < TTC ? (tt | 1) : TTC - 1;
+        return NA - 1 - (last_of_pair + (last_of_pair >> 1) + 1);
+      };
+      wait_loads(NA);  // the weight part has landed
+      u32x4 q[RT];
+      uint32_t sc[RT];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) q[rt] = *reinterpret_cast<const u32x4*>(sp + rt * 1024 + rd_payload);
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) sc[rt] = *reinterpret_cast<const uint32_t*>(sp + rd_bsc[rt]) >> sc_shift;
+      wait_loads(after_tile(0));
+      u32x4 aq, aqn = {0, 0, 0, 0};
+      uint32_t as, asn = 0;
+      read_a_tile(0, aq, as);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // read out: may be refilled
+      if (has_next) {
+        load_b_part(c + CSTEP);
+        load_a_tile(c + CSTEP, 0);
+        if (TTC == 1) load_a_scales(c + CSTEP, 0);
+      }
+      u32x4 fb[RT][4];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        f16x2 sv[2];
+        scale_pairs(sc[rt], sv);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) fb[rt][t] = dequant_dword(q[rt][t], sv[t >> 1]);
+      }
+      f16x2 asv[2], asvn[2];
+      scale_pairs(as, asv);
+      u32x4 fa[2], fan[2];
+      fa[0] = dequant_dword(aq[0], asv[0]);
+      fa[1] = dequant_dword(aq[1], asv[0]);
+#pragma unroll
+      for (int tt = 0; tt < TTC; ++tt) {
+        __builtin_amdgcn_sched_barrier(0);
+        if (tt + 1 < TTC) {
+          // pending behind tile tt+1: the rest of this chunk's tiles, the next chunk's weight part and its tiles 0..tt
+          wait_loads(after_tile(tt + 1) + (has_next ? LB + (tt + 1) + ((tt + 1) >> 1) : 0));
+          read_a_tile(tt + 1, aqn, asn);
+        }
+        // K steps 0 and 1 of tile tt; behind every MFMA one dword of the operands of its steps 2 and 3
+#pragma unroll
+        for (int m = 0; m < 8; ++m) {
+          const int t = m >> 2, rt = m & 3;
+#pragma unroll
+          for (int r2 = rt; r2 < RT; r2 += 4)
+            acc[r2][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, fb[r2][t]), __builtin_bit_cast(f16x8, fa[t]),
+                                                                 acc[r2][tt], 0, 0, 0);
+          fan[m >> 2][m & 3] = dequant_pair(aq[2 + (m >> 2)], m & 3, asv[1]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        if (tt + 1 < TTC) {
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // tile tt+1 is in registers: its slot may be refilled
+          if (has_next) {
+            load_a_tile(c + CSTEP, tt + 1);
+            if (((tt + 1) & 1) || tt + 2 == TTC) load_a_scales(c + CSTEP, (tt + 1) >> 1);
+          }
+          scale_pairs(asn, asvn);
+        }
+        // K steps 2 and 3 of tile tt; behind every MFMA one dword of the next tile's operands of steps 0 and 1
+#pragma unroll
+        for (int m = 0; m < 8; ++m) {
+          const int t = m >> 2, rt = m & 3;
+#pragma unroll
+          for (int r2 = rt; r2 < RT; r2 += 4)
+            acc[r2][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, fb[r2][2 + t]), __builtin_bit_cast(f16x8, fan[t]),
+                                                                 acc[r2][tt], 0, 0, 0);
+          if (tt + 1 < TTC) fa[m >> 2][m & 3] = dequant_pair(aqn[m >> 2], m & 3, asvn[0]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        aq = aqn;
+        asv[1] = asvn[1];
+      }
+    };
     auto run = [&](auto ttc_c) {
       constexpr int TTC = decltype(ttc_c)::value;
       constexpr bool kFits = RT * TTC <= 20;  // accumulator registers that leave room for the finer scheme
@@ -1479,7 +1603,8 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
         }
       }
       for (int c = c_first; c < chunks; c += CSTEP) {
-        if constexpr (!kFits) chunk_coarse(ttc_c, (uint32_t)c, acc);
+        if constexpr (!kFits && RT == 4) chunk_pipe(ttc_c, (uint32_t)c, acc);
+        else if constexpr (!kFits) chunk_coarse(ttc_c, (uint32_t)c, acc);
         else chunk(ttc_c, (uint32_t)c, acc);
       }
       finish(ttc_c, acc);
@@ -1573,11 +1698,20 @@ int launch_nvfp4_skinny_ring_cfg(const Params& p, hipStream_t stream, int slabs 
   constexpr int ring_kib = 8 * DEPTH * SLOT_KIB;
   constexpr int lds_bytes = (ring_kib > red_kib ? ring_kib : red_kib) * 1024;
   static_assert(lds_bytes <= 160 * 1024, "LDS");
-  if (note_launch("nvfp4_skinny_ring_kernel<RT=%d,TT=%d> grid=%ux%d", RT, TT, (unsigned)(p.n / (16 * RT)), slabs)) return NVF_OK;
+  const int splits = p.partial != nullptr ? p.splits : 1;
+  if (splits > 1 ? note_launch("nvfp4_skinny_ring_kernel<RT=%d,TT=%d> grid=%ux%dx%d split_k + splitk_reduce_kernel", RT, TT,
+                               (unsigned)(p.n / (16 * RT)), slabs, splits)
+                 : note_launch("nvfp4_skinny_ring_kernel<RT=%d,TT=%d> grid=%ux%d", RT, TT, (unsigned)(p.n / (16 * RT)), slabs))
+    return NVF_OK;
   static std::atomic<uint64_t> configured{0};  // one bit per device
   if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
-  hipLaunchKernelGGL(kern, dim3((unsigned)(p.n / (16 * RT)), (unsigned)slabs), dim3(512), lds_bytes, stream, p);
-  return check_launch("nvfp4_skinny_ring_kernel");
+  hipLaunchKernelGGL(kern, dim3((unsigned)(p.n / (16 * RT)), (unsigned)slabs, (unsigned)splits), dim3(512), lds_bytes, stream, p);
+  if (const int rc = check_launch("nvfp4_skinny_ring_kernel")) return rc;
+  if (p.partial == nullptr) return NVF_OK;
+  const int64_t mn = (int64_t)p.m * p.n;
+  hipLaunchKernelGGL(splitk_reduce_kernel<OUT_BF16>, dim3((unsigned)ceil_div(mn / 4, 256)), dim3(256), 0, stream, p.partial, splits, mn, p.alpha,
+                     static_cast<uint16_t*>(p.out));
+  return check_launch("splitk_reduce_kernel");
 }
 
 template <int RT, int TT, bool OUT_BF16, bool NSPLIT>
@@ -2346,6 +2480,22 @@ int nvfp4_splits(int64_t m, int64_t n, int64_t k, int cus) {
   return s < 2 ? 1 : (int)s;
 }
 
+// Split of K over workgroups for the weight-streaming kernel with one slab of 65..128 activation rows: every
+// workgroup converts all activation rows of its K range next to its weight rows, so 64 weight rows per workgroup
+// (4 tiles against 8 activation tiles: 12 conversions for 32 MFMA tiles) halve the conversion work of 16 (1 against
+// 8: 9 for 8), and where N / 64 workgroups leave compute units idle, K is split over as many workgroups as fit.
+int nvfp4_skinny_splits(int64_t m, int64_t n, int64_t k, int cus) {
+  if (m <= 64 || m > 128 || (k & 127) != 0 || (n & 63) != 0 || k * 64 >= (1ll << 31)) return 1;
+  const int64_t wgs = n / 64, chunks = k >> 7;
+  int64_t s = cus / wgs;
+  // at least three chunks per wavefront: with one (M=128, N=4096, K=4096 as 4 splits) the launch takes 16.4 us against
+  // 12.3 us without a split; with 3.5 (K=14336) 25.2 us against 35.7 us on the tile kernel's split
+  if (s > chunks / 24) s = chunks / 24;
+  if (s > 8) s = 8;
+  if (wgs * s * 2 < cus) return 1;  // would leave most compute units idle: the tile kernel's split has more items
+  return s < 2 ? 1 : (int)s;
+}
+
 template <bool OUT_BF16>
 int launch_nvfp4_splitk(const Params& p0, int splits, float* workspace, hipStream_t stream) {
   Params p = p0;
@@ -2382,6 +2532,15 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int6
   const bool dense = p.problem_sizes == nullptr;
   if constexpr (NVFP4) {
     if (dense && workspace != nullptr) {
+      const int skinny_splits = nvfp4_skinny_splits(p.m, p.n, p.k, cus);
+      if (skinny_splits > 1 && workspace_bytes >= (int64_t)skinny_splits * p.m * p.n * 4) {
+        Params q = p;
+        const int chunks = p.k >> 7;
+        q.partial = static_cast<float*>(workspace);
+        q.spans_per_split = (chunks + skinny_splits - 1) / skinny_splits;
+        q.splits = (chunks + q.spans_per_split - 1) / q.spans_per_split;  // no empty split
+        return launch_nvfp4_skinny_ring_cfg<4, 8, OUT_BF16>(q, stream, 1);
+      }
       const int splits = nvfp4_splits(p.m, p.n, p.k, cus);
       if (splits > 1 && workspace_bytes >= (int64_t)splits * p.m * p.n * 4)
         return launch_nvfp4_splitk<OUT_BF16>(p, splits, static_cast<float*>(workspace), stream);
@@ -2591,7 +2750,8 @@ int static_scratch(void** ptr) {
 
 int64_t nvfp4_gemm_workspace_bytes(int64_t m, int64_t n, int64_t k) {
   if (m <= 0 || n <= 0 || k <= 0 || m > INT32_MAX || n > INT32_MAX || k > INT32_MAX) return 0;
-  const int splits = nvfp4_splits(m, n, k, cu_count());
+  const int skinny_splits = nvfp4_skinny_splits(m, n, k, cu_count());
+  const int splits = skinny_splits > 1 ? skinny_splits : nvfp4_splits(m, n, k, cu_count());
   return splits > 1 ? (int64_t)splits * m * n * 4 : 0;
 }
 

@@ -40,8 +40,17 @@ def test_config3_llm_shapes(m, n, k, kernel):
 def test_config3_deep_k_with_a_workspace_splits_k():
     need = capi.lib().nvf_nvfp4_scaled_mm_workspace_bytes(128, 4096, 14336)
     assert need > 0
-    assert plan("nvfp4_scaled_mm", 128, 4096, 14336, ws=need).startswith("nvfp4_tile_kernel<128,128,split_k>")
-    assert plan("nvfp4_scaled_mm", 128, 4096, 14336, ws=need - 1).startswith("nvfp4_skinny_ring_kernel<")
+    # one slab of 65..128 rows against N / 64 < compute units: the weight-streaming kernel, K split over 4 workgroups
+    got = plan("nvfp4_scaled_mm", 128, 4096, 14336, ws=need)
+    assert got == "nvfp4_skinny_ring_kernel<RT=4,TT=8> grid=64x1x4 split_k + splitk_reduce_kernel", got
+    assert need == 4 * 128 * 4096 * 4
+    got = plan("nvfp4_scaled_mm", 128, 4096, 14336, ws=need - 1)
+    assert got.startswith("nvfp4_skinny_ring_kernel<") and "split_k" not in got, got
+    # a shallower K is not split (one chunk per wavefront costs more than the idle compute units)
+    assert capi.lib().nvf_nvfp4_scaled_mm_workspace_bytes(128, 4096, 4096) == 0
+    # few weight rows and a deep K: the tile kernel's split has more work items
+    need = capi.lib().nvf_nvfp4_scaled_mm_workspace_bytes(128, 1024, 8192)
+    assert plan("nvfp4_scaled_mm", 128, 1024, 8192, ws=need).startswith("nvfp4_tile_kernel<128,128,split_k>")
 
 
 def test_nvfp4_8192_cubed_takes_the_persistent_256x256_kernel():
