@@ -39,6 +39,8 @@ def parse():
     ap.add_argument("--no-extra", action="store_true", help="only the headline MXFP8 workload")
     ap.add_argument("--calib", action="store_true", help="profiling aid: also run a plain 1 GiB device copy a few times, "
                     "so that a counter run shows what FETCH_SIZE / WRITE_SIZE read for a kernel of known traffic")
+    ap.add_argument("--no-graph", action="store_true", help="profiling aid: skip the HIP-graph timings of the decode-sized GEMMs "
+                    "(counter runs attribute a replayed graph's kernels poorly)")
     ap.add_argument("--only", default="", help="profiling aid: run just this extra workload "
                     "(quant | fused | nvfp4 | llm | grouped | gnvfp4) and print its line")
     return ap.parse_args()
@@ -80,6 +82,35 @@ def main():
         wall = (time.perf_counter() - t0) * 1e3 / steps
         return e0.elapsed_time(e1) / steps, wall
 
+    def timed_graph(calls, replays=20):
+        if args.no_graph:
+            return float("nan")
+        return _timed_graph(calls, replays)
+
+    def _timed_graph(calls, replays):
+        """Average milliseconds per call of the list `calls`, captured once as a HIP graph (one node sequence per call) and
+        replayed: the launches cost no host time, so a call of a few microseconds is timed by what the GPU does."""
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            for fn in calls[:2]:
+                fn()  # one-time set-up of the kernels outside the capture
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                for fn in calls:
+                    fn()
+            t_end = time.perf_counter() + min(args.preheat_ms, 100.0) * 1e-3
+            while time.perf_counter() < t_end:
+                graph.replay()
+                torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(replays):
+                graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / (replays * len(calls))
+
     def ru(x, y):
         return (x + y - 1) // y * y
 
@@ -100,7 +131,7 @@ def main():
 
     # CPU baselines ("port": the oracle's recipes, i.e. its scalar C restatement for the quantizer and torch-CPU
     # dequantize + fp32 matmul for the GEMMs), timed on this box's host cores on a bounded sample of each workload.
-    cpu_threads = min(os.cpu_count() or 1, 16)
+    cpu_threads = os.cpu_count() or 1
     if not args.no_cpu:
         torch.set_num_threads(cpu_threads)
         from oracle import nvf_oracle as O
@@ -213,9 +244,17 @@ def main():
                                                "note": "one launch: the product is re-quantized to NVFP4 in the GEMM's epilogue"}
 
     def run_llm():
+        # BASELINE config 3.  The decode-sized shapes (M = 16, 128) are bound by streaming the weights once, and one
+        # weight tensor of 9-33 MB lives in the 256 MB last-level cache: they are therefore timed three ways - eager calls
+        # on one weight tensor (`gemm_us`, as a Python serving loop would issue them: the host's launch cost is in it),
+        # the same calls replayed from a HIP graph (`gemm_us_graph_warm`), and a graph that rotates over enough weight
+        # tensors to exceed the cache (`gemm_us_graph_rotated`: every call streams its weights from HBM).  The roofline
+        # fractions are those of the rotated figure.
         res = {}
         for (n, k) in ((4096, 4096), (14336, 4096), (4096, 14336)):
-            w, sw, gw = quantized_nvfp4(n, k, 0.02)
+            copies = int(320e6 // (n * k * 0.5625)) + 1
+            ws = [quantized_nvfp4(n, k, 0.02) for _ in range(copies)]
+            w, sw, gw = ws[0]
             for m in (16, 128, 2048):
                 x = torch.randn(m, k, device=dev, generator=gen).bfloat16()
                 gx = (2688.0 / x.float().abs().max()).float()
@@ -224,21 +263,33 @@ def main():
                 ms_q, _ = timed(lambda: ops.nv_block_quantize(x, gx, True, 16), 50, 5)
                 ms_g, _ = timed(lambda: nvf_cutlass.nvfp4_scaled_mm(qx, w, sx, sw, alpha, torch.bfloat16), 50, 5)
 
-                def seq():
+                def seq(wi=w, swi=sw):
                     q, s = ops.nv_block_quantize(x, gx, True, 16)
-                    return nvf_cutlass.nvfp4_scaled_mm(q, w, s, sw, alpha, torch.bfloat16)
+                    return nvf_cutlass.nvfp4_scaled_mm(q, wi, s, swi, alpha, torch.bfloat16)
 
                 ms_s, _ = timed(seq, 50, 5)
+                reps = copies if m < 2048 else 4
+                ms_gw = timed_graph([lambda: nvf_cutlass.nvfp4_scaled_mm(qx, w, sx, sw, alpha, torch.bfloat16)] * reps)
+                ms_gr = timed_graph([(lambda wi=wi, swi=swi: nvf_cutlass.nvfp4_scaled_mm(qx, wi, sx, swi, alpha, torch.bfloat16))
+                                     for (wi, swi, _) in ws[:reps]])
+                ms_sr = timed_graph([(lambda wi=wi, swi=swi: seq(wi, swi)) for (wi, swi, _) in ws[:reps]])
                 byts = n * k * 0.5625 + m * k * 0.5625 + 2 * m * n
                 res[f"M{m}_N{n}_K{k}"] = {"quant_us": round(ms_q * 1e3, 2), "gemm_us": round(ms_g * 1e3, 2), "seq_us": round(ms_s * 1e3, 2),
-                                          "gemm_TFLOP/s": round(2.0 * m * n * k / ms_g / 1e9, 1), "gemm_GB/s": round(byts / ms_g / 1e6, 1),
-                                          "frac_of_f16_peak": round(2.0 * m * n * k / ms_g / 1e9 / PEAK_F16_TFLOPS, 4),
-                                          "frac_of_hbm_peak": round(byts / ms_g / 1e6 / PEAK_HBM_GBS, 4)}
+                                          "gemm_us_graph_warm": round(ms_gw * 1e3, 2), "gemm_us_graph_rotated": round(ms_gr * 1e3, 2),
+                                          "seq_us_graph_rotated": round(ms_sr * 1e3, 2), "weight_tensors_in_rotation": reps,
+                                          "gemm_TFLOP/s": round(2.0 * m * n * k / ms_gr / 1e9, 1), "gemm_GB/s": round(byts / ms_gr / 1e6, 1),
+                                          "frac_of_f16_peak": round(2.0 * m * n * k / ms_gr / 1e9 / PEAK_F16_TFLOPS, 4),
+                                          "frac_of_hbm_peak": round(byts / ms_gr / 1e6 / PEAK_HBM_GBS, 4)}
                 if not args.no_cpu:
                     hq, hs, hw, hsw = (t.view(torch.uint8).cpu() for t in (qx, sx, w, sw))
                     al = float(alpha)
                     sec, _ = cpu_timed(lambda: O.ref_nvfp4_scaled_mm(hq, hw, hs, hsw, al), max_runs=1)
                     res[f"M{m}_N{n}_K{k}"]["cpu_us"] = round(sec * 1e6, 0)
+            del ws
+        res["timing"] = ("gemm_us / quant_us / seq_us: eager calls on one weight tensor, HIP events (host launch cost included); "
+                         "*_graph_warm: the same call replayed from a HIP graph; *_graph_rotated: a graph over enough weight tensors "
+                         "to exceed the 256 MB last-level cache (> 320 MB), so that the weights stream from HBM; TFLOP/s, GB/s and "
+                         "the fractions are those of gemm_us_graph_rotated")
         if not args.no_cpu:
             res["cpu_baseline"] = {"unit": "us per call (cpu_us of every shape)", "cores": cpu_threads, "kind": "port",
                                    "sample": "each of the nine shapes once, whole: torch-CPU dequantize of both operands + fp32 matmul"}
@@ -315,7 +366,12 @@ def main():
             ms, _ = timed(lambda: nvf_cutlass.nvfp4_scaled_grouped_mm(aq, bq4, asf, bsf8, alphas, st, ct, ps, eo, so, torch.bfloat16), 10, 2)
             tf = 2.0 * rows * n * k / ms / 1e9
             res[f"K{k}_N{n}"] = {"ms": round(ms, 4), "useful_TFLOP/s": round(tf, 1), "frac_of_f16_peak": round(tf / PEAK_F16_TFLOPS, 4),
-                                 "frac_of_fp8_peak": round(tf / PEAK_FP8_TFLOPS, 4), "frac_of_fp4_peak": round(tf / PEAK_FP4_TFLOPS, 4)}
+                                 "frac_of_fp8_peak": round(tf / PEAK_FP8_TFLOPS, 4), "frac_of_fp4_peak": round(tf / PEAK_FP4_TFLOPS, 4),
+                                 "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
+                                              "frac": round(tf / PEAK_F16_TFLOPS, 4),
+                                              "traffic": measured_traffic.get(f"nvfp4_grouped_mm_config5_K{k}_N{n}_bytes_per_call"),
+                                              "kernel": "nvfp4_gemm_256_kernel (+ nvfp4_group_panel_kernel, nvfp4_skinny_ring_kernel: the call's launches)",
+                                              "algorithmic_bytes": int(g * n * k * 0.5625 + rows * k * 0.5625 + 2 * rows * n)}}
             if not args.no_cpu:
                 ne = 16  # the first 16 experts and their rows
                 r_end, s_end = int(eo[ne]), int(so[ne])
