@@ -215,7 +215,8 @@ def test_nvfp4_gemm_llm_and_ragged_shapes(dev, shape):
                                    (32, 6592, 128), (25, 6560, 256), (40, 6560, 384), (50, 13056, 256),
                                    (100, 13056, 384), (128, 6560, 1152), (81, 96, 2048), (129, 64, 256), (200, 6560, 384),
                                    (256, 96, 1152), (192, 512, 2048), (100, 1024, 256), (250, 2048, 384), (150, 1024, 640),
-                                   (60, 160, 512), (250, 4096, 256)])
+                                   (60, 160, 512), (250, 4096, 256),
+                                   (16, 13056, 4352), (31, 6592, 4224), (12, 256, 6272), (32, 13120, 2176), (2, 64, 256)])
 def test_nvfp4_gemm_decode_sized_activations(dev, shape):
     """M <= 256 (in one launch of slabs of 128, 64 or 32 rows, the last one ragged) with K % 128 == 0 and N % 16 == 0 takes the kernel that streams the
     weights once and splits K over the wavefronts of a workgroup, the tiles travelling through a per-wavefront ring in LDS:
