@@ -2104,6 +2104,13 @@ int launch_nvfp4_group_panel(const Params& p0, int rows_lo, int rows_hi, hipStre
 }
 
 template <int TT, bool OUT_BF16>
+int launch_nvfp4_skinny_rt(const Params& p, int rt, hipStream_t stream, int slabs) {
+  return rt == 4 ? launch_nvfp4_skinny_ring_cfg<4, TT, OUT_BF16>(p, stream, slabs)
+       : rt == 2 ? launch_nvfp4_skinny_ring_cfg<2, TT, OUT_BF16>(p, stream, slabs)
+                 : launch_nvfp4_skinny_ring_cfg<1, TT, OUT_BF16>(p, stream, slabs);
+}
+
+template <int TT, bool OUT_BF16>
 int launch_nvfp4_skinny_tt(const Params& p, int cus, hipStream_t stream, int slabs = 1) {
   // The conversion work bounds this kernel, and every workgroup converts all activation rows it uses:
   // take as many weight rows per workgroup as still leaves about one workgroup per compute unit.
@@ -2113,30 +2120,53 @@ int launch_nvfp4_skinny_tt(const Params& p, int cus, hipStream_t stream, int sla
   return launch_nvfp4_skinny_ring_cfg<1, TT, OUT_BF16>(p, stream, slabs);
 }
 
+// Cost, in arbitrary units, of streaming the weights against M activation rows as slabs of `slab` rows with rt weight
+// tiles (16 rows) per workgroup.  Every workgroup converts rt weight tiles and the tt row tiles of its slab per
+// 128-deep chunk (a wavefront takes every eighth chunk), so few large workgroups convert least, while small ones (less
+// LDS, fewer accumulators) share a compute unit and fill the chip at small N.  The constants are a fit to timings of
+// the nine (slab, rt) forms over M = 48..256, N = 1024..14336, K = 2048..14336 (144 shapes: the form picked is within
+// 8 % of the fastest for 134 of them, 1.8 % off on average; a fixed rule by N alone was 13 % off).
+int64_t nvfp4_skinny_cost(int64_t m, int64_t n, int64_t k, int slab, int rt, int cus) {
+  if (n % (16 * rt) != 0) return INT64_MAX;
+  const int64_t slabs = m <= slab ? 1 : ceil_div(m, slab);
+  const int tt = m <= slab ? (m <= 16 ? 1 : m <= 32 ? 2 : m <= 64 ? 4 : 8) : slab / 16;
+  const int64_t wgs = slabs * (n / (16 * rt));
+  const int lds_kib = 8 * (rt + tt + (rt + 1) / 2 + (tt + 1) / 2);
+  int64_t per_cu = std::min(160 / lds_kib, 4);  // workgroups that share a compute unit
+  if (rt * tt > 16) per_cu = 1;                 // (their accumulators take the registers)
+  else if (rt * tt > 6) per_cu = std::min<int64_t>(per_cu, 2);
+  if (per_cu < 1) per_cu = 1;
+  const int64_t chunks = ceil_div(k >> 7, 8);
+  const int64_t resident = std::min(per_cu, ceil_div(wgs, cus));
+  const int64_t rounds = ceil_div(wgs, cus * per_cu);
+  const int64_t per_chunk = (rt + tt) * 183 + rt * tt * 18 + 100;
+  const int64_t wg_time = chunks * per_chunk * (100 + 73 * (resident - 1)) / 100 + rt * tt * 110 + 5070;
+  return rounds * wg_time;
+}
+
 template <bool OUT_BF16>
 int launch_nvfp4_skinny(const Params& p, int cus, hipStream_t stream) {
-  // More than 128 rows: slabs, each streaming the weights (the later ones out of the last-level cache), side by
-  // side in one launch (blockIdx.y = slab; the last one may be ragged).  Where N is so small that a workgroup has
-  // 16 weight rows, the slab height is 128, 64 or 32 rows, whichever fills the chip best: every workgroup
-  // converts all activation rows of its slab, lower slabs need less LDS, so that 2 to 4 workgroups share a
-  // compute unit, and with L workgroups per compute unit a launch takes about 17.5 L / 10.3 + 6.5 (L - 1) /
-  // 6.7 + 3.5 (L - 1) us at K = 7168 (measured: 128 x 1024 x 7168 17.6 -> 6.5 us, 256 x 4096 x 7168 34.9 -> 29.8 us).
-  int slab = 128;
-  if (!((p.n & 31) == 0 && p.n / 32 >= (int64_t)cus * 4 / 5)) {
-    auto load = [&](int rows) { return ceil_div(ceil_div(p.m, rows) * (int64_t)(p.n / 16), cus); };
-    const int64_t c128 = 175 * load(128), c64 = 38 + 65 * load(64), c32 = 32 + 35 * load(32);
-    slab = c128 <= c64 && c128 <= c32 ? 128 : (c64 <= c32 ? 64 : 32);
-  }
+  // Up to 32 rows: one slab, as many weight rows per workgroup as still leaves about one workgroup per compute unit
+  // (bound by the weight stream, not by conversions).
+  if (p.m <= 32) return p.m <= 16 ? launch_nvfp4_skinny_tt<1, OUT_BF16>(p, cus, stream) : launch_nvfp4_skinny_tt<2, OUT_BF16>(p, cus, stream);
+  // More rows: slabs of 128, 64 or 32 rows side by side in one launch (blockIdx.y = slab; the last one may be ragged;
+  // the slabs after the first find the weights in the last-level cache) with 1, 2 or 4 weight tiles per workgroup,
+  // whichever the cost estimate above prefers (M=128, N=4096, K=4096: 10.8 us as two slabs of 64 rows x 1 weight tile,
+  // 8.3 us x 2 tiles; M=256, N=4096, K=14336: 62 -> 34 us; M=256, N=6144, K=7168: 48 -> 29 us).
+  int slab = 128, rt = 1;
+  int64_t best = INT64_MAX;
+  for (const int s : {128, 64, 32})
+    for (const int r : {4, 2, 1}) {
+      const int64_t c = nvfp4_skinny_cost(p.m, p.n, p.k, s, r, cus);
+      if (c < best) best = c, slab = s, rt = r;
+    }
   if (p.m > slab) {
     const int slabs = (int)ceil_div(p.m, slab);
-    return slab == 128 ? launch_nvfp4_skinny_tt<8, OUT_BF16>(p, cus, stream, slabs)
-         : slab == 64  ? launch_nvfp4_skinny_tt<4, OUT_BF16>(p, cus, stream, slabs)
-                       : launch_nvfp4_skinny_tt<2, OUT_BF16>(p, cus, stream, slabs);
+    return slab == 128 ? launch_nvfp4_skinny_rt<8, OUT_BF16>(p, rt, stream, slabs)
+         : slab == 64  ? launch_nvfp4_skinny_rt<4, OUT_BF16>(p, rt, stream, slabs)
+                       : launch_nvfp4_skinny_rt<2, OUT_BF16>(p, rt, stream, slabs);
   }
-  return p.m <= 16 ? launch_nvfp4_skinny_tt<1, OUT_BF16>(p, cus, stream)
-       : p.m <= 32 ? launch_nvfp4_skinny_tt<2, OUT_BF16>(p, cus, stream)
-       : p.m <= 64 ? launch_nvfp4_skinny_tt<4, OUT_BF16>(p, cus, stream)
-                   : launch_nvfp4_skinny_tt<8, OUT_BF16>(p, cus, stream);
+  return p.m <= 64 ? launch_nvfp4_skinny_rt<4, OUT_BF16>(p, rt, stream, 1) : launch_nvfp4_skinny_rt<8, OUT_BF16>(p, rt, stream, 1);
 }
 
 // -------------------------------------------------------------------------------------------------

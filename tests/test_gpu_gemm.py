@@ -238,6 +238,31 @@ def test_nvfp4_gemm_decode_sized_activations(dev, shape):
         assert torch.equal(out, _run_nvfp4(a, b, sa_p, sb, alpha, dtype, dev))
 
 
+@pytest.mark.parametrize("nk", [(1024, 2048), (2048, 4096), (4096, 2048), (6144, 2176), (4096, 7168), (8192, 1152), (14336, 640)])
+def test_nvfp4_gemm_slab_height_and_weight_tiles_by_cost(dev, nk):
+    """33..256 rows: the weight-streaming kernel runs as slabs of 128, 64 or 32 rows with 1, 2 or 4 weight tiles per
+    workgroup, picked by a cost estimate.  Row counts on both sides of the slab heights (ragged last slabs), shapes that
+    select each of the nine forms; every element compared, both output types, run-to-run bit equality."""
+    from fuser_amd import capi
+
+    n, k = nk
+    gen = torch.Generator().manual_seed(n + k)
+    b, sb, gb = _nvfp4_operand(n, k, 0.02, gen)
+    forms = set()
+    for m in (33, 48, 64, 65, 96, 100, 128, 129, 192, 200, 256):
+        plan = capi.describe_dispatch("nvfp4_scaled_mm", m, n, k)
+        assert plan.startswith("nvfp4_skinny_ring_kernel<"), plan
+        forms.add(plan.split(" ")[0])
+        a, sa, ga = _nvfp4_operand(m, k, 1.0, gen)
+        alpha = 1.0 / (ga * gb)
+        ref = O.ref_nvfp4_scaled_mm(a, b, sa, sb, alpha)
+        for dtype in (torch.bfloat16, torch.float16):
+            out = _run_nvfp4(a, b, sa, sb, alpha, dtype, dev)
+            assert out.shape == (m, n) and max_rel_rowwise(out, ref) <= GEMM_MAX_REL, (m, n, k, dtype, plan)
+            assert torch.equal(out, _run_nvfp4(a, b, sa, sb, alpha, dtype, dev))
+    assert len(forms) >= 2, forms
+
+
 @pytest.mark.parametrize("shape", [(300, 2048, 2048), (512, 1536, 2304), (384, 3072, 4096), (640, 544, 2176), (1000, 288, 2560),
                                    (257, 32, 2048), (1024, 768, 2048), (2100, 96, 4096)])
 def test_nvfp4_gemm_many_rows_small_n_deep_k(dev, shape):
