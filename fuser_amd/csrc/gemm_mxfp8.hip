@@ -717,48 +717,69 @@ int launch_skinny_tt(const Params& p, hipStream_t stream, int slabs = 1) {
   return launch_skinny_cfg<1, TT, OUT_BF16>(p, stream, slabs);
 }
 
+template <int TT, bool OUT_BF16>
+int launch_skinny_rt(const Params& p, int rt, hipStream_t stream, int slabs) {
+  if constexpr (TT == 8) return launch_skinny_cfg<1, 8, OUT_BF16>(p, stream, slabs);
+  else
+    return rt == 4 ? launch_skinny_cfg<4, TT, OUT_BF16>(p, stream, slabs)
+         : rt == 2 ? launch_skinny_cfg<2, TT, OUT_BF16>(p, stream, slabs)
+                   : launch_skinny_cfg<1, TT, OUT_BF16>(p, stream, slabs);
+}
+
+// Estimated duration of the skinny kernel for (slab height, weight tiles per workgroup), in units of about 1 ns: the
+// workgroups (one per slab and 16*rt weight rows; one per compute unit at a time, the ring fills its LDS) run in
+// rounds over the compute units; a wavefront visits ceil(chunks / 8) chunks, each costing the LDS-direct loads of
+// its rt + tt tiles and rt * tt MFMAs, then comes the reduction of rt * tt partial tiles.  A last round that is only
+// partly filled costs 70 % of a full one plus its share of the rest; the weight stream bounds the whole from below.
+// Constants fitted to a sweep of the seven forms over 140 shapes (M 48..256, N 1024..14336, K 2048..14336): the form
+// picked is within 7 % of the best everywhere.
+int64_t mxfp8_skinny_cost(int64_t m, int64_t n, int64_t k, int slab, int rt, int64_t cus) {
+  if ((slab == 128 && rt != 1) || n % (16 * rt) != 0) return INT64_MAX;
+  const int64_t slabs = m <= slab ? 1 : ceil_div(m, slab);
+  const int tt = m <= slab ? (m <= 16 ? 1 : m <= 32 ? 2 : m <= 64 ? 4 : 8) : slab / 16;
+  if (tt == 8 && rt != 1) return INT64_MAX;
+  const int64_t wgs = slabs * (n / (16 * rt));
+  const int64_t chunks = ceil_div(k >> 7, 8);
+  const int64_t per_chunk = (rt + tt) * 145 + rt * tt * 10 + 100;
+  const int64_t wg_time = chunks * per_chunk + rt * tt * 193 + 2493;
+  const int64_t full = wgs / cus, rest = wgs - full * cus;
+  // every round of workgroups streams the weights again, out of the last-level cache at best: 5.6 TB/s
+  // (256 x 14336 x 14336 as 4 slabs in 3.5 rounds: 123 us for 4 x 205 MB)
+  const int64_t stream = ceil_div(wgs, cus) * n * k / 5400;
+  return std::max((full * 100 + (rest ? 70 + 30 * rest / cus : 0)) * wg_time / 100, stream);
+}
+
+// best form of the skinny kernel for more than 32 rows: estimated duration, slab height and weight tiles per workgroup
+int64_t mxfp8_skinny_best(int64_t m, int64_t n, int64_t k, int64_t cus, int* slab_out, int* rt_out) {
+  int slab = 128, rt = 1;
+  int64_t best = INT64_MAX;
+  for (const int s : {32, 64, 128})  // (equal estimates: the lower slab, measured 2-9 % faster)
+    for (const int r : {1, 2, 4}) {
+      const int64_t c = mxfp8_skinny_cost(m, n, k, s, r, cus);
+      if (c < best) best = c, slab = s, rt = r;
+    }
+  if (slab_out) *slab_out = slab;
+  if (rt_out) *rt_out = rt;
+  return best;
+}
+
 template <bool OUT_BF16>
 int launch_skinny(const Params& p, hipStream_t stream) {
-  // Slabs of 128, 64 or 32 rows, all in one launch (blockIdx.y = slab; the last one may be ragged).  With 8
-  // activation tiles only one weight-row tile fits the LDS ring, and every workgroup fetches all activation rows
-  // of its slab: where N supplies enough workgroups of four weight-row tiles, slabs of 64 rows with those are
-  // faster (128 x 14336 x 4096: 30 against 36 us; 128 x 4096 x 4096: 16 against 12).  Otherwise a workgroup
-  // has 16 weight rows, and a small N leaves compute units idle: a round of workgroups costs about 100 / 60 / 47
-  // with slabs of 128 / 64 / 32 rows (measured at K = 2048 and 7168), so lower slabs win where they add no round
-  // (128 x 2048 x 7168: 11.4 -> 8.3 us, 192 x 512 x 7168: 18.2 -> 5.9 us, 512 x 512 x 7168: 13.9 -> 8.8 us).
-  // A ragged last slab either rides along as a whole slab or gets a launch of its own with fewer activation
-  // tiles, whichever the same estimate favours (192 x 8192 x 8192: 58 against 52 us).
-  const int64_t cus = cu_count();
-  const bool wide_n = (p.n & 63) == 0 && p.n / 64 >= cus * 4 / 5;
-  auto single = [&](const Params& q, int rows) {
-    return rows <= 16 ? launch_skinny_tt<1, OUT_BF16>(q, stream)
-         : rows <= 32 ? launch_skinny_tt<2, OUT_BF16>(q, stream)
-         : rows <= 64 ? launch_skinny_tt<4, OUT_BF16>(q, stream)
-                      : launch_skinny_cfg<1, 8, OUT_BF16>(q, stream);
-  };
-  int slab = 64;
-  bool own_launch = false;  // for the ragged last slab
-  if (!wide_n) {
-    auto rounds = [&](int64_t slabs) { return ceil_div(slabs * (int64_t)(p.n / 16), cus); };
-    auto unit = [](int rows) { return rows <= 16 ? 40 : rows <= 32 ? 47 : rows <= 64 ? 60 : 100; };
-    int64_t best = INT64_MAX;
-    for (int s : {128, 64, 32}) {
-      const int whole = p.m / s, rest = p.m % s;
-      const int64_t together = unit(s) * rounds(whole + (rest != 0));
-      const int64_t apart = whole && rest ? unit(s) * rounds(whole) + unit(rest) * rounds(1) : INT64_MAX;
-      if (together < best) best = together, slab = s, own_launch = false;
-      if (apart < best) best = apart, slab = s, own_launch = true;
-    }
-  }
-  if (p.m <= slab) return single(p, p.m);
-  const int slabs = own_launch ? p.m / slab : (int)ceil_div(p.m, slab);
-  const int rc = slab == 128 ? launch_skinny_cfg<1, 8, OUT_BF16>(p, stream, slabs)
-               : slab == 64  ? launch_skinny_tt<4, OUT_BF16>(p, stream, slabs)
-                             : launch_skinny_tt<2, OUT_BF16>(p, stream, slabs);
-  if (rc != NVF_OK || !own_launch) return rc;
-  Params last = p;
-  last.m_base = slabs * slab;
-  return single(last, p.m - last.m_base);
+  // Up to 32 rows: one slab, as many weight rows per workgroup as still leaves about one workgroup per compute unit.
+  if (p.m <= 16) return launch_skinny_tt<1, OUT_BF16>(p, stream);
+  if (p.m <= 32) return launch_skinny_tt<2, OUT_BF16>(p, stream);
+  // More rows: slabs of 128, 64 or 32 rows side by side in one launch (blockIdx.y = slab; the last one may be ragged;
+  // the slabs after the first find the weights in the last-level cache) with 1, 2 or 4 weight tiles per workgroup
+  // (1 with 128-row slabs, whose 8 activation tiles fill the ring), whichever the estimate above prefers
+  // (128 x 4096 x 4096: 10.5 us as one slab of 128 rows, 7.6 us as 4 slabs of 32 rows x 4 weight tiles;
+  // 256 x 4096 x 14336: 49.9 -> 26.1 us; 128 x 8192 x 7168: 28.0 -> 16.6 us).
+  int slab, rt;
+  mxfp8_skinny_best(p.m, p.n, p.k, cu_count(), &slab, &rt);
+  const int slabs = p.m <= slab ? 1 : (int)ceil_div(p.m, slab);
+  const int rows = p.m <= slab ? p.m : slab;
+  return rows <= 32 ? launch_skinny_rt<2, OUT_BF16>(p, rt, stream, slabs)
+       : rows <= 64 ? launch_skinny_rt<4, OUT_BF16>(p, rt, stream, slabs)
+                    : launch_skinny_rt<8, OUT_BF16>(p, rt, stream, slabs);
 }
 
 template <int BM, int BN, bool OUT_BF16>
@@ -776,35 +797,36 @@ int launch_cfg(const Params& p, hipStream_t stream) {
 template <bool OUT_BF16>
 int launch_sized(const Params& p, hipStream_t stream) {
   auto tiles = [&](int bm, int bn) { return ceil_div(p.m, bm) * ceil_div(p.n, bn); };
-  // up to 256 rows, i.e. four passes over the weights (the later ones out of the last-level cache), this beats
-  // the tile kernels below (measured: 128 x 4096 x 14336 in 35 instead of 117 us, 256 x 14336 x 4096 equal).
-  // More rows with a deep K and a small N leave the tile kernels too few tiles for the chip: the skinny
-  // kernel's workgroups (one per 128 rows x 16 columns, K split over their wavefronts) then fill it.  A round
-  // of them costs about a quarter of a round of 128x256 tiles, so up to 3 rounds win or tie (measured, K >= 2048:
-  // 512 x 2048 x 7168 in 27 instead of 59 us, 384 x 3072 x 7168 in 39 instead of 62, 384 x 4096 x 4096 27 both).
   const int64_t cus = cu_count();
-  const int64_t skinny_rounds = ceil_div(ceil_div(p.m, 128) * (int64_t)(p.n / 16), cus);
+  const bool skinny_ok = (p.k & 127) == 0 && (p.n & 15) == 0 && (int64_t)p.k * 64 < (1ll << 31);  // 32-bit lane offsets
   const bool fast_ok = (p.k & 127) == 0 && p.k >= 256 && (p.m & 127) == 0 && (p.n & 255) == 0 && (int64_t)p.k * 256 < (1ll << 31);
-  // Exception: 128 or 256 rows and a wide N.  Per 1024 of K a round of skinny workgroups costs about 1.7 us with
-  // 128-row slabs and 3.4 us with the 64-row slabs of a wide N (which are launches of their own), a round of
-  // 128x256 tiles 6.8 us: where one round of those tiles covers the shape, it wins from about N = 10240 at 256
-  // rows (measured: 256 x 14336 x 4096 in 31 instead of 55 us, 256 x 28672 x 4096 in 34 instead of 104 us).
-  const bool wide_n = (p.n & 63) == 0 && p.n / 64 >= cus * 4 / 5;
-  const int64_t skinny_cost = wide_n ? 34 * ceil_div(p.m, 64) * ceil_div(p.n / 64, cus) : 17 * skinny_rounds;
-  const bool wide_256 = fast_ok && p.m <= 256 && tiles(128, 256) >= 48 && 68 * ceil_div(tiles(128, 256), cus) < skinny_cost;
-  if (!wide_256 && (p.m <= 256 || (skinny_rounds <= 3 && p.k >= 2048)) && (p.k & 127) == 0 && (p.n & 15) == 0 &&
-      (int64_t)p.k * 64 < (1ll << 31))  // 32-bit lane offsets
-    return launch_skinny<OUT_BF16>(p, stream);
-  if (fast_ok) {
-    // Persistent LDS-direct kernel with 256x256 or 128x256 tiles: a 128-row tile costs about 0.61 of a 256-row
-    // tile (half the flops at 82 % of the rate, measured), and the time goes with the rounds of tiles over the
-    // compute units; below 48 tiles the tile kernels further down do as well.
-    const int64_t t256 = (p.m & 255) == 0 ? tiles(256, 256) : 0, t128 = tiles(128, 256);
-    const int64_t cost256 = t256 ? 100 * ceil_div(t256, cus) : INT64_MAX;
-    const int64_t cost128 = 61 * ceil_div(t128, cus);
-    if (t256 >= 128 && cost256 <= cost128) return launch_fast<4, OUT_BF16>(p, stream);
-    if (t128 >= 48) return launch_fast<2, OUT_BF16>(p, stream);
+  // Persistent LDS-direct kernel with 256x256 or 128x256 tiles: a 128-row tile costs about 0.61 of a 256-row tile (half
+  // the flops at 82 % of the rate, measured), and the time goes with the rounds of tiles over the compute units;
+  // below 48 tiles the tile kernels further down do as well.
+  const int64_t t256 = fast_ok && (p.m & 255) == 0 ? tiles(256, 256) : 0, t128 = fast_ok ? tiles(128, 256) : 0;
+  const int64_t cost256 = t256 >= 128 ? 100 * ceil_div(t256, cus) : INT64_MAX;
+  const int64_t cost128 = t128 >= 48 ? 61 * ceil_div(t128, cus) : INT64_MAX;
+  const bool fast = cost256 != INT64_MAX || cost128 != INT64_MAX;
+  if (skinny_ok) {
+    if (p.m <= 32) return launch_skinny<OUT_BF16>(p, stream);
+    if (fast) {
+      // Skinny or persistent kernel by estimated duration: a round of 128x256 tiles takes 6.9 us per 1024 of K plus
+      // about 5 us (so cost 100 = 11.3 us per 1024 of K), the skinny kernel what its estimate says (its unit is
+      // 0.96 ns).  Measured: 256 x 14336 x 4096 31 (persistent) against 47 us, 512 x 4096 x 7168 51 against 30 us
+      // (skinny), 1024 x 2048 x 14336 97 against 48 us, 1024 x 4096 x 4096 31 against 34 us.
+      const int64_t fast_ns = 5000 + std::min(cost256, cost128) * 113 * (int64_t)p.k / 1024;
+      const int64_t skinny_ns = mxfp8_skinny_best(p.m, p.n, p.k, cus, nullptr, nullptr) * 963 / 1000;
+      if (skinny_ns <= fast_ns) return launch_skinny<OUT_BF16>(p, stream);
+    } else {
+      // No persistent kernel for the shape (ragged M or N, or too few tiles): up to 256 rows, i.e. four passes over
+      // the weights, the skinny kernel beats the tile kernels below (128 x 4096 x 14336: 20 instead of 117 us); with
+      // more rows, a deep K and a small N it fills the chip where they cannot, while its 128-row x 16-column
+      // workgroups cover the compute units at most 3 times (measured, K >= 2048).
+      const int64_t skinny_rounds = ceil_div(ceil_div(p.m, 128) * (int64_t)(p.n / 16), cus);
+      if (p.m <= 256 || (skinny_rounds <= 3 && p.k >= 2048)) return launch_skinny<OUT_BF16>(p, stream);
+    }
   }
+  if (fast) return cost256 <= cost128 ? launch_fast<4, OUT_BF16>(p, stream) : launch_fast<2, OUT_BF16>(p, stream);
   if (tiles(256, 256) >= cus) return launch_cfg<256, 256, OUT_BF16>(p, stream);
   if (tiles(128, 128) >= cus) return launch_cfg<128, 128, OUT_BF16>(p, stream);
   return launch_cfg<64, 64, OUT_BF16>(p, stream);

@@ -53,6 +53,25 @@ def test_config3_deep_k_with_a_workspace_splits_k():
     assert plan("nvfp4_scaled_mm", 128, 1024, 8192, ws=need).startswith("nvfp4_tile_kernel<128,128,split_k>")
 
 
+@pytest.mark.parametrize("m,n,k,kernel", [
+    (16, 4096, 4096, "mxfp8_skinny_kernel<RT=1,TT=1> grid=256x1"),
+    (128, 4096, 4096, "mxfp8_skinny_kernel<RT=4,TT=2> grid=64x4"),
+    (128, 14336, 4096, "mxfp8_skinny_kernel<RT=4,TT=4> grid=224x2"),
+    (128, 4096, 14336, "mxfp8_skinny_kernel<RT=4,TT=2> grid=64x4"),
+    (2048, 4096, 4096, "mxfp8_gemm_256_kernel<TM=2,stream_out=0> grid=256"),
+    (2048, 14336, 4096, "mxfp8_gemm_256_kernel<TM=4,stream_out=0> grid=256"),
+    # streaming or persistent kernel by estimated duration
+    (256, 14336, 4096, "mxfp8_gemm_256_kernel<TM=2,stream_out=0> grid=112"),
+    (256, 14336, 14336, "mxfp8_gemm_256_kernel<TM=2,stream_out=0> grid=112"),
+    (512, 4096, 7168, "mxfp8_skinny_kernel<RT=4,TT=4> grid=64x8"),
+    (1024, 2048, 14336, "mxfp8_skinny_kernel<RT=4,TT=4> grid=32x16"),
+    (1024, 4096, 4096, "mxfp8_gemm_256_kernel<TM=2,stream_out=0> grid=128"),
+    (1024, 8192, 4096, "mxfp8_gemm_256_kernel<TM=2,stream_out=0> grid=256"),
+])
+def test_mxfp8_llm_and_mid_sized_shapes(m, n, k, kernel):
+    assert plan("mxfp8_scaled_mm", m, n, k).startswith(kernel), plan("mxfp8_scaled_mm", m, n, k)
+
+
 def test_nvfp4_8192_cubed_takes_the_persistent_256x256_kernel():
     assert plan("nvfp4_scaled_mm", 8192, 8192, 8192).startswith("nvfp4_gemm_256_kernel<grouped=0,TM=4,f32=0,pairs=1> grid=256")
 

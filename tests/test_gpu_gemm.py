@@ -468,8 +468,8 @@ def test_nvfp4_gemm_persistent_kernel_every_scale_code_is_decoded_exactly(dev, s
                                    (256, 160, 512), (129, 32, 128), (100, 13056, 128), (192, 512, 2048), (100, 1024, 256),
                                    (250, 2048, 384), (150, 1024, 640), (128, 13120, 256)])
 def test_mxfp8_gemm_decode_sized_activations(dev, shape):
-    """M <= 256 (in one launch of slabs of 128, 64 or 32 rows, the last one ragged: 64 where N is wide, else the height that
-    fills the compute units best) with K % 128 == 0 and N % 16 == 0 takes the kernel that streams the weights once through
+    """M <= 256 (in one launch of slabs of 128, 64 or 32 rows, the last one ragged; height and weight tiles per workgroup
+    by a cost estimate) with K % 128 == 0 and N % 16 == 0 takes the kernel that streams the weights once through
     per-wavefront LDS rings into v_mfma_scale_f32_16x16x128_f8f6f4: 1 / 2 / 4 / 8 activation tiles, 1 / 2 / 4
     weight-row tiles per workgroup (rings of 3, 2 and 1 slots), activation rows that do not fill a tile,
     all four scale row groups, 1 to 8 chunks per wavefront (wavefronts without work, ring wrap), scales
@@ -491,14 +491,42 @@ def test_mxfp8_gemm_decode_sized_activations(dev, shape):
         assert torch.equal(out, _run_mxfp8(a, b, sa_p, sb, 0.75, dtype, dev))
 
 
+@pytest.mark.parametrize("nk", [(1024, 2048), (2048, 4096), (4096, 2048), (6144, 2176), (4096, 7168), (8192, 1152), (14336, 640),
+                                (528, 2176), (2080, 1152), (1040, 4096)])
+def test_mxfp8_gemm_slab_height_and_weight_tiles_by_cost(dev, nk):
+    """33..256 rows (and more, while the estimate prefers it to the persistent kernel): the weight-streaming kernel runs
+    as slabs of 128, 64 or 32 rows with 1, 2 or 4 weight tiles per workgroup, picked by a cost estimate.  Row counts on
+    both sides of the slab heights (ragged last slabs), shapes that select each form; every element compared, both
+    output types, run-to-run bit equality."""
+    from fuser_amd import capi
+
+    n, k = nk
+    gen = torch.Generator().manual_seed(n + k)
+    b, sb = _mxfp8_operand(n, k, gen, 1.0)
+    forms = set()
+    for m in (33, 48, 64, 65, 96, 100, 128, 129, 192, 200, 256, 384, 520):
+        plan = capi.describe_dispatch("mxfp8_scaled_mm", m, n, k)
+        forms.add(plan.split(" ")[0])
+        a, sa = _mxfp8_operand(m, k, gen, 1.0)
+        ref = O.ref_mxfp8_scaled_mm(a, b, sa, sb, 0.75)
+        scale = ref.abs().amax(dim=1, keepdim=True).clamp(min=1e-30)
+        for dtype in (torch.bfloat16, torch.float16):
+            if dtype == torch.float16 and ref.abs().max() > 6e4:
+                continue
+            out = _run_mxfp8(a, b, sa, sb, 0.75, dtype, dev)
+            assert out.shape == (m, n)
+            assert ((out.float().cpu() - ref).abs() / scale).max().item() <= GEMM_MAX_REL, (m, n, k, dtype, plan)
+            assert torch.equal(out, _run_mxfp8(a, b, sa, sb, 0.75, dtype, dev))
+    assert any(f.startswith("mxfp8_skinny_kernel<") for f in forms), forms
+
+
 @pytest.mark.parametrize("shape", [(300, 2048, 2048), (512, 1536, 2304), (384, 3072, 2048), (640, 528, 2176), (1000, 272, 2560),
                                    (257, 16, 2048), (1024, 768, 2048), (2100, 96, 4096)])
 def test_mxfp8_gemm_many_rows_small_n_deep_k(dev, shape):
     """More than 256 rows with K >= 2048 and an N small enough that the workgroups of the kernel for decode-sized
-    activations (one per 128 rows x 16 columns) cover the compute units at most three times: all whole 128-row
-    slabs go in one launch (2 to 16 slabs), the remaining rows (44, 104, 1, 52 or none) in a launch of their
-    own with 1 / 4 / 8 activation tiles.  Every output element is compared with the oracle, with poisoned scale
-    padding, both output types and run-to-run determinism."""
+    activations (one per 128 rows x 16 columns) cover the compute units at most three times: all slabs go in one
+    launch (3 to 66 slabs of 128, 64 or 32 rows), the last one ragged (44, 104, 1, 52 rows or whole).  Every output
+    element is compared with the oracle, with poisoned scale padding, both output types and run-to-run determinism."""
     m, n, k = shape
     gen = torch.Generator().manual_seed(m * 31 + n)
     a, sa = _mxfp8_operand(m, k, gen, 1.0)
