@@ -2144,6 +2144,20 @@ int64_t nvfp4_skinny_cost(int64_t m, int64_t n, int64_t k, int slab, int rt, int
   return rounds * wg_time;
 }
 
+// best (slab height, weight tiles per workgroup) for more than 32 rows and its estimated cost
+int64_t nvfp4_skinny_best(int64_t m, int64_t n, int64_t k, int cus, int* slab_out, int* rt_out) {
+  int slab = 128, rt = 1;
+  int64_t best = INT64_MAX;
+  for (const int s : {128, 64, 32})
+    for (const int r : {4, 2, 1}) {
+      const int64_t c = nvfp4_skinny_cost(m, n, k, s, r, cus);
+      if (c < best) best = c, slab = s, rt = r;
+    }
+  if (slab_out) *slab_out = slab;
+  if (rt_out) *rt_out = rt;
+  return best;
+}
+
 template <bool OUT_BF16>
 int launch_nvfp4_skinny(const Params& p, int cus, hipStream_t stream) {
   // Up to 32 rows: one slab, as many weight rows per workgroup as still leaves about one workgroup per compute unit
@@ -2153,13 +2167,8 @@ int launch_nvfp4_skinny(const Params& p, int cus, hipStream_t stream) {
   // the slabs after the first find the weights in the last-level cache) with 1, 2 or 4 weight tiles per workgroup,
   // whichever the cost estimate above prefers (M=128, N=4096, K=4096: 10.8 us as two slabs of 64 rows x 1 weight tile,
   // 8.3 us x 2 tiles; M=256, N=4096, K=14336: 62 -> 34 us; M=256, N=6144, K=7168: 48 -> 29 us).
-  int slab = 128, rt = 1;
-  int64_t best = INT64_MAX;
-  for (const int s : {128, 64, 32})
-    for (const int r : {4, 2, 1}) {
-      const int64_t c = nvfp4_skinny_cost(p.m, p.n, p.k, s, r, cus);
-      if (c < best) best = c, slab = s, rt = r;
-    }
+  int slab, rt;
+  nvfp4_skinny_best(p.m, p.n, p.k, cus, &slab, &rt);
   if (p.m > slab) {
     const int slabs = (int)ceil_div(p.m, slab);
     return slab == 128 ? launch_nvfp4_skinny_rt<8, OUT_BF16>(p, rt, stream, slabs)
@@ -2575,25 +2584,43 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int6
       if (splits > 1 && workspace_bytes >= (int64_t)splits * p.m * p.n * 4)
         return launch_nvfp4_splitk<OUT_BF16>(p, splits, static_cast<float*>(workspace), stream);
     }
-    // up to 256 rows (two passes over the weights) this beats the tile kernel (measured: 256 x 14336 x 4096 in
-    // 46 instead of 65 us; at 512 rows the tile kernel wins)
-    // More rows with a deep K and a small N leave the kernels below too few tiles for the chip (without a
-    // workspace there is no split of K); the skinny kernel splits K over a workgroup's wavefronts, and its
-    // workgroups (one per 128 rows x 16 columns at such N) win or tie while they cover the compute units at most
-    // 3 times, 2 times for K < 4096 (measured: 512 x 2048 x 7168 in 34 instead of 45 us, 384 x 3072 x 7168 in
-    // 49 instead of 59, 1024 x 1536 x 7168 in 50 instead of 59, 300 x 3072 x 2048 in 18 instead of 16).
-    const int64_t skinny_rounds = ceil_div(ceil_div(p.m, 128) * (int64_t)(p.n / 16), cus);
-    if (dense && (p.m <= 256 || (p.k >= 2048 && skinny_rounds <= (p.k >= 4096 ? 3 : 2))) && (p.k & 127) == 0 && (p.n & 15) == 0 &&
-        (int64_t)p.k * 64 < (1ll << 31))  // 32-bit lane offsets
-      return launch_nvfp4_skinny<OUT_BF16>(p, cus, stream);
-    if (dense && (p.m & 127) == 0 && (p.n & 255) == 0 && (p.k & 127) == 0 && p.k >= 256) {
-      // Persistent kernel with 256x256 or 128x256 tiles, or the tile kernel below?  Costs in units of one round
-      // of 256x256 tiles over the compute units = 100: a 128-row tile costs 58 (half the flops at 86 % of the
-      // rate), and the tile kernel, which has no rounds to speak of, runs at about 70 % of the rate (all measured).
+    // Dense: the weight-streaming kernel, the persistent kernel with 256x256 or 128x256 tiles, or the tile kernels
+    // below?  Costs in units of one round of 256x256 tiles over the compute units = 100 (24 us per 1024 of K): a
+    // round of 128-row tiles costs 58 (half the flops at 86 % of the rate); the tile kernels run their 128x128 tiles
+    // two to a compute unit: 68 per such round, 45 for a last round of one tile per compute unit, and 22..47 when
+    // there is no more than that in all (all measured: M = 128..1024, N = 2048..14336, K = 4096 and 14336).
+    const bool skinny_ok = dense && (p.k & 127) == 0 && (p.n & 15) == 0 && (int64_t)p.k * 64 < (1ll << 31);  // 32-bit lane offsets
+    const bool persistent_ok = dense && (p.m & 127) == 0 && (p.n & 255) == 0 && (p.k & 127) == 0 && p.k >= 256;
+    int64_t cost256 = INT64_MAX, cost128 = INT64_MAX, cost_tile = INT64_MAX;
+    if (persistent_ok) {
       const int64_t t256 = (p.m & 255) == 0 ? tiles(256, 256) : 0, t128 = tiles(128, 256);
-      const int64_t cost256 = t256 ? 100 * ceil_div(t256, cus) : INT64_MAX;
-      const int64_t cost128 = 58 * ceil_div(t128, cus);
-      const int64_t cost_tile = 144 * t128 / (2 * cus);
+      cost256 = t256 ? 100 * ceil_div(t256, cus) : INT64_MAX;
+      cost128 = 58 * ceil_div(t128, cus);
+      const int64_t small = 2 * t128, full = small / (2 * cus), rest = small - full * 2 * cus;
+      cost_tile = full * 68 + (rest == 0 ? 0 : rest > cus ? 68 : full ? 45 : 22 + 25 * rest / cus);
+    }
+    if (skinny_ok) {
+      bool skinny;
+      if (p.m <= 256) {
+        skinny = true;  // at most two passes over the weights (256 x 14336 x 4096: 38 instead of 58 us on tiles)
+      } else if (persistent_ok && p.k >= 2048) {
+        // by estimated duration; the streaming kernel's estimate is in ns within 0.8 (K = 2048) .. 1.1 (K = 14336)
+        // (measured: 512 x 4096 x 14336 115 -> 57 us, 384 x 8192 x 7168 82 -> 57 us, 640 x 14336 x 14336 381 -> 268 us;
+        // 1024 x 8192 x 4096 stays on 128x256 tiles: 64 against 76 us)
+        const int64_t rest_ns = 6000 + std::min(cost256, std::min(cost128, cost_tile)) * 240 * (int64_t)p.k / 1024;
+        const int64_t skinny_ns = nvfp4_skinny_best(p.m, p.n, p.k, cus, nullptr, nullptr) * (p.k < 3072 ? 82 : p.k < 6144 ? 96 : p.k < 10240 ? 103 : 110) / 100;
+        skinny = skinny_ns <= rest_ns;
+      } else {
+        // Ragged shapes, which only the tile kernels below take otherwise: with a deep K and a small N the
+        // streaming kernel fills the chip where they cannot, while its workgroups (one per 128 rows x 16 columns at
+        // such N) cover the compute units at most 3 times, 2 times for K < 4096 (measured: 300 x 3072 x 2048 in 18
+        // instead of 16 us, 1000 x 288 x 2560, 2100 x 96 x 4096).
+        const int64_t skinny_rounds = ceil_div(ceil_div(p.m, 128) * (int64_t)(p.n / 16), cus);
+        skinny = p.k >= 2048 && skinny_rounds <= (p.k >= 4096 ? 3 : 2);
+      }
+      if (skinny) return launch_nvfp4_skinny<OUT_BF16>(p, cus, stream);
+    }
+    if (persistent_ok) {
       if (cost256 <= cost128 && cost256 <= cost_tile) return launch_nvfp4_fast<OUT_BF16, false, 4>(p, cus, stream);
       if (cost128 <= cost_tile) return launch_nvfp4_fast<OUT_BF16, false, 2>(p, cus, stream);
     }

@@ -72,6 +72,21 @@ def test_mxfp8_llm_and_mid_sized_shapes(m, n, k, kernel):
     assert plan("mxfp8_scaled_mm", m, n, k).startswith(kernel), plan("mxfp8_scaled_mm", m, n, k)
 
 
+@pytest.mark.parametrize("m,n,k,kernel", [
+    # streaming, persistent (256x256 / 128x256 tiles) or tile kernel by estimated duration
+    (512, 4096, 4096, "nvfp4_skinny_ring_kernel<RT=4,TT=8> grid=64x4"),
+    (1024, 2048, 4096, "nvfp4_skinny_ring_kernel<RT=4,TT=8> grid=32x8"),
+    (640, 8192, 4096, "nvfp4_skinny_ring_kernel<RT=4,TT=8> grid=128x5"),
+    (1024, 4096, 14336, "nvfp4_skinny_ring_kernel<RT=4,TT=8> grid=64x8"),
+    (256, 14336, 4096, "nvfp4_skinny_ring_kernel<RT=4,TT=8> grid=224x2"),
+    (1024, 8192, 4096, "nvfp4_gemm_256_kernel<grouped=0,TM=2,f32=0,pairs=1> grid=256"),
+    (512, 14336, 4096, "nvfp4_gemm_256_kernel<grouped=0,TM=2,f32=0,pairs=1> grid=224"),
+    (768, 14336, 4096, "nvfp4_gemm_256_kernel<grouped=0,TM=4,f32=0,pairs=1> grid=168"),
+])
+def test_nvfp4_mid_sized_shapes(m, n, k, kernel):
+    assert plan("nvfp4_scaled_mm", m, n, k).startswith(kernel), plan("nvfp4_scaled_mm", m, n, k)
+
+
 def test_nvfp4_8192_cubed_takes_the_persistent_256x256_kernel():
     assert plan("nvfp4_scaled_mm", 8192, 8192, 8192).startswith("nvfp4_gemm_256_kernel<grouped=0,TM=4,f32=0,pairs=1> grid=256")
 

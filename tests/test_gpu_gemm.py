@@ -264,7 +264,8 @@ def test_nvfp4_gemm_slab_height_and_weight_tiles_by_cost(dev, nk):
 
 
 @pytest.mark.parametrize("shape", [(300, 2048, 2048), (512, 1536, 2304), (384, 3072, 4096), (640, 544, 2176), (1000, 288, 2560),
-                                   (257, 32, 2048), (1024, 768, 2048), (2100, 96, 4096)])
+                                   (257, 32, 2048), (1024, 768, 2048), (2100, 96, 4096), (512, 4096, 4096), (640, 2048, 2048),
+                                   (1024, 2048, 4096), (384, 8192, 2048), (640, 8192, 2176)])
 def test_nvfp4_gemm_many_rows_small_n_deep_k(dev, shape):
     """More than 256 rows with K >= 2048 and an N small enough that the workgroups of the kernel for decode-sized
     activations (one per 128 rows x 16 columns) cover the compute units at most two or three times: all slabs
