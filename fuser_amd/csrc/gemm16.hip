@@ -2506,6 +2506,53 @@ int launch_nvfp4_tile(const Params& p, int grid, hipStream_t stream) {
   return check_launch("nvfp4_tile_kernel");
 }
 
+// Dense NVFP4 without a workspace: the weight-streaming kernel, the persistent kernel with 256x256 or 128x256 tiles,
+// or the tile kernels?  Costs in units of one round of 256x256 tiles over the compute units = 100 (24 us per 1024 of
+// K): a round of 128-row tiles costs 58 (half the flops at 86 % of the rate); the tile kernels run their 128x128 tiles
+// two to a compute unit: 68 per such round, 45 for a last round of one tile per compute unit, and 22..47 when there
+// is no more than that in all (all measured: M = 128..1024, N = 2048..14336, K = 4096 and 14336).
+struct DensePlan {
+  enum Kernel { kStream, kTiles256, kTiles128, kOther } kernel;
+};
+DensePlan nvfp4_dense_plan(int64_t m, int64_t n, int64_t k, int cus) {
+  const bool stream_ok = (k & 127) == 0 && (n & 15) == 0 && k * 64 < (1ll << 31);  // 32-bit lane offsets
+  const bool persistent_ok = (m & 127) == 0 && (n & 255) == 0 && (k & 127) == 0 && k >= 256;
+  int64_t cost256 = INT64_MAX, cost128 = INT64_MAX, cost_tile = INT64_MAX;
+  if (persistent_ok) {
+    const int64_t t256 = (m & 255) == 0 ? (m / 256) * (n / 256) : 0, t128 = (m / 128) * (n / 256);
+    cost256 = t256 ? 100 * ceil_div(t256, cus) : INT64_MAX;
+    cost128 = 58 * ceil_div(t128, cus);
+    const int64_t small = 2 * t128, full = small / (2 * cus), rest = small - full * 2 * cus;
+    cost_tile = full * 68 + (rest == 0 ? 0 : rest > cus ? 68 : full ? 45 : 22 + 25 * rest / cus);
+  }
+  if (stream_ok) {
+    bool stream;
+    if (m <= 256) {
+      stream = true;  // at most two passes over the weights (256 x 14336 x 4096: 38 instead of 58 us on tiles)
+    } else if (persistent_ok && k >= 2048) {
+      // by estimated duration; the streaming kernel's estimate is in ns within 0.8 (K = 2048) .. 1.1 (K = 14336)
+      // (measured: 512 x 4096 x 14336 115 -> 57 us, 384 x 8192 x 7168 82 -> 57 us, 640 x 14336 x 14336 381 -> 268 us;
+      // 1024 x 8192 x 4096 stays on 128x256 tiles: 64 against 76 us)
+      const int64_t rest_ns = 6000 + std::min(cost256, std::min(cost128, cost_tile)) * 240 * k / 1024;
+      const int64_t stream_ns = nvfp4_skinny_best(m, n, k, cus, nullptr, nullptr) * (k < 3072 ? 82 : k < 6144 ? 96 : k < 10240 ? 103 : 110) / 100;
+      stream = stream_ns <= rest_ns;
+    } else {
+      // Ragged shapes, which only the tile kernels take otherwise: with a deep K and a small N the streaming kernel
+      // fills the chip where they cannot, while its workgroups (one per 128 rows x 16 columns at such N) cover the
+      // compute units at most 3 times, 2 times for K < 4096 (measured: 300 x 3072 x 2048 in 18 instead of 16 us,
+      // 1000 x 288 x 2560, 2100 x 96 x 4096).
+      const int64_t rounds = ceil_div(ceil_div(m, 128) * (n / 16), cus);
+      stream = k >= 2048 && rounds <= (k >= 4096 ? 3 : 2);
+    }
+    if (stream) return {DensePlan::kStream};
+  }
+  if (persistent_ok) {
+    if (cost256 <= cost128 && cost256 <= cost_tile) return {DensePlan::kTiles256};
+    if (cost128 <= cost_tile) return {DensePlan::kTiles128};
+  }
+  return {DensePlan::kOther};
+}
+
 // Split of K for dense NVFP4 shapes with fewer 128x128 tiles than compute units and a deep K (decode and
 // small prefill batches against a down projection): about two work items per compute unit, at least eight
 // 128-deep spans each.  Every split writes and the reduction re-reads an fp32 copy of the output, so for
@@ -2513,23 +2560,28 @@ int launch_nvfp4_tile(const Params& p, int grid, hipStream_t stream) {
 int nvfp4_splits(int64_t m, int64_t n, int64_t k, int cus) {
   const int64_t tiles = ceil_div(m, 128) * ceil_div(n, 128), nspans = ceil_div(k, 128);
   if (m <= 64 || tiles >= cus || nspans < 64) return 1;
+  // not where the weight-streaming kernel runs, which splits K over the wavefronts of a workgroup (256 x 2048 x 8192:
+  // 14 us against 28 us for this split; 512 x 4096 x 14336: 56 against 78 us)
+  if (nvfp4_dense_plan(m, n, k, cus).kernel == DensePlan::kStream) return 1;
   int64_t s = (2 * (int64_t)cus) / tiles;
   if (s > nspans / 8) s = nspans / 8;
   if (s > 32) s = 32;
   return s < 2 ? 1 : (int)s;
 }
 
-// Split of K over workgroups for the weight-streaming kernel with one slab of 65..128 activation rows: every
+// Split of K over workgroups for the weight-streaming kernel with one slab of 65..96 activation rows: every
 // workgroup converts all activation rows of its K range next to its weight rows, so 64 weight rows per workgroup
 // (4 tiles against 8 activation tiles: 12 conversions for 32 MFMA tiles) halve the conversion work of 16 (1 against
 // 8: 9 for 8), and where N / 64 workgroups leave compute units idle, K is split over as many workgroups as fit.
 int nvfp4_skinny_splits(int64_t m, int64_t n, int64_t k, int cus) {
-  if (m <= 64 || m > 128 || (k & 127) != 0 || (n & 63) != 0 || k * 64 >= (1ll << 31)) return 1;
+  // (measured against the forms without a split: 65 x 4096 x 14336 18.7 against 21.7 us, 96 x 8192 x 14336 30.9
+  // against 33.2, 65 x 6144 x 8192 17.7 against 19.1; from 97 rows on, or with a weight matrix of less than 48 Mi
+  // elements, the second launch costs more than the split gains: 128 x 8192 x 14336 38.1 against 35.3, 65 x 4096 x 8192
+  // 16.3 against 13.9, 65 x 2048 x 14336 15.5 against 14.0)
+  if (m <= 64 || m > 96 || (k & 127) != 0 || (n & 63) != 0 || k * 64 >= (1ll << 31) || n * k < (48ll << 20)) return 1;
   const int64_t wgs = n / 64, chunks = k >> 7;
   int64_t s = cus / wgs;
-  // at least three chunks per wavefront: with one (M=128, N=4096, K=4096 as 4 splits) the launch takes 16.4 us against
-  // 12.3 us without a split; with 3.5 (K=14336) 25.2 us against 35.7 us on the tile kernel's split
-  if (s > chunks / 24) s = chunks / 24;
+  if (s > chunks / 28) s = chunks / 28;
   if (s > 8) s = 8;
   if (wgs * s * 2 < cus) return 1;  // would leave most compute units idle: the tile kernel's split has more items
   return s < 2 ? 1 : (int)s;
@@ -2584,45 +2636,11 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int6
       if (splits > 1 && workspace_bytes >= (int64_t)splits * p.m * p.n * 4)
         return launch_nvfp4_splitk<OUT_BF16>(p, splits, static_cast<float*>(workspace), stream);
     }
-    // Dense: the weight-streaming kernel, the persistent kernel with 256x256 or 128x256 tiles, or the tile kernels
-    // below?  Costs in units of one round of 256x256 tiles over the compute units = 100 (24 us per 1024 of K): a
-    // round of 128-row tiles costs 58 (half the flops at 86 % of the rate); the tile kernels run their 128x128 tiles
-    // two to a compute unit: 68 per such round, 45 for a last round of one tile per compute unit, and 22..47 when
-    // there is no more than that in all (all measured: M = 128..1024, N = 2048..14336, K = 4096 and 14336).
-    const bool skinny_ok = dense && (p.k & 127) == 0 && (p.n & 15) == 0 && (int64_t)p.k * 64 < (1ll << 31);  // 32-bit lane offsets
-    const bool persistent_ok = dense && (p.m & 127) == 0 && (p.n & 255) == 0 && (p.k & 127) == 0 && p.k >= 256;
-    int64_t cost256 = INT64_MAX, cost128 = INT64_MAX, cost_tile = INT64_MAX;
-    if (persistent_ok) {
-      const int64_t t256 = (p.m & 255) == 0 ? tiles(256, 256) : 0, t128 = tiles(128, 256);
-      cost256 = t256 ? 100 * ceil_div(t256, cus) : INT64_MAX;
-      cost128 = 58 * ceil_div(t128, cus);
-      const int64_t small = 2 * t128, full = small / (2 * cus), rest = small - full * 2 * cus;
-      cost_tile = full * 68 + (rest == 0 ? 0 : rest > cus ? 68 : full ? 45 : 22 + 25 * rest / cus);
-    }
-    if (skinny_ok) {
-      bool skinny;
-      if (p.m <= 256) {
-        skinny = true;  // at most two passes over the weights (256 x 14336 x 4096: 38 instead of 58 us on tiles)
-      } else if (persistent_ok && p.k >= 2048) {
-        // by estimated duration; the streaming kernel's estimate is in ns within 0.8 (K = 2048) .. 1.1 (K = 14336)
-        // (measured: 512 x 4096 x 14336 115 -> 57 us, 384 x 8192 x 7168 82 -> 57 us, 640 x 14336 x 14336 381 -> 268 us;
-        // 1024 x 8192 x 4096 stays on 128x256 tiles: 64 against 76 us)
-        const int64_t rest_ns = 6000 + std::min(cost256, std::min(cost128, cost_tile)) * 240 * (int64_t)p.k / 1024;
-        const int64_t skinny_ns = nvfp4_skinny_best(p.m, p.n, p.k, cus, nullptr, nullptr) * (p.k < 3072 ? 82 : p.k < 6144 ? 96 : p.k < 10240 ? 103 : 110) / 100;
-        skinny = skinny_ns <= rest_ns;
-      } else {
-        // Ragged shapes, which only the tile kernels below take otherwise: with a deep K and a small N the
-        // streaming kernel fills the chip where they cannot, while its workgroups (one per 128 rows x 16 columns at
-        // such N) cover the compute units at most 3 times, 2 times for K < 4096 (measured: 300 x 3072 x 2048 in 18
-        // instead of 16 us, 1000 x 288 x 2560, 2100 x 96 x 4096).
-        const int64_t skinny_rounds = ceil_div(ceil_div(p.m, 128) * (int64_t)(p.n / 16), cus);
-        skinny = p.k >= 2048 && skinny_rounds <= (p.k >= 4096 ? 3 : 2);
-      }
-      if (skinny) return launch_nvfp4_skinny<OUT_BF16>(p, cus, stream);
-    }
-    if (persistent_ok) {
-      if (cost256 <= cost128 && cost256 <= cost_tile) return launch_nvfp4_fast<OUT_BF16, false, 4>(p, cus, stream);
-      if (cost128 <= cost_tile) return launch_nvfp4_fast<OUT_BF16, false, 2>(p, cus, stream);
+    if (dense) {
+      const DensePlan plan = nvfp4_dense_plan(p.m, p.n, p.k, cus);
+      if (plan.kernel == DensePlan::kStream) return launch_nvfp4_skinny<OUT_BF16>(p, cus, stream);
+      if (plan.kernel == DensePlan::kTiles256) return launch_nvfp4_fast<OUT_BF16, false, 4>(p, cus, stream);
+      if (plan.kernel == DensePlan::kTiles128) return launch_nvfp4_fast<OUT_BF16, false, 2>(p, cus, stream);
     }
   }
   if constexpr (!NVFP4) {

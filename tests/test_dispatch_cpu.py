@@ -37,20 +37,25 @@ def test_config3_llm_shapes(m, n, k, kernel):
     assert got.startswith(kernel) and ";" not in got, got
 
 
-def test_config3_deep_k_with_a_workspace_splits_k():
-    need = capi.lib().nvf_nvfp4_scaled_mm_workspace_bytes(128, 4096, 14336)
-    assert need > 0
-    # one slab of 65..128 rows against N / 64 < compute units: the weight-streaming kernel, K split over 4 workgroups
-    got = plan("nvfp4_scaled_mm", 128, 4096, 14336, ws=need)
+def test_deep_k_with_a_workspace_splits_k_only_where_it_wins():
+    lib = capi.lib()
+    # config 3, M=128: the forms of the weight-streaming kernel without a split are as fast: no workspace asked for
+    assert lib.nvf_nvfp4_scaled_mm_workspace_bytes(128, 4096, 14336) == 0
+    assert lib.nvf_nvfp4_scaled_mm_workspace_bytes(128, 4096, 4096) == 0
+    # one slab of 65..96 rows against N / 64 < compute units and 28+ chunks per split: K split over workgroups
+    need = lib.nvf_nvfp4_scaled_mm_workspace_bytes(96, 4096, 14336)
+    assert need == 4 * 96 * 4096 * 4
+    got = plan("nvfp4_scaled_mm", 96, 4096, 14336, ws=need)
     assert got == "nvfp4_skinny_ring_kernel<RT=4,TT=8> grid=64x1x4 split_k + splitk_reduce_kernel", got
-    assert need == 4 * 128 * 4096 * 4
-    got = plan("nvfp4_scaled_mm", 128, 4096, 14336, ws=need - 1)
+    got = plan("nvfp4_scaled_mm", 96, 4096, 14336, ws=need - 1)
     assert got.startswith("nvfp4_skinny_ring_kernel<") and "split_k" not in got, got
-    # a shallower K is not split (one chunk per wavefront costs more than the idle compute units)
-    assert capi.lib().nvf_nvfp4_scaled_mm_workspace_bytes(128, 4096, 4096) == 0
-    # few weight rows and a deep K: the tile kernel's split has more work items
-    need = capi.lib().nvf_nvfp4_scaled_mm_workspace_bytes(128, 1024, 8192)
-    assert plan("nvfp4_scaled_mm", 128, 1024, 8192, ws=need).startswith("nvfp4_tile_kernel<128,128,split_k>")
+    assert lib.nvf_nvfp4_scaled_mm_workspace_bytes(96, 4096, 4096) == 0
+    # few tiles and a deep K: the streaming kernel where it runs (K % 128 == 0), else the tile kernel's split
+    assert lib.nvf_nvfp4_scaled_mm_workspace_bytes(128, 1024, 8192) == 0
+    assert plan("nvfp4_scaled_mm", 128, 1024, 8192).startswith("nvfp4_skinny_ring_kernel<")
+    need = lib.nvf_nvfp4_scaled_mm_workspace_bytes(128, 1024, 8224)
+    assert need == 8 * 128 * 1024 * 4
+    assert plan("nvfp4_scaled_mm", 128, 1024, 8224, ws=need).startswith("nvfp4_tile_kernel<128,128,split_k>")
 
 
 @pytest.mark.parametrize("m,n,k,kernel", [

@@ -286,21 +286,20 @@ def test_nvfp4_gemm_many_rows_small_n_deep_k(dev, shape):
         assert torch.equal(out, _run_nvfp4(a, b, sa_p, sb, alpha, dtype, dev))
 
 
-@pytest.mark.parametrize("shape", [(128, 1024, 8192), (100, 256, 8224), (200, 512, 10240), (65, 160, 9216), (300, 2048, 14336),
-                                   (100, 4096, 6272), (128, 3072, 9216), (81, 8192, 6144), (65, 4096, 14336)])
+@pytest.mark.parametrize("shape", [(128, 1024, 8224), (100, 256, 8224), (200, 512, 10272), (65, 160, 9248), (300, 2048, 14368),
+                                   (80, 6144, 8192), (70, 8192, 7168), (72, 4736, 10752), (65, 4096, 14336)])
 def test_nvfp4_gemm_split_k_with_workspace(dev, shape):
-    """Few 128x128 output tiles and a deep K: with the scratch memory that
-    nvf_nvfp4_scaled_mm_workspace_bytes asks for, K is split over workgroups and fp32 partial tiles are
-    added in a fixed order.  Ragged M / N / K (K not a multiple of the 128-deep span, splits that do not
-    divide the spans), both output types, against the oracle; run-to-run bit equality; a workspace that is
-    too small, NULL or misaligned falls back to the kernels without one.  The last four shapes (one slab of 65..128
-    rows, N / 64 workgroups covering half the chip or less, K % 128 == 0) split K over workgroups of the
-    weight-streaming kernel instead of the tile kernel: 2, 4 and 3 splits, with 49, 72, 48 and 112 chunks (uneven
-    shares), five to eight activation row tiles."""
+    """Few 128x128 output tiles and a deep K that the weight-streaming kernel cannot take (K % 128 != 0): with the
+    scratch memory that nvf_nvfp4_scaled_mm_workspace_bytes asks for, K is split over workgroups of the tile kernel
+    and fp32 partial tiles are added in a fixed order.  Ragged M / N / K (splits that do not divide the spans), both
+    output types, against the oracle; run-to-run bit equality; a workspace that is too small, NULL or misaligned falls
+    back to the kernels without one.  The last four shapes (one slab of 65..96 rows, N / 64 workgroups covering half
+    the chip or less, K % 128 == 0, 28+ chunks per split, 48 Mi weights or more) split K over workgroups of the
+    weight-streaming kernel instead: 2, 2, 3 and 4 splits, with 64, 56, 84 and 112 chunks, five activation row tiles."""
     from fuser_amd import capi
 
     m, n, k = shape
-    if shape in ((100, 4096, 6272), (128, 3072, 9216), (81, 8192, 6144), (65, 4096, 14336)):
+    if shape in ((80, 6144, 8192), (70, 8192, 7168), (72, 4736, 10752), (65, 4096, 14336)):
         assert "nvfp4_skinny_ring_kernel<RT=4,TT=8>" in capi.describe_dispatch("nvfp4_scaled_mm", m, n, k, 1, capi.BF16, 1 << 30)
     gen = torch.Generator().manual_seed(m + k)
     a, sa, ga = _nvfp4_operand(m, k, 1.0, gen)
