@@ -2616,6 +2616,12 @@ int launch_tile(const Params& p, int grid, hipStream_t stream) {
   else return launch_cfg<BM, BN, BF16_MMA, OUT_BF16>(p, grid, stream);
 }
 
+// Grouped NVFP4: rows in all from which a call counts as a prefill, whose large groups get launches of their own on the
+// persistent kernel.  Below, those launches find a handful of tiles each and run one after the other at a tile's
+// latency (256 experts, Zipf loads, K=7168: 2048 rows 732 -> 576 us, 4096 rows 769 -> 608 us without them; 8192 rows
+// 807 with against 753 without, but evenly loaded experts 639 against 771).
+constexpr int64_t kPrefillRows = 6144;
+
 template <bool NVFP4, bool BF16_MMA, bool OUT_BF16>
 int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int64_t workspace_bytes, hipStream_t stream) {
   // Pick the largest tile that still yields about one work item per compute unit.
@@ -2660,16 +2666,16 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int6
       if (p.k < 4096 && (p.n & 255) == 0) rc = launch_nvfp4_skinny_grouped<2, 2, OUT_BF16, true>(p, 1, 32, stream);
       else rc = launch_nvfp4_skinny_grouped<4, 2, OUT_BF16, false>(p, 1, 32, stream);
       if (rc != NVF_OK) return rc;
-      if ((p.k < 4096 || m_hint < 2048) && (p.n & 255) == 0 && p.k >= 256) {
+      if ((p.k < 4096 || m_hint < kPrefillRows) && (p.n & 255) == 0 && p.k >= 256) {
         // shallow K: one 128x256 tile of the persistent kernel per weight panel converts a group's rows once per 256
         // weight rows; the streaming kernel whose wavefronts own rows converts them once per wavefront.  Few rows
         // in all (a decode step): such groups are rare and the persistent kernel costs least when it finds none.
         Params mid = p;
         mid.rows_lo = 33;
         mid.rows_hi = 128;
-        if (m_hint >= 2048) mid.min_rows = 129;  // the 256x256 kernel follows: take the ends of its groups along
+        if (m_hint >= kPrefillRows) mid.min_rows = 129;  // the 256x256 kernel follows: take the ends of its groups along
         tail_done = mid.min_rows != 0;
-        if (m_hint >= 2048 && (p.n & 511) == 0 && p.k >= 1024) {
+        if (m_hint >= kPrefillRows && (p.n & 511) == 0 && p.k >= 1024) {
           // a prefill: the groups of up to 80 rows on the panel kernel, which multiplies row tiles of 16 (config 5,
           // K=2048: 5376 tiles of 128x256 in 680 us -> 325 us + 1792 tiles in 227 us)
           rc = launch_nvfp4_group_panel<4, 5, 2, OUT_BF16>(p, 33, 80, stream);
@@ -2703,7 +2709,7 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int6
     // Grouped NVFP4 with room for whole 256-row tiles: those go to the 256x256 kernel (about 1.4 times as
     // fast per flop), the ends of the groups to the 128x128 tile kernel.  The group sizes live on the
     // device, so both kernels are always launched; one that finds no work returns at once.
-    if (!dense && (p.n & 255) == 0 && (p.k & 127) == 0 && p.k >= 256 && m_hint >= 2048) {
+    if (!dense && (p.n & 255) == 0 && (p.k & 127) == 0 && p.k >= 256 && m_hint >= kPrefillRows) {
       const int rc = launch_nvfp4_fast<OUT_BF16, true>(p, cus, stream);
       if (rc != NVF_OK || p.tail_done) return rc;
       Params rest = p;

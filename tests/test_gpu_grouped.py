@@ -252,18 +252,18 @@ def test_nvfp4_grouped_mm_fewer_rows_in_all_than_the_smallest_mid_sized_group(de
     assert max_rel_rowwise(out[:m_total], ref[:m_total]) <= GEMM_MAX_REL
 
 
-@pytest.mark.parametrize("sizes,n,k", [([600, 0, 256, 255, 1, 1030, 512], 512, 384), ([300, 2100, 0, 257], 256, 256),
-                                       ([2560, 700, 3000, 0, 1280, 2900], 2048, 256), ([511] * 5, 512, 640),
-                                       ([2248, 130, 400], 256, 384),
-                                       ([40, 64, 2100, 33, 65, 100, 128, 50, 0, 32], 256, 512),
-                                       ([40, 64, 2100, 33, 65, 100, 128, 50, 0, 32], 384, 256)])
+@pytest.mark.parametrize("sizes,n,k", [([600, 0, 256, 255, 1, 1030, 512, 3600], 512, 384), ([300, 2100, 0, 257, 3585], 256, 256),
+                                       ([2560, 700, 3000, 0, 1280, 2900], 2048, 256), ([511] * 13, 512, 640),
+                                       ([3700, 2248, 130, 400], 256, 384),
+                                       ([40, 64, 2100, 33, 65, 100, 128, 50, 0, 32, 3620], 256, 512),
+                                       ([40, 64, 2100, 33, 65, 100, 128, 50, 0, 32, 3620], 384, 256)])
 def test_nvfp4_grouped_mm_whole_tiles_and_group_ends(dev, sizes, n, k):
-    """At least 2048 rows, N % 256 == 0, K % 128 == 0: the whole 256-row tiles of every group, and a last tile of
+    """A prefill-sized call (6144 rows or more), N % 256 == 0, K % 128 == 0: the whole 256-row tiles of every group, and a last tile of
     more than 128 rows, run on the persistent 256x256 kernel (the rows past such a group read as zero payload
     with whatever the scale padding holds - it is poisoned here - and are not stored), the other group ends
     on the 128x128 tile kernel.  Groups with no whole tile, only whole tiles, one row past a tile, 255 of 256
     rows, empty groups; two, three and five spans per tile; the third case has more than 320 tiles, i.e. two
-    per workgroup for some; the [2248, 130, 400] case ends with a 144-row tile whose 256 rows would reach past the
+    per workgroup for some; the [3700, 2248, 130, 400] case ends with a 144-row tile whose 256 rows would reach past the
     activation tensor.  The last two cases add groups of every
     weight-streaming class next to a large one (wavefronts owning rows, and wavefronts splitting K).  Every
     output element is compared."""
@@ -345,7 +345,7 @@ def test_nvfp4_grouped_mm_small_groups_stream_their_weights(dev, n, k):
 
 @pytest.mark.parametrize("n,k", [(512, 4096), (1024, 4224), (512, 2048), (1024, 1024), (512, 1152)])
 def test_nvfp4_grouped_mm_mid_sized_groups_of_a_prefill(dev, n, k):
-    """A prefill-sized call (2048 rows or more) with K >= 1024 and N % 512 == 0: groups of 33..80 rows run on the kernel
+    """A prefill-sized call (6144 rows or more) with K >= 1024 and N % 512 == 0: groups of 33..80 rows run on the kernel
     that converts a group's activation rows once per 512 weight rows (work items found from the device-resident
     sizes; three, four and five row tiles, sizes on both sides of its borders), their neighbours of 81..128 rows and
     the ends of the larger ones on 128x256 tiles of the persistent kernel, the rest of those on its 256x256 tiles.  8, 9,
@@ -354,9 +354,9 @@ def test_nvfp4_grouped_mm_mid_sized_groups_of_a_prefill(dev, n, k):
     bit equality."""
     from fuser_amd import capi, nvf_cutlass
 
-    sizes = [33, 80, 48, 49, 64, 65, 81, 32, 0, 128, 34, 47, 79, 300, 66, 50, 40, 72, 1, 129] + [56, 77, 35, 63] * 6
+    sizes = [33, 80, 48, 49, 64, 65, 81, 32, 0, 128, 34, 47, 79, 300, 66, 50, 40, 72, 1, 129] + [56, 77, 35, 63] * 6 + [3400]
     g, m = len(sizes), sum(sizes) + 3
-    assert sum(sizes) >= 2048
+    assert sum(sizes) >= 6144
     assert "nvfp4_group_panel_kernel" in capi.describe_dispatch("nvfp4_scaled_grouped_mm", m, n, k, groups=g)
     gen = torch.Generator().manual_seed(n + k)
     x = torch.randn(m, k, generator=gen).bfloat16()
