@@ -2110,22 +2110,13 @@ int launch_nvfp4_skinny_rt(const Params& p, int rt, hipStream_t stream, int slab
                  : launch_nvfp4_skinny_ring_cfg<1, TT, OUT_BF16>(p, stream, slabs);
 }
 
-template <int TT, bool OUT_BF16>
-int launch_nvfp4_skinny_tt(const Params& p, int cus, hipStream_t stream, int slabs = 1) {
-  // The conversion work bounds this kernel, and every workgroup converts all activation rows it uses:
-  // take as many weight rows per workgroup as still leaves about one workgroup per compute unit.
-  const int64_t want = (int64_t)cus * 4 / 5;
-  if ((p.n & 63) == 0 && p.n / 64 >= want) return launch_nvfp4_skinny_ring_cfg<4, TT, OUT_BF16>(p, stream, slabs);
-  if ((p.n & 31) == 0 && p.n / 32 >= want) return launch_nvfp4_skinny_ring_cfg<2, TT, OUT_BF16>(p, stream, slabs);
-  return launch_nvfp4_skinny_ring_cfg<1, TT, OUT_BF16>(p, stream, slabs);
-}
-
 // Cost, in arbitrary units, of streaming the weights against M activation rows as slabs of `slab` rows with rt weight
 // tiles (16 rows) per workgroup.  Every workgroup converts rt weight tiles and the tt row tiles of its slab per
 // 128-deep chunk (a wavefront takes every eighth chunk), so few large workgroups convert least, while small ones (less
 // LDS, fewer accumulators) share a compute unit and fill the chip at small N.  The constants are a fit to timings of
 // the nine (slab, rt) forms over M = 48..256, N = 1024..14336, K = 2048..14336 (144 shapes: the form picked is within
-// 8 % of the fastest for 134 of them, 1.8 % off on average; a fixed rule by N alone was 13 % off).
+// 8 % of the fastest for 134 of them, 1.8 % off on average; a fixed rule by N alone was 13 % off); for 1..32 rows
+// (112 shapes) its pick of rt is 0.2 % off the fastest on average.
 int64_t nvfp4_skinny_cost(int64_t m, int64_t n, int64_t k, int slab, int rt, int cus) {
   if (n % (16 * rt) != 0) return INT64_MAX;
   const int64_t slabs = m <= slab ? 1 : ceil_div(m, slab);
@@ -2160,9 +2151,7 @@ int64_t nvfp4_skinny_best(int64_t m, int64_t n, int64_t k, int cus, int* slab_ou
 
 template <bool OUT_BF16>
 int launch_nvfp4_skinny(const Params& p, int cus, hipStream_t stream) {
-  // Up to 32 rows: one slab, as many weight rows per workgroup as still leaves about one workgroup per compute unit
-  // (bound by the weight stream, not by conversions).
-  if (p.m <= 32) return p.m <= 16 ? launch_nvfp4_skinny_tt<1, OUT_BF16>(p, cus, stream) : launch_nvfp4_skinny_tt<2, OUT_BF16>(p, cus, stream);
+  // Up to 32 rows: one slab of 1 or 2 row tiles (16 x 6144 x 7168: 8.0 us with 1 weight tile per workgroup, 7.0 with 2).
   // More rows: slabs of 128, 64 or 32 rows side by side in one launch (blockIdx.y = slab; the last one may be ragged;
   // the slabs after the first find the weights in the last-level cache) with 1, 2 or 4 weight tiles per workgroup,
   // whichever the cost estimate above prefers (M=128, N=4096, K=4096: 10.8 us as two slabs of 64 rows x 1 weight tile,
@@ -2175,7 +2164,10 @@ int launch_nvfp4_skinny(const Params& p, int cus, hipStream_t stream) {
          : slab == 64  ? launch_nvfp4_skinny_rt<4, OUT_BF16>(p, rt, stream, slabs)
                        : launch_nvfp4_skinny_rt<2, OUT_BF16>(p, rt, stream, slabs);
   }
-  return p.m <= 64 ? launch_nvfp4_skinny_rt<4, OUT_BF16>(p, rt, stream, 1) : launch_nvfp4_skinny_rt<8, OUT_BF16>(p, rt, stream, 1);
+  return p.m <= 16 ? launch_nvfp4_skinny_rt<1, OUT_BF16>(p, rt, stream, 1)
+       : p.m <= 32 ? launch_nvfp4_skinny_rt<2, OUT_BF16>(p, rt, stream, 1)
+       : p.m <= 64 ? launch_nvfp4_skinny_rt<4, OUT_BF16>(p, rt, stream, 1)
+                   : launch_nvfp4_skinny_rt<8, OUT_BF16>(p, rt, stream, 1);
 }
 
 // -------------------------------------------------------------------------------------------------

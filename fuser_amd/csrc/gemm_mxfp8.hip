@@ -709,15 +709,6 @@ int launch_skinny_cfg(const Params& p, hipStream_t stream, int slabs = 1) {
 }
 
 template <int TT, bool OUT_BF16>
-int launch_skinny_tt(const Params& p, hipStream_t stream, int slabs = 1) {
-  // as many weight rows per workgroup as still leaves about one workgroup per compute unit
-  const int64_t want = (int64_t)cu_count() * 4 / 5;
-  if ((p.n & 63) == 0 && p.n / 64 >= want) return launch_skinny_cfg<4, TT, OUT_BF16>(p, stream, slabs);
-  if ((p.n & 31) == 0 && p.n / 32 >= want) return launch_skinny_cfg<2, TT, OUT_BF16>(p, stream, slabs);
-  return launch_skinny_cfg<1, TT, OUT_BF16>(p, stream, slabs);
-}
-
-template <int TT, bool OUT_BF16>
 int launch_skinny_rt(const Params& p, int rt, hipStream_t stream, int slabs) {
   if constexpr (TT == 8) return launch_skinny_cfg<1, 8, OUT_BF16>(p, stream, slabs);
   else
@@ -765,10 +756,8 @@ int64_t mxfp8_skinny_best(int64_t m, int64_t n, int64_t k, int64_t cus, int* sla
 
 template <bool OUT_BF16>
 int launch_skinny(const Params& p, hipStream_t stream) {
-  // Up to 32 rows: one slab, as many weight rows per workgroup as still leaves about one workgroup per compute unit.
-  if (p.m <= 16) return launch_skinny_tt<1, OUT_BF16>(p, stream);
-  if (p.m <= 32) return launch_skinny_tt<2, OUT_BF16>(p, stream);
-  // More rows: slabs of 128, 64 or 32 rows side by side in one launch (blockIdx.y = slab; the last one may be ragged;
+  // Up to 32 rows: one slab of 1 or 2 activation tiles (16 x 6144 x 4096: 8.0 us with 1 weight tile per workgroup in 1.5
+  // rounds, 6.2 us with 2); more rows: slabs of 128, 64 or 32 rows side by side in one launch (blockIdx.y = slab; the last one may be ragged;
   // the slabs after the first find the weights in the last-level cache) with 1, 2 or 4 weight tiles per workgroup
   // (1 with 128-row slabs, whose 8 activation tiles fill the ring), whichever the estimate above prefers
   // (128 x 4096 x 4096: 10.5 us as one slab of 128 rows, 7.6 us as 4 slabs of 32 rows x 4 weight tiles;
@@ -777,7 +766,8 @@ int launch_skinny(const Params& p, hipStream_t stream) {
   mxfp8_skinny_best(p.m, p.n, p.k, cu_count(), &slab, &rt);
   const int slabs = p.m <= slab ? 1 : (int)ceil_div(p.m, slab);
   const int rows = p.m <= slab ? p.m : slab;
-  return rows <= 32 ? launch_skinny_rt<2, OUT_BF16>(p, rt, stream, slabs)
+  return rows <= 16 ? launch_skinny_rt<1, OUT_BF16>(p, rt, stream, slabs)
+       : rows <= 32 ? launch_skinny_rt<2, OUT_BF16>(p, rt, stream, slabs)
        : rows <= 64 ? launch_skinny_rt<4, OUT_BF16>(p, rt, stream, slabs)
                     : launch_skinny_rt<8, OUT_BF16>(p, rt, stream, slabs);
 }
