@@ -2505,6 +2505,7 @@ int launch_nvfp4_tile(const Params& p, int grid, hipStream_t stream) {
 // is no more than that in all (all measured: M = 128..1024, N = 2048..14336, K = 4096 and 14336).
 struct DensePlan {
   enum Kernel { kStream, kTiles256, kTiles128, kOther } kernel;
+  int64_t ns;  // estimated duration (INT64_MAX: no estimate)
 };
 DensePlan nvfp4_dense_plan(int64_t m, int64_t n, int64_t k, int cus) {
   const bool stream_ok = (k & 127) == 0 && (n & 15) == 0 && k * 64 < (1ll << 31);  // 32-bit lane offsets
@@ -2517,16 +2518,17 @@ DensePlan nvfp4_dense_plan(int64_t m, int64_t n, int64_t k, int cus) {
     const int64_t small = 2 * t128, full = small / (2 * cus), rest = small - full * 2 * cus;
     cost_tile = full * 68 + (rest == 0 ? 0 : rest > cus ? 68 : full ? 45 : 22 + 25 * rest / cus);
   }
+  const int64_t cost_min = std::min(cost256, std::min(cost128, cost_tile));
+  const int64_t rest_ns = persistent_ok ? 6000 + cost_min * 240 * k / 1024 : INT64_MAX;
   if (stream_ok) {
+    // the streaming kernel's estimate is in ns within 0.8 (K = 2048) .. 1.1 (K = 14336)
+    const int64_t stream_ns = nvfp4_skinny_best(m, n, k, cus, nullptr, nullptr) * (k < 3072 ? 82 : k < 6144 ? 96 : k < 10240 ? 103 : 110) / 100;
     bool stream;
     if (m <= 256) {
       stream = true;  // at most two passes over the weights (256 x 14336 x 4096: 38 instead of 58 us on tiles)
     } else if (persistent_ok && k >= 2048) {
-      // by estimated duration; the streaming kernel's estimate is in ns within 0.8 (K = 2048) .. 1.1 (K = 14336)
-      // (measured: 512 x 4096 x 14336 115 -> 57 us, 384 x 8192 x 7168 82 -> 57 us, 640 x 14336 x 14336 381 -> 268 us;
-      // 1024 x 8192 x 4096 stays on 128x256 tiles: 64 against 76 us)
-      const int64_t rest_ns = 6000 + std::min(cost256, std::min(cost128, cost_tile)) * 240 * k / 1024;
-      const int64_t stream_ns = nvfp4_skinny_best(m, n, k, cus, nullptr, nullptr) * (k < 3072 ? 82 : k < 6144 ? 96 : k < 10240 ? 103 : 110) / 100;
+      // by estimated duration (measured: 512 x 4096 x 14336 115 -> 57 us, 384 x 8192 x 7168 82 -> 57 us,
+      // 640 x 14336 x 14336 381 -> 268 us; 1024 x 8192 x 4096 stays on 128x256 tiles: 64 against 76 us)
       stream = stream_ns <= rest_ns;
     } else {
       // Ragged shapes, which only the tile kernels take otherwise: with a deep K and a small N the streaming kernel
@@ -2536,13 +2538,30 @@ DensePlan nvfp4_dense_plan(int64_t m, int64_t n, int64_t k, int cus) {
       const int64_t rounds = ceil_div(ceil_div(m, 128) * (n / 16), cus);
       stream = k >= 2048 && rounds <= (k >= 4096 ? 3 : 2);
     }
-    if (stream) return {DensePlan::kStream};
+    if (stream) return {DensePlan::kStream, stream_ns};
   }
   if (persistent_ok) {
-    if (cost256 <= cost128 && cost256 <= cost_tile) return {DensePlan::kTiles256};
-    if (cost128 <= cost_tile) return {DensePlan::kTiles128};
+    if (cost256 <= cost128 && cost256 <= cost_tile) return {DensePlan::kTiles256, rest_ns};
+    if (cost128 <= cost_tile) return {DensePlan::kTiles128, rest_ns};
   }
-  return {DensePlan::kOther};
+  return {DensePlan::kOther, rest_ns};
+}
+
+// Dense shapes whose M is not a multiple of 128 and that only the tile kernels would take whole: the number of rows
+// (the last multiple of 128) that go to a launch of their own, if that shape gets a better kernel; else 0.  If that
+// kernel is the weight-streaming one, which takes any number of rows, the answer is m: no cut, all rows to it.
+int64_t nvfp4_rows_before_remainder(int64_t m, int64_t n, int64_t k, int cus) {
+  if (m <= 128 || (m & 127) == 0 || (k & 15) != 0) return 0;
+  if (nvfp4_dense_plan(m, n, k, cus).kernel != DensePlan::kOther) return 0;
+  // the cut is the last multiple of 128 or of 256 (which allows 256x256 tiles), whichever is estimated faster
+  int64_t best = INT64_MAX, cut = 0;
+  for (const int64_t c : {m & ~(int64_t)127, m & ~(int64_t)255}) {
+    if (c < 128) continue;
+    const DensePlan main = nvfp4_dense_plan(c, n, k, cus), rest = nvfp4_dense_plan(m - c, n, k, cus);
+    if (main.kernel == DensePlan::kOther || rest.kernel != DensePlan::kStream || main.ns == INT64_MAX) continue;
+    if (main.ns + rest.ns < best) best = main.ns + rest.ns, cut = main.kernel == DensePlan::kStream ? m : c;
+  }
+  return cut;
 }
 
 // Split of K for dense NVFP4 shapes with fewer 128x128 tiles than compute units and a deep K (decode and
@@ -2787,8 +2806,28 @@ int launch_gemm16(int op, const Gemm16Args& a, hipStream_t stream) {
     return launch_nvfp4_wide<true>(p, cus, stream);
   }
   if (op == 0 || op == 1) {
-    return bf16 ? launch_sized<true, false, true>(p, a.m, cus, a.workspace, a.workspace_bytes, stream)
-                : launch_sized<true, false, false>(p, a.m, cus, a.workspace, a.workspace_bytes, stream);
+    auto launch = [&](const Params& q, void* workspace, int64_t workspace_bytes) {
+      return bf16 ? launch_sized<true, false, true>(q, q.m, cus, workspace, workspace_bytes, stream)
+                  : launch_sized<true, false, false>(q, q.m, cus, workspace, workspace_bytes, stream);
+    };
+    // Dense with M not a multiple of 128 (a prefill of any token count), which leaves the whole call to the tile
+    // kernels: the rows up to the last multiple of 128 go to whatever kernel that shape gets, the remaining rows
+    // (at most 127, a whole number of 128-row scale tiles further on) to the weight-streaming kernel in a launch of
+    // their own (4000 x 4096 x 4096: 145 -> 116 us; 8100 x 8192 x 8192: 1002 -> 850 us).
+    const int64_t main_rows = op == 0 ? nvfp4_rows_before_remainder(p.m, p.n, p.k, cus) : 0;
+    if (main_rows == p.m) return bf16 ? launch_nvfp4_skinny<true>(p, cus, stream) : launch_nvfp4_skinny<false>(p, cus, stream);
+    if (main_rows) {
+      Params main = p, rest = p;
+      main.m = (int)main_rows;
+      rest.m = p.m - main.m;
+      const int64_t sf_padded = ((int64_t)(p.k >> 4) + 3) & ~(int64_t)3;
+      rest.a = p.a + (int64_t)main.m * (p.k >> 1);
+      rest.sfa = p.sfa + (int64_t)main.m * sf_padded;
+      rest.out = static_cast<uint8_t*>(p.out) + (int64_t)main.m * p.n * 2;
+      if (const int rc = launch(main, a.workspace, a.workspace_bytes)) return rc;
+      return launch(rest, nullptr, 0);
+    }
+    return launch(p, a.workspace, a.workspace_bytes);
   }
   return bf16 ? launch_sized<false, true, true>(p, a.m, cus, nullptr, 0, stream)
               : launch_sized<false, false, false>(p, a.m, cus, nullptr, 0, stream);
@@ -2823,6 +2862,10 @@ int static_scratch(void** ptr) {
 
 int64_t nvfp4_gemm_workspace_bytes(int64_t m, int64_t n, int64_t k) {
   if (m <= 0 || n <= 0 || k <= 0 || m > INT32_MAX || n > INT32_MAX || k > INT32_MAX) return 0;
+  if (const int64_t main_rows = nvfp4_rows_before_remainder(m, n, k, cu_count())) {
+    if (main_rows == m) return 0;  // all rows to the weight-streaming kernel
+    m = main_rows;                 // the launch that may split K
+  }
   const int skinny_splits = nvfp4_skinny_splits(m, n, k, cu_count());
   const int splits = skinny_splits > 1 ? skinny_splits : nvfp4_splits(m, n, k, cu_count());
   return splits > 1 ? (int64_t)splits * m * n * 4 : 0;

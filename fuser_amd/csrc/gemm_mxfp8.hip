@@ -784,39 +784,81 @@ int launch_cfg(const Params& p, hipStream_t stream) {
   return check_launch("mxfp8_gemm_kernel");
 }
 
-template <bool OUT_BF16>
-int launch_sized(const Params& p, hipStream_t stream) {
-  auto tiles = [&](int bm, int bn) { return ceil_div(p.m, bm) * ceil_div(p.n, bn); };
-  const int64_t cus = cu_count();
-  const bool skinny_ok = (p.k & 127) == 0 && (p.n & 15) == 0 && (int64_t)p.k * 64 < (1ll << 31);  // 32-bit lane offsets
-  const bool fast_ok = (p.k & 127) == 0 && p.k >= 256 && (p.m & 127) == 0 && (p.n & 255) == 0 && (int64_t)p.k * 256 < (1ll << 31);
-  // Persistent LDS-direct kernel with 256x256 or 128x256 tiles: a 128-row tile costs about 0.61 of a 256-row tile (half
-  // the flops at 82 % of the rate, measured), and the time goes with the rounds of tiles over the compute units;
-  // below 48 tiles the tile kernels further down do as well.
-  const int64_t t256 = fast_ok && (p.m & 255) == 0 ? tiles(256, 256) : 0, t128 = fast_ok ? tiles(128, 256) : 0;
+// Which kernel a shape gets.  Persistent LDS-direct kernel with 256x256 or 128x256 tiles: a 128-row tile costs about
+// 0.61 of a 256-row tile (half the flops at 82 % of the rate, measured), and the time goes with the rounds of tiles
+// over the compute units; below 48 tiles the tile kernels do as well.
+enum class Plan { kStream, kTiles256, kTiles128, kOther };
+// (ns: the estimated duration, where there is an estimate)
+Plan mxfp8_plan(int64_t m, int64_t n, int64_t k, int64_t cus, int64_t* ns = nullptr) {
+  if (ns) *ns = INT64_MAX;
+  const bool skinny_ok = (k & 127) == 0 && (n & 15) == 0 && k * 64 < (1ll << 31);  // 32-bit lane offsets
+  const bool fast_ok = (k & 127) == 0 && k >= 256 && (m & 127) == 0 && (n & 255) == 0 && k * 256 < (1ll << 31);
+  const int64_t t256 = fast_ok && (m & 255) == 0 ? (m / 256) * (n / 256) : 0, t128 = fast_ok ? (m / 128) * (n / 256) : 0;
   const int64_t cost256 = t256 >= 128 ? 100 * ceil_div(t256, cus) : INT64_MAX;
   const int64_t cost128 = t128 >= 48 ? 61 * ceil_div(t128, cus) : INT64_MAX;
   const bool fast = cost256 != INT64_MAX || cost128 != INT64_MAX;
+  const int64_t fast_ns = fast ? 5000 + std::min(cost256, cost128) * 113 * k / 1024 : INT64_MAX;
   if (skinny_ok) {
-    if (p.m <= 32) return launch_skinny<OUT_BF16>(p, stream);
+    const int64_t skinny_ns = mxfp8_skinny_best(m, n, k, cus, nullptr, nullptr) * 963 / 1000;
+    if (ns) *ns = skinny_ns;
+    if (m <= 32) return Plan::kStream;
     if (fast) {
       // Skinny or persistent kernel by estimated duration: a round of 128x256 tiles takes 6.9 us per 1024 of K plus
       // about 5 us (so cost 100 = 11.3 us per 1024 of K), the skinny kernel what its estimate says (its unit is
       // 0.96 ns).  Measured: 256 x 14336 x 4096 31 (persistent) against 47 us, 512 x 4096 x 7168 51 against 30 us
       // (skinny), 1024 x 2048 x 14336 97 against 48 us, 1024 x 4096 x 4096 31 against 34 us.
-      const int64_t fast_ns = 5000 + std::min(cost256, cost128) * 113 * (int64_t)p.k / 1024;
-      const int64_t skinny_ns = mxfp8_skinny_best(p.m, p.n, p.k, cus, nullptr, nullptr) * 963 / 1000;
-      if (skinny_ns <= fast_ns) return launch_skinny<OUT_BF16>(p, stream);
+      if (skinny_ns <= fast_ns) return Plan::kStream;
     } else {
       // No persistent kernel for the shape (ragged M or N, or too few tiles): up to 256 rows, i.e. four passes over
-      // the weights, the skinny kernel beats the tile kernels below (128 x 4096 x 14336: 20 instead of 117 us); with
-      // more rows, a deep K and a small N it fills the chip where they cannot, while its 128-row x 16-column
-      // workgroups cover the compute units at most 3 times (measured, K >= 2048).
-      const int64_t skinny_rounds = ceil_div(ceil_div(p.m, 128) * (int64_t)(p.n / 16), cus);
-      if (p.m <= 256 || (skinny_rounds <= 3 && p.k >= 2048)) return launch_skinny<OUT_BF16>(p, stream);
+      // the weights, the skinny kernel beats the tile kernels (128 x 4096 x 14336: 20 instead of 117 us); with more
+      // rows, a deep K and a small N it fills the chip where they cannot, while its 128-row x 16-column workgroups
+      // cover the compute units at most 3 times (measured, K >= 2048).
+      const int64_t skinny_rounds = ceil_div(ceil_div(m, 128) * (n / 16), cus);
+      if (m <= 256 || (skinny_rounds <= 3 && k >= 2048)) return Plan::kStream;
     }
   }
-  if (fast) return cost256 <= cost128 ? launch_fast<4, OUT_BF16>(p, stream) : launch_fast<2, OUT_BF16>(p, stream);
+  if (ns) *ns = fast_ns;
+  if (fast) return cost256 <= cost128 ? Plan::kTiles256 : Plan::kTiles128;
+  return Plan::kOther;
+}
+
+template <bool OUT_BF16>
+int launch_sized(const Params& p, hipStream_t stream) {
+  auto tiles = [&](int bm, int bn) { return ceil_div(p.m, bm) * ceil_div(p.n, bn); };
+  const int64_t cus = cu_count();
+  switch (mxfp8_plan(p.m, p.n, p.k, cus)) {
+    case Plan::kStream: return launch_skinny<OUT_BF16>(p, stream);
+    case Plan::kTiles256: return launch_fast<4, OUT_BF16>(p, stream);
+    case Plan::kTiles128: return launch_fast<2, OUT_BF16>(p, stream);
+    case Plan::kOther: break;
+  }
+  // M not a multiple of 128 (a prefill of any token count) and too many rows for the skinny kernel: the rows up to
+  // the last multiple of 128 go to whatever kernel that shape gets, the remaining rows (at most 127, a whole number
+  // of 128-row scale tiles further on) to the skinny kernel in a launch of their own (4000 x 4096 x 4096: 197 -> 77 us;
+  // 8100 x 8192 x 8192: 1475 -> 390 us).
+  // The cut is the last multiple of 128 or of 256 (which allows 256x256 tiles), whichever is estimated faster
+  // (8100 x 8192 x 8192: 546 us cut at 8064, 128x256 tiles; 390 us cut at 7936).
+  if (p.m > 128 && (p.m & 127) != 0 && (p.k & 31) == 0) {
+    int64_t best = INT64_MAX;
+    int cut = 0;
+    for (const int c : {p.m & ~127, p.m & ~255}) {
+      int64_t ns_main, ns_rest;
+      if (c < 128 || mxfp8_plan(c, p.n, p.k, cus, &ns_main) == Plan::kOther || mxfp8_plan(p.m - c, p.n, p.k, cus, &ns_rest) != Plan::kStream) continue;
+      if (ns_main + ns_rest < best) best = ns_main + ns_rest, cut = mxfp8_plan(c, p.n, p.k, cus) == Plan::kStream ? p.m : c;
+    }
+    if (cut == p.m) return launch_skinny<OUT_BF16>(p, stream);  // (the skinny kernel takes any number of rows)
+    if (cut) {
+      Params main = p, rest = p;
+      main.m = cut;
+      rest.m = p.m - cut;
+      const int64_t sf_padded = ((int64_t)(p.k >> 5) + 3) & ~(int64_t)3;
+      rest.a = p.a + (int64_t)cut * p.k;
+      rest.sfa = p.sfa + (int64_t)cut * sf_padded;
+      rest.out = static_cast<uint8_t*>(p.out) + (int64_t)cut * p.n * 2;
+      if (const int rc = launch_sized<OUT_BF16>(main, stream)) return rc;
+      return launch_sized<OUT_BF16>(rest, stream);
+    }
+  }
   if (tiles(256, 256) >= cus) return launch_cfg<256, 256, OUT_BF16>(p, stream);
   if (tiles(128, 128) >= cus) return launch_cfg<128, 128, OUT_BF16>(p, stream);
   return launch_cfg<64, 64, OUT_BF16>(p, stream);

@@ -92,6 +92,20 @@ def test_nvfp4_mid_sized_shapes(m, n, k, kernel):
     assert plan("nvfp4_scaled_mm", m, n, k).startswith(kernel), plan("nvfp4_scaled_mm", m, n, k)
 
 
+@pytest.mark.parametrize("op", ["nvfp4_scaled_mm", "mxfp8_scaled_mm"])
+def test_dense_m_not_a_multiple_of_128_is_cut_into_a_main_part_and_a_remainder(op):
+    # a prefill of any token count: the rows up to a multiple of 128 / 256 on the persistent kernel, the rest streamed
+    got = plan(op, 4000, 4096, 4096).split("; ")
+    assert len(got) == 2 and "gemm_256_kernel<" in got[0] and "TM=4" in got[0] and "skinny" in got[1], got
+    got = plan(op, 8100, 8192, 8192).split("; ")
+    assert len(got) == 2 and "gemm_256_kernel<" in got[0] and "TM=4" in got[0] and "grid=256" in got[0] and "skinny" in got[1], got
+    # where the main part would stream as well, one launch takes all rows
+    got = plan(op, 1000, 4096, 14336).split("; ")
+    assert len(got) == 1 and "skinny" in got[0], got
+    # multiples of 128 and small shapes: as before
+    assert "; " not in plan(op, 4096, 4096, 4096) and "; " not in plan(op, 300, 4096, 4096)
+
+
 def test_nvfp4_8192_cubed_takes_the_persistent_256x256_kernel():
     assert plan("nvfp4_scaled_mm", 8192, 8192, 8192).startswith("nvfp4_gemm_256_kernel<grouped=0,TM=4,f32=0,pairs=1> grid=256")
 

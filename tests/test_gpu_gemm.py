@@ -286,6 +286,48 @@ def test_nvfp4_gemm_many_rows_small_n_deep_k(dev, shape):
         assert torch.equal(out, _run_nvfp4(a, b, sa_p, sb, alpha, dtype, dev))
 
 
+@pytest.mark.parametrize("shape", [(2100, 4096, 2048), (2504, 2048, 2048), (1000, 14336, 2048), (2304 + 255, 4096, 2048), (4300, 2048, 2048), (1000, 2048, 256)])
+def test_dense_gemms_with_m_not_a_multiple_of_128(dev, shape):
+    """A prefill of any token count: M > 128 and not a multiple of 128 is cut at a multiple of 128 or 256; the rows
+    before the cut go to the persistent (or streaming) kernel, the 1..255 rows after it to the weight-streaming kernel
+    in a launch of its own, which reads its activation scales a whole number of 128-row scale tiles further on.  Both
+    ops, both output types, every element against the oracle, poisoned scale padding, rows of the two launches next to
+    the cut compared like all others, run-to-run bit equality."""
+    from fuser_amd import capi
+
+    m, n, k = shape
+    gen = torch.Generator().manual_seed(m + n + k)
+    plans = []
+    # NVFP4
+    a, sa, ga = _nvfp4_operand(m, k, 1.0, gen)
+    b, sb, gb = _nvfp4_operand(n, k, 0.02, gen)
+    alpha = 1.0 / (ga * gb)
+    ref = O.ref_nvfp4_scaled_mm(a, b, sa, sb, alpha)
+    sa_p = sa.clone()
+    sa_p[O.linear_to_swizzled_128_4(torch.ones(m, k // 16, dtype=torch.uint8)) == 0] = 0x7F
+    plans.append(capi.describe_dispatch("nvfp4_scaled_mm", m, n, k))
+    for dtype in (torch.bfloat16, torch.float16):
+        out = _run_nvfp4(a, b, sa_p, sb, alpha, dtype, dev)
+        assert out.shape == (m, n) and max_rel_rowwise(out, ref) <= GEMM_MAX_REL, (shape, dtype, plans[-1])
+        assert torch.equal(out, _run_nvfp4(a, b, sa_p, sb, alpha, dtype, dev))
+    # MXFP8
+    a8, sa8 = _mxfp8_operand(m, k, gen, 1.0)
+    b8, sb8 = _mxfp8_operand(n, k, gen, 1.0)
+    ref = O.ref_mxfp8_scaled_mm(a8, b8, sa8, sb8, 0.75)
+    sa8_p = sa8.clone()
+    sa8_p[O.linear_to_swizzled_128_4(torch.ones(m, k // 32, dtype=torch.uint8)) == 0] = 0xFF
+    scale = ref.abs().amax(dim=1, keepdim=True).clamp(min=1e-30)
+    plans.append(capi.describe_dispatch("mxfp8_scaled_mm", m, n, k))
+    for dtype in (torch.bfloat16, torch.float16):
+        if dtype == torch.float16 and ref.abs().max() > 6e4:
+            continue
+        out = _run_mxfp8(a8, b8, sa8_p, sb8, 0.75, dtype, dev)
+        assert out.shape == (m, n)
+        assert ((out.float().cpu() - ref).abs() / scale).max().item() <= GEMM_MAX_REL, (shape, dtype, plans[-1])
+        assert torch.equal(out, _run_mxfp8(a8, b8, sa8_p, sb8, 0.75, dtype, dev))
+    assert all("; " in p for p in plans) or shape == (1000, 2048, 256), plans  # (the last shape: cut for MXFP8 only)
+
+
 @pytest.mark.parametrize("shape", [(128, 1024, 8224), (100, 256, 8224), (200, 512, 10272), (65, 160, 9248), (300, 2048, 14368),
                                    (80, 6144, 8192), (70, 8192, 7168), (72, 4736, 10752), (65, 4096, 14336)])
 def test_nvfp4_gemm_split_k_with_workspace(dev, shape):
