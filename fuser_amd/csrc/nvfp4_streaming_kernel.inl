@@ -1,0 +1,694 @@
+// Weight-streaming NVFP4 kernel of gemm16.hip (included there, inside namespace nvf): the kernel, its launchers and the
+// cost estimate that picks slab height and weight tiles per workgroup.
+// -------------------------------------------------------------------------------------------------
+// NVFP4 skinny path: dense, up to 128 activation rows per launch (decode-sized activations; up to 256 rows in
+// two launches), K % 128 == 0, N % (16*RT) == 0.  A launch streams the weight matrix exactly once, so the op
+// is bound by HBM and by the conversion work, not by the MFMAs:
+//   * A workgroup owns 16*RT weight rows for the whole of K and all M activation rows; its 8
+//     wavefronts split K in interleaved 128-element chunks and their partial sums are added in a fixed
+//     order through LDS (no atomics, no workspace, deterministic).
+//   * In v_mfma_f32_16x16x32_f16 lane (i, g) supplies 8 elements of row i, and both operands use the same
+//     (lane group, element) -> k assignment, so a lane holds the 16 payload bytes [32g, 32g+32) of its
+//     row's chunk, converts them to fp16 in registers and feeds MFMA t = 0..3 with elements 8t..8t+7.
+//     Weight rows are the first operand (output rows), activation rows the second, so a lane ends up
+//     with 4 consecutive N-elements of one output row.
+//   * A load in that lane order (lane = row % 16 + 16 * piece) touches 64 unrelated 16-byte pieces and
+//     occupies the address unit for 64 cycles, which - not HBM, not latency - bounded an earlier version
+//     that loaded straight into registers.  The tiles are therefore fetched with LDS-direct loads in
+//     memory order (4 neighbouring lanes = 64 contiguous bytes of a row; scales as the 256 contiguous
+//     bytes that hold a 16-row tile's scale words) into a private LDS ring of each wavefront and read
+//     back in MFMA order; no barrier is involved because a wavefront only reads what it loaded itself.
+//   LDS per slot: NT payload tiles of 16 rows x 64 B, piece p of row r at piece position p ^ ((r >> 2) & 3)
+//   (conflict-free reads), then per operand one 1 KiB scale block per pair of tiles: [tile][col tile][row][16 B].
+// -------------------------------------------------------------------------------------------------
+// LDS-direct load.  lds_byte_addr and base are wave-uniform; lane L's 16 bytes land at lds_byte_addr + 16 * L.
+// Issued from inline assembly: the compiler neither waits for it nor orders LDS reads against it, the
+// kernels do that with explicit s_waitcnt vmcnt(n).
+__device__ __forceinline__ void lds_dma16(uint32_t lds_byte_addr, const uint8_t* base, uint32_t voff) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_byte_addr), "v"(voff), "s"(base) : "memory", "m0");
+}
+
+// 32 packed e2m1 values and their two e4m3 block scales -> four MFMA operands of 8 fp16 values
+__device__ __forceinline__ void dequant_frags(const u32x4 q, uint32_t s2, u32x4 out[4]) {
+  const float f0 = __builtin_amdgcn_cvt_f32_fp8((int)s2, 0), f1 = __builtin_amdgcn_cvt_f32_fp8((int)s2, 1);
+  const f16x2 sv[2] = {__builtin_bit_cast(f16x2, __builtin_amdgcn_cvt_pkrtz(f0, f0)),
+                       __builtin_bit_cast(f16x2, __builtin_amdgcn_cvt_pkrtz(f1, f1))};
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {  // dword w = elements 8w..8w+7, scale block w/2
+    const f16x2 h0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(q[w], 1.0f, 0) * sv[w >> 1];
+    const f16x2 h1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(q[w], 1.0f, 1) * sv[w >> 1];
+    const f16x2 h2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(q[w], 1.0f, 2) * sv[w >> 1];
+    const f16x2 h3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(q[w], 1.0f, 3) * sv[w >> 1];
+    out[w] = u32x4{__builtin_bit_cast(uint32_t, h0), __builtin_bit_cast(uint32_t, h1), __builtin_bit_cast(uint32_t, h2),
+                   __builtin_bit_cast(uint32_t, h3)};
+  }
+}
+
+// GROUPED: one workgroup per (group, block of 16*RT weight rows); it serves groups of rows_lo .. rows_hi rows
+// (at most 16*TT) and returns at once for the others, which other launches take.
+// NSPLIT (grouped only, where the groups supply enough workgroups): the 8 wavefronts own 8 different blocks of
+// 16*RT weight rows and each walks all of K on its own - a long pipeline per wavefront and no reduction -
+// instead of sharing one block and splitting K.
+template <int RT, int TT, bool OUT_BF16, int DEPTH, bool GROUPED = false, bool NSPLIT = false>
+__global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) {
+  static_assert(GROUPED || !NSPLIT, "the dense op has too few row blocks to give every wavefront its own");
+  constexpr int W = 8;
+  constexpr int NT = RT + TT;
+  constexpr int B_SC = (RT + 1) / 2, A_SC = (TT + 1) / 2;     // scale blocks (1 KiB) per operand
+  constexpr int SLOT_BYTES = (NT + B_SC + A_SC) * 1024;
+  constexpr int NDMA = NT + B_SC + A_SC;                      // loads per chunk and wavefront
+  // DEPTH 2: two chunks in flight per wavefront.  DEPTH 1 (many tiles per chunk): the next chunk is requested
+  // as soon as the current one has been read out of LDS, and lands under its long conversion + MFMA phase.
+  static_assert((DEPTH == 1 || DEPTH == 2) && W * DEPTH * SLOT_BYTES <= 160 * 1024 && DEPTH * NDMA <= 63, "ring does not fit");
+  extern __shared__ f32x4 red[];  // ring during the K loop, then [W][tiles][64 lanes] partial sums
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15, g = lane >> 4;
+  const int kbytes = p.k >> 1;
+  int chunks = p.k >> 7;
+  const int sf_padded = p.k >> 4;  // K % 128 == 0: no padding columns
+  // dense with a workspace: blockIdx.z owns the chunks [c_lo, c_lo + chunks) of K and leaves an fp32 partial result
+  int c_lo = 0;
+  if (!GROUPED && p.partial != nullptr) {
+    c_lo = (int)blockIdx.z * p.spans_per_split;
+    chunks = min(chunks - c_lo, p.spans_per_split);
+  }
+  int n0, m_loc, grp = 0, asf_word0 = 0;  // asf_word0: which 32-row group of its 128-row scale tile the slab starts in
+  int64_t a_row0 = p.m_base, asf_row0 = p.m_base, b_row0 = 0;  // first activation row, its scale row, first weight row
+  if constexpr (GROUPED) {
+    const int nblocks = p.n / (16 * RT * (NSPLIT ? W : 1));
+    grp = blockIdx.x / nblocks;
+    n0 = ((blockIdx.x - grp * nblocks) * (NSPLIT ? W : 1) + (NSPLIT ? wave : 0)) * (16 * RT);
+    m_loc = __builtin_amdgcn_readfirstlane(p.problem_sizes[grp * 3]);
+    if (m_loc < p.rows_lo || m_loc > p.rows_hi) return;
+    a_row0 = __builtin_amdgcn_readfirstlane(p.expert_offsets[grp]);
+    asf_row0 = __builtin_amdgcn_readfirstlane(p.sf_offsets[grp]);  // the group's own scale slab
+    b_row0 = (int64_t)grp * p.n;
+  } else {
+    n0 = blockIdx.x * (16 * RT);
+    // activation rows of this workgroup: [m_base, m_base + m_loc); blockIdx.y counts slabs of 16*TT rows
+    // (TT = 2, 4 or 8 when there is more than one, so that a slab lies inside one 32-row scale group)
+    const int m_base = p.m_base + (int)blockIdx.y * (16 * TT);
+    a_row0 = m_base;
+    asf_row0 = m_base & ~127;
+    asf_word0 = (m_base & 127) >> 5;
+    m_loc = min(p.m - m_base, 16 * TT);
+  }
+  const int tt_count = (m_loc + 15) >> 4;
+
+  // ---- load side (memory order): lane L fetches row L/4, piece (L%4) ^ ((L/16)&3) of a payload tile
+  const int lrow = lane >> 2, lpiece = (lane & 3) ^ ((lane >> 4) & 3);
+  const uint8_t* b_base = p.b + (b_row0 + n0) * kbytes + c_lo * 64;
+  const uint8_t* bsf_base = p.sfb + b_row0 * sf_padded + swizzle_128x4(n0 & ~127, 0, sf_padded) + (int64_t)c_lo * 1024;
+  const uint8_t* a_base = p.a + a_row0 * kbytes + c_lo * 64;
+  const uint8_t* asf_base = p.sfa + asf_row0 * sf_padded + (int64_t)c_lo * 1024;  // the 128-row scale tile of these rows (row0 % 128 == 0)
+  uint32_t b_off[RT], a_off[TT], bsf_off[B_SC], asf_off[A_SC];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) b_off[rt] = (uint32_t)(rt * 16 + lrow) * (uint32_t)kbytes + lpiece * 16;
+#pragma unroll
+  for (int tt = 0; tt < TT; ++tt) a_off[tt] = (uint32_t)min(tt * 16 + lrow, m_loc - 1) * (uint32_t)kbytes + lpiece * 16;
+  // scale block j of an operand: lane L = tile 2j + (L>>5), col tile (L>>4)&1, row L&15: the 16 bytes that
+  // hold the scale words of rows {row, row+32, row+64, row+96} (mod 128) for that col tile
+#pragma unroll
+  for (int j = 0; j < B_SC; ++j) {
+    const int t = min(2 * j + (lane >> 5), RT - 1);
+    const int row = (n0 & 127) + t * 16 + (lane & 15);
+    bsf_off[j] = (uint32_t)((row & 31) * 16 + ((lane >> 4) & 1) * 512);
+  }
+#pragma unroll
+  for (int j = 0; j < A_SC; ++j) {
+    const int t = min(2 * j + (lane >> 5), TT - 1);
+    const int row = t * 16 + (lane & 15);  // < 128: inside the first 128-row tile of the activations' scales
+    asf_off[j] = (uint32_t)((row & 31) * 16 + ((lane >> 4) & 1) * 512);
+  }
+  const uint32_t lds_base = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)red);
+  const uint32_t ring_base = lds_base + (uint32_t)wave * (DEPTH * SLOT_BYTES);
+  auto issue_chunk = [&](int c_in, int slot) {  // c_in is wave-uniform
+    if (c_in >= chunks) return;
+    const uint32_t c = (uint32_t)c_in;
+    const uint32_t sb = ring_base + (uint32_t)slot * SLOT_BYTES;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) lds_dma16(sb + rt * 1024, b_base, b_off[rt] + c * 64u);
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) {
+      // with one slot every wait is for everything, so tiles without rows need not be fetched
+      if (DEPTH == 2 || tt < tt_count) lds_dma16(sb + (RT + tt) * 1024, a_base, a_off[tt] + c * 64u);
+    }
+#pragma unroll
+    for (int j = 0; j < B_SC; ++j) lds_dma16(sb + (NT + j) * 1024, bsf_base, bsf_off[j] + c * 1024u);
+#pragma unroll
+    for (int j = 0; j < A_SC; ++j) {
+      if (DEPTH == 2 || 2 * j < tt_count) lds_dma16(sb + (NT + B_SC + j) * 1024, asf_base, asf_off[j] + c * 1024u);
+    }
+  };
+
+  // ---- read side (MFMA order): lane (r, g) = row r, payload piece g, scale blocks 2g, 2g+1 of the chunk
+  const int rd_payload = r * 64 + ((g ^ ((r >> 2) & 3)) * 16);
+  int rd_bsc[RT], rd_asc[TT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const int rowgroup = (((n0 & 127) + rt * 16) >> 5) & 3;  // which of the 4 words of the 16 bytes
+    rd_bsc[rt] = (NT + (rt >> 1)) * 1024 + ((rt & 1) * 2 + (g >> 1)) * 256 + r * 16 + rowgroup * 4;
+  }
+#pragma unroll
+  for (int tt = 0; tt < TT; ++tt)
+    rd_asc[tt] = (NT + B_SC + (tt >> 1)) * 1024 + ((tt & 1) * 2 + (g >> 1)) * 256 + r * 16 + (asf_word0 + ((tt * 16) >> 5)) * 4;
+  const int sc_shift = (g & 1) * 16;
+
+  const float alpha = p.alpha[grp];
+  uint16_t* out = static_cast<uint16_t*>(p.out);
+  // Accumulators acc[RT][TTC] of the TTC activation tiles this workgroup was compiled for (tt_count <= TTC of them
+  // hold rows) -> result: stored directly (NSPLIT) or summed over the wavefronts through LDS.
+  auto finish = [&](auto ttc_c, auto& acc) {
+    constexpr int TTC = decltype(ttc_c)::value;
+    if constexpr (NSPLIT) {
+      // every wavefront holds finished sums: element e of lane l = weight row 4*(l/16) + e, activation row l%16
+#pragma unroll
+      for (int tt = 0; tt < TTC; ++tt) {
+        const int tok = tt * 16 + r;
+        if (tok < m_loc) {
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt) {
+            u32x2 v;
+            v[0] = pack2(acc[rt][tt][0] * alpha, acc[rt][tt][1] * alpha, OUT_BF16);
+            v[1] = pack2(acc[rt][tt][2] * alpha, acc[rt][tt][3] * alpha, OUT_BF16);
+            *reinterpret_cast<u32x2*>(out + (a_row0 + tok) * p.n + n0 + rt * 16 + 4 * g) = v;
+          }
+        }
+      }
+      return;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no LDS-direct load may be pending when the ring is reused
+    __syncthreads();
+
+    // ---- sum the wavefronts' partial tiles in wave order and store: all tiles in one round if they fit the
+    // ring's memory (RT * TT <= 8), else one round per weight-row tile
+    constexpr int ROUNDS = RT * TT <= 8 ? 1 : RT;
+    constexpr int RPR = RT / ROUNDS;  // weight-row tiles per round
+    const int tiles = RPR * tt_count;   // tile index inside a round: rt * tt_count + tt
+    const int units = tiles * 64;
+#pragma unroll
+    for (int round = 0; round < ROUNDS; ++round) {
+      if (round > 0) __syncthreads();
+#pragma unroll
+      for (int r2 = 0; r2 < RPR; ++r2)
+#pragma unroll
+        for (int tt = 0; tt < TTC; ++tt)
+          if (tt < tt_count) red[(wave * tiles + r2 * tt_count + tt) * 64 + lane] = acc[round * RPR + r2][tt];
+      __syncthreads();
+      for (int u = tid; u < units; u += 512) {
+        const int l = u & 63, tile = u >> 6;
+        const int r2 = tile / tt_count, tt = tile - r2 * tt_count;
+        f32x4 s = red[u];
+#pragma unroll
+        for (int w = 1; w < W; ++w) s += red[w * units + u];
+        const int tok = tt * 16 + (l & 15);
+        if (tok < m_loc) {
+          const int64_t at = (a_row0 + tok) * p.n + n0 + (round * RPR + r2) * 16 + 4 * (l >> 4);
+          if (!GROUPED && p.partial != nullptr) {  // this K range's sums as they are; the reduction applies alpha
+            *reinterpret_cast<f32x4*>(p.partial + (int64_t)blockIdx.z * p.m * p.n + at) = s;
+          } else {
+            u32x2 v;
+            v[0] = pack2(s[0] * alpha, s[1] * alpha, OUT_BF16);
+            v[1] = pack2(s[2] * alpha, s[3] * alpha, OUT_BF16);
+            *reinterpret_cast<u32x2*>(out + at) = v;
+          }
+        }
+      }
+    }
+  };
+
+  constexpr int CSTEP = NSPLIT ? 1 : W;  // distance of a wavefront's consecutive chunks
+  const int c_first = NSPLIT ? 0 : wave;
+  // Many activation tiles (TT > 2): the chunk loop is compiled for the group's number of row tiles (no branches in
+  // it, accumulators for just those tiles); for counts whose accumulators leave the registers for it, a chunk's
+  // conversions are folded into its MFMA steps.
+  constexpr bool kFineRing = TT > 2 && DEPTH == 1;
+  if constexpr (kFineRing) {
+    auto load_b_part = [&](uint32_t c) {
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) lds_dma16(ring_base + rt * 1024, b_base, b_off[rt] + c * 64u);
+#pragma unroll
+      for (int j = 0; j < B_SC; ++j) lds_dma16(ring_base + (NT + j) * 1024, bsf_base, bsf_off[j] + c * 1024u);
+    };
+    int fine_lrow = lrow;  // re-derived per use: eight row offsets kept in registers would not fit
+    auto load_a_tile = [&](uint32_t c, int tt) {
+      asm volatile("" : "+v"(fine_lrow));
+      lds_dma16(ring_base + (RT + tt) * 1024, a_base, (uint32_t)min(tt * 16 + fine_lrow, m_loc - 1) * (uint32_t)kbytes + lpiece * 16 + c * 64u);
+    };
+    auto load_a_scales = [&](uint32_t c, int j) { lds_dma16(ring_base + (NT + B_SC + j) * 1024, asf_base, asf_off[j] + c * 1024u); };
+    const char* sp = reinterpret_cast<const char*>(red) + wave * SLOT_BYTES;
+    auto read_a_tile = [&](int tt, u32x4& aq, uint32_t& as) {
+      aq = *reinterpret_cast<const u32x4*>(sp + (RT + tt) * 1024 + rd_payload);
+      as = *reinterpret_cast<const uint32_t*>(sp + rd_asc[tt]) >> sc_shift;
+    };
+    // e4m3 scales of a lane's two blocks -> fp16 pairs; one dword (8 values of one block) -> one MFMA operand
+    auto scale_pairs = [&](uint32_t s2, f16x2 sv[2]) {
+      const float f0 = __builtin_amdgcn_cvt_f32_fp8((int)s2, 0), f1 = __builtin_amdgcn_cvt_f32_fp8((int)s2, 1);
+      sv[0] = __builtin_bit_cast(f16x2, __builtin_amdgcn_cvt_pkrtz(f0, f0));
+      sv[1] = __builtin_bit_cast(f16x2, __builtin_amdgcn_cvt_pkrtz(f1, f1));
+    };
+    auto dequant_dword = [&](uint32_t qw, f16x2 sv) {
+      const f16x2 h0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(qw, 1.0f, 0) * sv;
+      const f16x2 h1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(qw, 1.0f, 1) * sv;
+      const f16x2 h2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(qw, 1.0f, 2) * sv;
+      const f16x2 h3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(qw, 1.0f, 3) * sv;
+      return u32x4{__builtin_bit_cast(uint32_t, h0), __builtin_bit_cast(uint32_t, h1), __builtin_bit_cast(uint32_t, h2),
+                   __builtin_bit_cast(uint32_t, h3)};
+    };
+    // One chunk with TTC activation tiles.  The whole slot is read out into registers at once and refilled with
+    // the wavefront's next chunk, which then has a whole chunk's time to land.  The chunk is four 32-deep MFMA
+    // steps of TTC groups of RT MFMAs; the operands of the next step - one dword of every weight and activation
+    // tile - are converted between the groups of the current one, so that they issue while the matrix pipe works.
+    auto chunk = [&](auto ttc_c, uint32_t c, auto& acc) {
+      constexpr int TTC = decltype(ttc_c)::value;
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      u32x4 q[RT], aq[TTC];
+      uint32_t sc[RT], as[TTC];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) q[rt] = *reinterpret_cast<const u32x4*>(sp + rt * 1024 + rd_payload);
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) sc[rt] = *reinterpret_cast<const uint32_t*>(sp + rd_bsc[rt]) >> sc_shift;
+#pragma unroll
+      for (int tt = 0; tt < TTC; ++tt) read_a_tile(tt, aq[tt], as[tt]);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // read out: may be refilled
+      if (c + CSTEP < (uint32_t)chunks) {
+        load_b_part(c + CSTEP);
+#pragma unroll
+        for (int tt = 0; tt < TTC; ++tt) {
+          load_a_tile(c + CSTEP, tt);
+          if ((tt & 1) || tt + 1 == TTC) load_a_scales(c + CSTEP, tt >> 1);
+        }
+      }
+      f16x2 sv[RT][2], asv[TTC][2];
+      u32x4 fb[RT], fa[TTC], fbn[RT], fan[TTC];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        scale_pairs(sc[rt], sv[rt]);
+        fb[rt] = dequant_dword(q[rt][0], sv[rt][0]);
+      }
+#pragma unroll
+      for (int tt = 0; tt < TTC; ++tt) {
+        scale_pairs(as[tt], asv[tt]);
+        fa[tt] = dequant_dword(aq[tt][0], asv[tt][0]);
+      }
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        auto part_work = [&](int part) {  // parts 0 .. RT-1: weight tiles, RT .. RT+TTC-1: activation tiles
+          if (t == 3) return;
+          if (part < RT) fbn[part] = dequant_dword(q[part][t + 1], sv[part][(t + 1) >> 1]);
+          else fan[part - RT] = dequant_dword(aq[part - RT][t + 1], asv[part - RT][(t + 1) >> 1]);
+        };
+#pragma unroll
+        for (int tt = 0; tt < TTC; ++tt) {
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt)
+            acc[rt][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, fb[rt]), __builtin_bit_cast(f16x8, fa[tt]),
+                                                                 acc[rt][tt], 0, 0, 0);
+#pragma unroll
+          for (int part = tt * (RT + TTC) / TTC; part < (tt + 1) * (RT + TTC) / TTC; ++part) part_work(part);
+        }
+        if (t < 3) {
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt) fb[rt] = fbn[rt];
+#pragma unroll
+          for (int tt = 0; tt < TTC; ++tt) fa[tt] = fan[tt];
+        }
+      }
+    };
+    // One whole-slot refill per chunk, as in the kernels with few activation tiles: for tile counts whose
+    // accumulators leave no registers for the finer scheme.
+    auto chunk_coarse = [&](auto ttc_c, uint32_t c, auto& acc) {
+      constexpr int TTC = decltype(ttc_c)::value;
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      u32x4 q[RT];
+      uint32_t sc[RT];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) q[rt] = *reinterpret_cast<const u32x4*>(sp + rt * 1024 + rd_payload);
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) sc[rt] = *reinterpret_cast<const uint32_t*>(sp + rd_bsc[rt]) >> sc_shift;
+      u32x4 fb[RT][4];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) dequant_frags(q[rt], sc[rt], fb[rt]);
+#pragma unroll
+      for (int tt = 0; tt < TTC; ++tt) {
+        __builtin_amdgcn_sched_barrier(0);
+        u32x4 aq;
+        uint32_t as;
+        read_a_tile(tt, aq, as);
+        if (tt + 1 == TTC) {
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the last read of the slot is complete
+          if (c + CSTEP < (uint32_t)chunks) {
+            load_b_part(c + CSTEP);
+#pragma unroll
+            for (int t2 = 0; t2 < TTC; ++t2) {
+              load_a_tile(c + CSTEP, t2);
+              if ((t2 & 1) || t2 + 1 == TTC) load_a_scales(c + CSTEP, t2 >> 1);
+            }
+          }
+        }
+        u32x4 fa[4];
+        dequant_frags(aq, as, fa);
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt)
+            acc[rt][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, fb[rt][t]),
+                                                                 __builtin_bit_cast(f16x8, fa[t]), acc[rt][tt], 0, 0, 0);
+      }
+    };
+    // s_waitcnt vmcnt(n) for a wave-uniform n (the operand is an immediate)
+    auto wait_loads = [&](int n) {
+      switch (n) {
+#define NVF_VMCNT_CASE(n) case n: asm volatile("s_waitcnt vmcnt(" #n ")" ::: "memory"); break;
+        NVF_VMCNT_CASE(1) NVF_VMCNT_CASE(2) NVF_VMCNT_CASE(3) NVF_VMCNT_CASE(4) NVF_VMCNT_CASE(5) NVF_VMCNT_CASE(6)
+        NVF_VMCNT_CASE(7) NVF_VMCNT_CASE(8) NVF_VMCNT_CASE(9) NVF_VMCNT_CASE(10) NVF_VMCNT_CASE(11) NVF_VMCNT_CASE(12)
+        NVF_VMCNT_CASE(13) NVF_VMCNT_CASE(14) NVF_VMCNT_CASE(15) NVF_VMCNT_CASE(16) NVF_VMCNT_CASE(17) NVF_VMCNT_CASE(18)
+        NVF_VMCNT_CASE(19) NVF_VMCNT_CASE(20) NVF_VMCNT_CASE(21) NVF_VMCNT_CASE(22) NVF_VMCNT_CASE(23) NVF_VMCNT_CASE(24)
+        NVF_VMCNT_CASE(25) NVF_VMCNT_CASE(26) NVF_VMCNT_CASE(27) NVF_VMCNT_CASE(28) NVF_VMCNT_CASE(29) NVF_VMCNT_CASE(30)
+#undef NVF_VMCNT_CASE
+        default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      }
+    };
+    // one dword of an MFMA operand: two of a raw dword's eight values (byte `sel`), times their block's scale
+    auto dequant_pair = [&](uint32_t qw, int sel, f16x2 sv) {
+      const f16x2 h = (sel == 0   ? __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(qw, 1.0f, 0)
+                       : sel == 1 ? __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(qw, 1.0f, 1)
+                       : sel == 2 ? __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(qw, 1.0f, 2)
+                                  : __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(qw, 1.0f, 3)) * sv;
+      return __builtin_bit_cast(uint32_t, h);
+    };
+    // One chunk for tile counts whose accumulators leave no registers for the scheme above (RT * TTC > 20).  A
+    // wavefront issues one conversion instruction per 8 cycles at best and an MFMA of this shape per 16, so a chunk
+    // that converts a tile and then multiplies it takes the sum of both; here the two instructions that make one
+    // dword of an activation operand follow every MFMA, so that they issue while the matrix pipe works: the 8 MFMAs
+    // on the first half of a tile's K range (2 steps x RT weight tiles) carry the conversion of its second half, the 8
+    // on the second half that of the next tile's first half.  Only the weight operands of the whole chunk are
+    // converted up front.  A tile's raw bytes are read out of LDS one tile ahead and its slot is refilled with the
+    // wavefront's next chunk at once, the weight part right at the start of the chunk: every load has most of a
+    // chunk's time to land.  Loads complete in the order of issue, and that order is fixed - weight part, then per
+    // tile its bytes and, after every second tile and the last, the scale block of the pair - so the waits are for
+    // counts that follow from it.
+    auto chunk_pipe = [&](auto ttc_c, uint32_t c, auto& acc) {
+      constexpr int TTC = decltype(ttc_c)::value;
+      constexpr int NS = (TTC + 1) / 2, NA = TTC + NS, LB = RT + B_SC;
+      const bool has_next = c + CSTEP < (uint32_t)chunks;
+      // loads of this chunk still pending once tile tt and the scale block of its pair have landed
+      auto after_tile = [&](int tt) {
+        const int last_of_pair = (tt | 1) < TTC ? (tt | 1) : TTC - 1;
+        return NA - 1 - (last_of_pair + (last_of_pair >> 1) + 1);
+      };
+      wait_loads(NA);  // the weight part has landed
+      u32x4 q[RT];
+      uint32_t sc[RT];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) q[rt] = *reinterpret_cast<const u32x4*>(sp + rt * 1024 + rd_payload);
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) sc[rt] = *reinterpret_cast<const uint32_t*>(sp + rd_bsc[rt]) >> sc_shift;
+      wait_loads(after_tile(0));
+      u32x4 aq, aqn = {0, 0, 0, 0};
+      uint32_t as, asn = 0;
+      read_a_tile(0, aq, as);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // read out: may be refilled
+      if (has_next) {
+        load_b_part(c + CSTEP);
+        load_a_tile(c + CSTEP, 0);
+        if (TTC == 1) load_a_scales(c + CSTEP, 0);
+      }
+      u32x4 fb[RT][4];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        f16x2 sv[2];
+        scale_pairs(sc[rt], sv);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) fb[rt][t] = dequant_dword(q[rt][t], sv[t >> 1]);
+      }
+      f16x2 asv[2], asvn[2];
+      scale_pairs(as, asv);
+      u32x4 fa[2], fan[2];
+      fa[0] = dequant_dword(aq[0], asv[0]);
+      fa[1] = dequant_dword(aq[1], asv[0]);
+#pragma unroll
+      for (int tt = 0; tt < TTC; ++tt) {
+        __builtin_amdgcn_sched_barrier(0);
+        if (tt + 1 < TTC) {
+          // pending behind tile tt+1: the rest of this chunk's tiles, the next chunk's weight part and its tiles 0..tt
+          wait_loads(after_tile(tt + 1) + (has_next ? LB + (tt + 1) + ((tt + 1) >> 1) : 0));
+          read_a_tile(tt + 1, aqn, asn);
+        }
+        // K steps 0 and 1 of tile tt; behind every MFMA one dword of the operands of its steps 2 and 3
+#pragma unroll
+        for (int m = 0; m < 8; ++m) {
+          const int t = m >> 2, rt = m & 3;
+#pragma unroll
+          for (int r2 = rt; r2 < RT; r2 += 4)
+            acc[r2][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, fb[r2][t]), __builtin_bit_cast(f16x8, fa[t]),
+                                                                 acc[r2][tt], 0, 0, 0);
+          fan[m >> 2][m & 3] = dequant_pair(aq[2 + (m >> 2)], m & 3, asv[1]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        if (tt + 1 < TTC) {
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // tile tt+1 is in registers: its slot may be refilled
+          if (has_next) {
+            load_a_tile(c + CSTEP, tt + 1);
+            if (((tt + 1) & 1) || tt + 2 == TTC) load_a_scales(c + CSTEP, (tt + 1) >> 1);
+          }
+          scale_pairs(asn, asvn);
+        }
+        // K steps 2 and 3 of tile tt; behind every MFMA one dword of the next tile's operands of steps 0 and 1
+#pragma unroll
+        for (int m = 0; m < 8; ++m) {
+          const int t = m >> 2, rt = m & 3;
+#pragma unroll
+          for (int r2 = rt; r2 < RT; r2 += 4)
+            acc[r2][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, fb[r2][2 + t]), __builtin_bit_cast(f16x8, fan[t]),
+                                                                 acc[r2][tt], 0, 0, 0);
+          if (tt + 1 < TTC) fa[m >> 2][m & 3] = dequant_pair(aqn[m >> 2], m & 3, asvn[0]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        aq = aqn;
+        asv[1] = asvn[1];
+      }
+    };
+    auto run = [&](auto ttc_c) {
+      constexpr int TTC = decltype(ttc_c)::value;
+      constexpr bool kFits = RT * TTC <= 20;  // accumulator registers that leave room for the finer scheme
+      f32x4 acc[RT][TTC];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int tt = 0; tt < TTC; ++tt) acc[rt][tt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+      if (c_first < chunks) {
+        load_b_part((uint32_t)c_first);
+#pragma unroll
+        for (int tt = 0; tt < TTC; ++tt) {
+          load_a_tile((uint32_t)c_first, tt);
+          if ((tt & 1) || tt + 1 == TTC) load_a_scales((uint32_t)c_first, tt >> 1);
+        }
+      }
+      for (int c = c_first; c < chunks; c += CSTEP) {
+        if constexpr (!kFits && RT == 4) chunk_pipe(ttc_c, (uint32_t)c, acc);
+        else if constexpr (!kFits) chunk_coarse(ttc_c, (uint32_t)c, acc);
+        else chunk(ttc_c, (uint32_t)c, acc);
+      }
+      finish(ttc_c, acc);
+    };
+    switch (tt_count) {
+      case 1: run(std::integral_constant<int, 1>{}); break;
+      case 2: run(std::integral_constant<int, 2>{}); break;
+      case 3: run(std::integral_constant<int, 3>{}); break;
+      case 4: run(std::integral_constant<int, (TT >= 4 ? 4 : 1)>{}); break;
+      case 5: run(std::integral_constant<int, (TT >= 5 ? 5 : 1)>{}); break;
+      case 6: run(std::integral_constant<int, (TT >= 6 ? 6 : 1)>{}); break;
+      case 7: run(std::integral_constant<int, (TT >= 7 ? 7 : 1)>{}); break;
+      case 8: run(std::integral_constant<int, (TT >= 8 ? 8 : 1)>{}); break;
+      default: break;
+    }
+  } else {
+    f32x4 acc[RT][TT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int tt = 0; tt < TT; ++tt) acc[rt][tt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) issue_chunk(c_first + d * CSTEP, d);
+    int slot = 0;
+    for (int c = c_first; c < chunks; c += CSTEP) {
+      // the oldest chunk in flight has landed when only the loads of the next one (if there is one) are pending
+      if (DEPTH == 2 && c + CSTEP < chunks)
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NDMA) : "memory");
+      else
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      const char* sp = reinterpret_cast<const char*>(red) + (wave * DEPTH + slot) * SLOT_BYTES;
+      // the activation tiles are read out of LDS together with the weight tiles (few of them) or one at a time
+      // right before their conversion (many: their registers would not fit)
+      constexpr bool kLazyA = TT > 2;
+      constexpr int NQ = kLazyA ? RT : NT;
+      u32x4 q[NQ];
+      uint32_t sc[NQ];
+#pragma unroll
+      for (int t = 0; t < NQ; ++t) q[t] = *reinterpret_cast<const u32x4*>(sp + t * 1024 + rd_payload);
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) sc[rt] = *reinterpret_cast<const uint32_t*>(sp + rd_bsc[rt]) >> sc_shift;
+      if constexpr (!kLazyA) {
+#pragma unroll
+        for (int tt = 0; tt < TT; ++tt) sc[RT + tt] = *reinterpret_cast<const uint32_t*>(sp + rd_asc[tt]) >> sc_shift;
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // read out: the slot may be refilled
+        issue_chunk(c + DEPTH * CSTEP, slot);
+      }
+      u32x4 fb[RT][4];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) dequant_frags(q[rt], sc[rt], fb[rt]);
+#pragma unroll
+      for (int tt = 0; tt < TT; ++tt) {
+        if (tt < tt_count) {
+          u32x4 aq;
+          uint32_t as;
+          if constexpr (kLazyA) {
+            aq = *reinterpret_cast<const u32x4*>(sp + (RT + tt) * 1024 + rd_payload);
+            as = *reinterpret_cast<const uint32_t*>(sp + rd_asc[tt]) >> sc_shift;
+            if (tt + 1 == tt_count) {
+              asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the last read of the slot is complete
+              issue_chunk(c + DEPTH * CSTEP, slot);
+            }
+          } else {
+            aq = q[kLazyA ? 0 : RT + tt];
+            as = sc[kLazyA ? 0 : RT + tt];
+          }
+          u32x4 fa[4];
+          dequant_frags(aq, as, fa);
+#pragma unroll
+          for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+              acc[rt][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, fb[rt][t]),
+                                                                   __builtin_bit_cast(f16x8, fa[t]), acc[rt][tt], 0, 0, 0);
+        }
+      }
+      if constexpr (DEPTH == 2) slot ^= 1;
+    }
+    finish(std::integral_constant<int, TT>{}, acc);
+  }
+}
+
+template <int RT, int TT, bool OUT_BF16>
+int launch_nvfp4_skinny_ring_cfg(const Params& p, hipStream_t stream, int slabs = 1) {
+  constexpr int SLOT_KIB = RT + TT + (RT + 1) / 2 + (TT + 1) / 2;
+  // one slot per wavefront also where two would fit (M=16, N=14336, K=4096: 8.0 -> 7.5 us; K=14336: 9.6 -> 9.2 us)
+  constexpr int DEPTH = 1;
+  auto kern = nvfp4_skinny_ring_kernel<RT, TT, OUT_BF16, DEPTH>;
+  // the ring; the reduction reuses it and needs 8 KiB per partial tile of a round
+  constexpr int red_kib = 8 * (RT * TT <= 8 ? RT * TT : TT);
+  constexpr int ring_kib = 8 * DEPTH * SLOT_KIB;
+  constexpr int lds_bytes = (ring_kib > red_kib ? ring_kib : red_kib) * 1024;
+  static_assert(lds_bytes <= 160 * 1024, "LDS");
+  const int splits = p.partial != nullptr ? p.splits : 1;
+  if (splits > 1 ? note_launch("nvfp4_skinny_ring_kernel<RT=%d,TT=%d> grid=%ux%dx%d split_k + splitk_reduce_kernel", RT, TT,
+                               (unsigned)(p.n / (16 * RT)), slabs, splits)
+                 : note_launch("nvfp4_skinny_ring_kernel<RT=%d,TT=%d> grid=%ux%d", RT, TT, (unsigned)(p.n / (16 * RT)), slabs))
+    return NVF_OK;
+  static std::atomic<uint64_t> configured{0};  // one bit per device
+  if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
+  hipLaunchKernelGGL(kern, dim3((unsigned)(p.n / (16 * RT)), (unsigned)slabs, (unsigned)splits), dim3(512), lds_bytes, stream, p);
+  if (const int rc = check_launch("nvfp4_skinny_ring_kernel")) return rc;
+  if (p.partial == nullptr) return NVF_OK;
+  const int64_t mn = (int64_t)p.m * p.n;
+  hipLaunchKernelGGL(splitk_reduce_kernel<OUT_BF16>, dim3((unsigned)ceil_div(mn / 4, 256)), dim3(256), 0, stream, p.partial, splits, mn, p.alpha,
+                     static_cast<uint16_t*>(p.out));
+  return check_launch("splitk_reduce_kernel");
+}
+
+template <int RT, int TT, bool OUT_BF16, bool NSPLIT>
+int launch_nvfp4_skinny_grouped(const Params& p0, int rows_lo, int rows_hi, hipStream_t stream) {
+  constexpr int SLOT_KIB = RT + TT + (RT + 1) / 2 + (TT + 1) / 2;
+  // One slot per wavefront also where two would fit: measured faster for the groups of up to 32 rows (512 rows
+  // over 256 experts, K=7168: 401 -> 375 us; K=2048: 432 -> 413 us).  Forcing the registers down to two
+  // workgroups per compute unit on top of that costs more than it gains (450 us).
+  constexpr int DEPTH = 1;
+  auto kern = nvfp4_skinny_ring_kernel<RT, TT, OUT_BF16, DEPTH, true, NSPLIT>;
+  constexpr int red_kib = NSPLIT ? 0 : 8 * (RT * TT <= 8 ? RT * TT : TT);
+  constexpr int ring_kib = 8 * DEPTH * SLOT_KIB;
+  constexpr int lds_bytes = (ring_kib > red_kib ? ring_kib : red_kib) * 1024;
+  static_assert(lds_bytes <= 160 * 1024, "LDS");
+  Params p = p0;
+  p.rows_lo = rows_lo;
+  p.rows_hi = rows_hi;
+  const int64_t wgs = (int64_t)p.groups * (p.n / (16 * RT * (NSPLIT ? 8 : 1)));
+  if (wgs >= ((int64_t)1 << 31)) return fail(NVF_ERR_UNSUPPORTED_SHAPE, "too many (group, row block) pairs for one launch");
+  if (note_launch("nvfp4_skinny_ring_kernel<RT=%d,TT=%d,grouped,nsplit=%d> grid=%lld rows=%d..%d", RT, TT, (int)NSPLIT, (long long)wgs, rows_lo,
+                  rows_hi))
+    return NVF_OK;
+  static std::atomic<uint64_t> configured{0};  // one bit per device
+  if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
+  hipLaunchKernelGGL(kern, dim3((unsigned)wgs), dim3(512), lds_bytes, stream, p);
+  return check_launch("nvfp4_skinny_ring_kernel (grouped)");
+}
+
+template <int TT, bool OUT_BF16>
+int launch_nvfp4_skinny_rt(const Params& p, int rt, hipStream_t stream, int slabs) {
+  return rt == 4 ? launch_nvfp4_skinny_ring_cfg<4, TT, OUT_BF16>(p, stream, slabs)
+       : rt == 2 ? launch_nvfp4_skinny_ring_cfg<2, TT, OUT_BF16>(p, stream, slabs)
+                 : launch_nvfp4_skinny_ring_cfg<1, TT, OUT_BF16>(p, stream, slabs);
+}
+
+// Cost, in arbitrary units, of streaming the weights against M activation rows as slabs of `slab` rows with rt weight
+// tiles (16 rows) per workgroup.  Every workgroup converts rt weight tiles and the tt row tiles of its slab per
+// 128-deep chunk (a wavefront takes every eighth chunk), so few large workgroups convert least, while small ones (less
+// LDS, fewer accumulators) share a compute unit and fill the chip at small N.  The constants are a fit to timings of
+// the nine (slab, rt) forms over M = 48..256, N = 1024..14336, K = 2048..14336 (144 shapes: the form picked is within
+// 8 % of the fastest for 134 of them, 1.8 % off on average; a fixed rule by N alone was 13 % off); for 1..32 rows
+// (112 shapes) its pick of rt is 0.2 % off the fastest on average.
+int64_t nvfp4_skinny_cost(int64_t m, int64_t n, int64_t k, int slab, int rt, int cus) {
+  if (n % (16 * rt) != 0) return INT64_MAX;
+  const int64_t slabs = m <= slab ? 1 : ceil_div(m, slab);
+  const int tt = m <= slab ? (m <= 16 ? 1 : m <= 32 ? 2 : m <= 64 ? 4 : 8) : slab / 16;
+  const int64_t wgs = slabs * (n / (16 * rt));
+  const int lds_kib = 8 * (rt + tt + (rt + 1) / 2 + (tt + 1) / 2);
+  int64_t per_cu = std::min(160 / lds_kib, 4);  // workgroups that share a compute unit
+  if (rt * tt > 16) per_cu = 1;                 // (their accumulators take the registers)
+  else if (rt * tt > 6) per_cu = std::min<int64_t>(per_cu, 2);
+  if (per_cu < 1) per_cu = 1;
+  const int64_t chunks = ceil_div(k >> 7, 8);
+  const int64_t resident = std::min(per_cu, ceil_div(wgs, cus));
+  const int64_t rounds = ceil_div(wgs, cus * per_cu);
+  const int64_t per_chunk = (rt + tt) * 183 + rt * tt * 18 + 100;
+  const int64_t wg_time = chunks * per_chunk * (100 + 73 * (resident - 1)) / 100 + rt * tt * 110 + 5070;
+  return rounds * wg_time;
+}
+
+// best (slab height, weight tiles per workgroup) for more than 32 rows and its estimated cost
+int64_t nvfp4_skinny_best(int64_t m, int64_t n, int64_t k, int cus, int* slab_out, int* rt_out) {
+  int slab = 128, rt = 1;
+  int64_t best = INT64_MAX;
+  for (const int s : {128, 64, 32})
+    for (const int r : {4, 2, 1}) {
+      const int64_t c = nvfp4_skinny_cost(m, n, k, s, r, cus);
+      if (c < best) best = c, slab = s, rt = r;
+    }
+  if (slab_out) *slab_out = slab;
+  if (rt_out) *rt_out = rt;
+  return best;
+}
+
+template <bool OUT_BF16>
+int launch_nvfp4_skinny(const Params& p, int cus, hipStream_t stream) {
+  // Up to 32 rows: one slab of 1 or 2 row tiles (16 x 6144 x 7168: 8.0 us with 1 weight tile per workgroup, 7.0 with 2).
+  // More rows: slabs of 128, 64 or 32 rows side by side in one launch (blockIdx.y = slab; the last one may be ragged;
+  // the slabs after the first find the weights in the last-level cache) with 1, 2 or 4 weight tiles per workgroup,
+  // whichever the cost estimate above prefers (M=128, N=4096, K=4096: 10.8 us as two slabs of 64 rows x 1 weight tile,
+  // 8.3 us x 2 tiles; M=256, N=4096, K=14336: 62 -> 34 us; M=256, N=6144, K=7168: 48 -> 29 us).
+  int slab, rt;
+  nvfp4_skinny_best(p.m, p.n, p.k, cus, &slab, &rt);
+  if (p.m > slab) {
+    const int slabs = (int)ceil_div(p.m, slab);
+    return slab == 128 ? launch_nvfp4_skinny_rt<8, OUT_BF16>(p, rt, stream, slabs)
+         : slab == 64  ? launch_nvfp4_skinny_rt<4, OUT_BF16>(p, rt, stream, slabs)
+                       : launch_nvfp4_skinny_rt<2, OUT_BF16>(p, rt, stream, slabs);
+  }
+  return p.m <= 16 ? launch_nvfp4_skinny_rt<1, OUT_BF16>(p, rt, stream, 1)
+       : p.m <= 32 ? launch_nvfp4_skinny_rt<2, OUT_BF16>(p, rt, stream, 1)
+       : p.m <= 64 ? launch_nvfp4_skinny_rt<4, OUT_BF16>(p, rt, stream, 1)
+                   : launch_nvfp4_skinny_rt<8, OUT_BF16>(p, rt, stream, 1);
+}
