@@ -409,8 +409,10 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int6
 // product itself (that op's optional dump of what it quantized).  Both take the same kernel for a shape, so that
 // the dump holds exactly the accumulators the quantized result was made from.
 template <bool FP4>
+int launch_nvfp4_wide_part(const Params& p, int cus, hipStream_t stream);
+
+template <bool FP4>
 int launch_nvfp4_wide(const Params& p, int cus, hipStream_t stream) {
-  auto tiles = [&](int bm, int bn) { return ceil_div(p.m, bm) * ceil_div(p.n, bn); };
   if (FP4 && ((p.m & 127) != 0 || ((p.n >> 4) & 3) != 0)) {
     // ragged: the padding rows / columns of the scale buffer's last 128x4 tiles are written as zero first
     const int64_t words = round_up(p.m, 128) * round_up(p.n >> 4, 4) / 4;
@@ -419,6 +421,26 @@ int launch_nvfp4_wide(const Params& p, int cus, hipStream_t stream) {
       if (const int rc = check_launch("zero_fill_kernel")) return rc;
     }
   }
+  if ((p.n & 255) == 0 && (p.k & 127) == 0 && p.k >= 256 && p.m > 256 && (p.m & 127) != 0 && ceil_div(p.m / 128 * 128, 128) * (p.n / 256) >= cus / 2) {
+    // M not a multiple of 128 and enough rows for the persistent kernel: the rows up to the last multiple of 128 go
+    // there, the rest to the tile kernels (their part of the result and of its scale tiles starts a whole number of
+    // 128-row tiles further on)
+    Params main = p, rest = p;
+    main.m = p.m & ~127;
+    rest.m = p.m - main.m;
+    rest.a = p.a + (int64_t)main.m * (p.k >> 1);
+    rest.sfa = p.sfa + (int64_t)main.m * round_up(p.k >> 4, 4);
+    rest.out = static_cast<uint8_t*>(p.out) + (FP4 ? (int64_t)main.m * (p.n >> 1) : (int64_t)main.m * p.n * 4);
+    if (FP4) rest.out_sf = p.out_sf + (int64_t)main.m * round_up(p.n >> 4, 4);
+    if (const int rc = launch_nvfp4_wide_part<FP4>(main, cus, stream)) return rc;
+    return launch_nvfp4_wide_part<FP4>(rest, cus, stream);
+  }
+  return launch_nvfp4_wide_part<FP4>(p, cus, stream);
+}
+
+template <bool FP4>
+int launch_nvfp4_wide_part(const Params& p, int cus, hipStream_t stream) {
+  auto tiles = [&](int bm, int bn) { return ceil_div(p.m, bm) * ceil_div(p.n, bn); };
   if ((p.n & 255) == 0 && (p.k & 127) == 0 && p.k >= 256) {
     // as for the 16-bit results: persistent 256x256 or 128x256 tiles where they fill the compute units
     const int64_t t256 = (p.m & 255) == 0 ? tiles(256, 256) : 0, t128 = (p.m & 127) == 0 ? tiles(128, 256) : 0;
