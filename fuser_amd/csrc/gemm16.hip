@@ -63,6 +63,10 @@ struct Params {
   // layout of [roundUp(m,128), roundUp(n/16,4)], gnorm = the result's global (encode) scale on the device
   uint8_t* out_sf = nullptr;
   const float* gnorm = nullptr;
+  // dense NVFP4 with a 16-bit result: elements between rows of the result; 0: n (a launch that computes some of the
+  // columns sets it)
+  int ldc = 0;
+  __host__ __device__ int out_pitch() const { return ldc ? ldc : n; }
 };
 
 __device__ __forceinline__ uint32_t pack2(float a, float b, bool out_bf16) {
@@ -480,6 +484,7 @@ int launch_gemm16(int op, const Gemm16Args& a, hipStream_t stream) {
   p.m = (int)a.m;
   p.n = (int)a.n;
   p.k = (int)a.k;
+  p.ldc = (int)a.ldc;
   const int cus = cu_count();
   const bool bf16 = a.dtype == NVF_BF16;
   if (op == 0 && a.dtype == NVF_F32) return launch_nvfp4_wide<false>(p, cus, stream);
@@ -497,6 +502,28 @@ int launch_gemm16(int op, const Gemm16Args& a, hipStream_t stream) {
     // kernels: the rows up to the last multiple of 128 go to whatever kernel that shape gets, the remaining rows
     // (at most 127, a whole number of 128-row scale tiles further on) to the weight-streaming kernel in a launch of
     // their own (4000 x 4096 x 4096: 145 -> 116 us; 8100 x 8192 x 8192: 1002 -> 850 us).
+    // Dense with N not a multiple of 256 (29568, 1408) and enough rows for the persistent kernel: the columns up to the
+    // last multiple of 256 go to whatever kernel that shape gets, the remaining columns (weight rows) to a launch of
+    // their own that writes into the same rows of the result.
+    if (op == 0 && (p.n & 255) != 0 && p.n > 256 && p.m >= 512 && (p.k & 127) == 0 && p.k >= 256) {
+      const DensePlan::Kernel main_kernel = nvfp4_dense_plan(p.m & ~127, p.n & ~255, p.k, cus).kernel;
+      if (main_kernel == DensePlan::kStream)  // (takes any M and any N % 16 == 0)
+        return bf16 ? launch_nvfp4_skinny<true>(p, cus, stream) : launch_nvfp4_skinny<false>(p, cus, stream);
+      if (main_kernel != DensePlan::kOther) {
+        Gemm16Args main = a, rest = a;
+        main.n = p.n & ~255;
+        rest.n = p.n - main.n;
+        main.ldc = rest.ldc = a.ldc ? a.ldc : a.n;
+        main.workspace = rest.workspace = nullptr;  // (a split of K keeps partial results at the pitch of its own N)
+        main.workspace_bytes = rest.workspace_bytes = 0;
+        const int64_t sf_padded = ((int64_t)(p.k >> 4) + 3) & ~(int64_t)3;
+        rest.b = static_cast<const uint8_t*>(a.b) + main.n * (p.k >> 1);
+        rest.sfb = static_cast<const uint8_t*>(a.sfb) + main.n * sf_padded;
+        rest.out = static_cast<uint8_t*>(a.out) + main.n * 2;
+        if (const int rc = launch_gemm16(op, main, stream)) return rc;
+        return launch_gemm16(op, rest, stream);
+      }
+    }
     const int64_t main_rows = op == 0 ? nvfp4_rows_before_remainder(p.m, p.n, p.k, cus) : 0;
     if (main_rows == p.m) return bf16 ? launch_nvfp4_skinny<true>(p, cus, stream) : launch_nvfp4_skinny<false>(p, cus, stream);
     if (main_rows) {
@@ -506,7 +533,7 @@ int launch_gemm16(int op, const Gemm16Args& a, hipStream_t stream) {
       const int64_t sf_padded = ((int64_t)(p.k >> 4) + 3) & ~(int64_t)3;
       rest.a = p.a + (int64_t)main.m * (p.k >> 1);
       rest.sfa = p.sfa + (int64_t)main.m * sf_padded;
-      rest.out = static_cast<uint8_t*>(p.out) + (int64_t)main.m * p.n * 2;
+      rest.out = static_cast<uint8_t*>(p.out) + (int64_t)main.m * p.out_pitch() * 2;
       if (const int rc = launch(main, a.workspace, a.workspace_bytes)) return rc;
       return launch(rest, nullptr, 0);
     }

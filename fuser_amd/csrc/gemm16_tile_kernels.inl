@@ -448,7 +448,7 @@ __global__ __launch_bounds__(256) void nvfp4_tile_kernel(const Params p) {
             *reinterpret_cast<f32x4*>(frow + ncol) = f32x4{acc[i][j][rq * 4 + 0] * alpha, acc[i][j][rq * 4 + 1] * alpha,
                                                            acc[i][j][rq * 4 + 2] * alpha, acc[i][j][rq * 4 + 3] * alpha};
           } else {
-            uint16_t* orow = static_cast<uint16_t*>(p.out) + (row_off + mrow) * (int64_t)p.n;
+            uint16_t* orow = static_cast<uint16_t*>(p.out) + (row_off + mrow) * (int64_t)p.out_pitch();
             u32x2 v;
             v[0] = pack2(acc[i][j][rq * 4 + 0] * alpha, acc[i][j][rq * 4 + 1] * alpha, OUT_BF16);
             v[1] = pack2(acc[i][j][rq * 4 + 2] * alpha, acc[i][j][rq * 4 + 3] * alpha, OUT_BF16);

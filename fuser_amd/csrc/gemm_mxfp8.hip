@@ -29,6 +29,8 @@ struct Params {
   void* out;
   int m, n, k;
   int m_base = 0;  // skinny kernel: first activation row this launch computes, a multiple of the slab height (32, 64 or 128)
+  int ldc = 0;     // elements between rows of the result; 0: n (a launch that computes some of the columns sets it)
+  __host__ __device__ int out_pitch() const { return ldc ? ldc : n; }
 };
 
 __device__ __forceinline__ uint32_t pack2(float a, float b, bool out_bf16) {
@@ -191,7 +193,7 @@ __global__ __launch_bounds__(256) void mxfp8_gemm_kernel(const Params p) {
   for (int i = 0; i < TM; ++i) {
     const int mrow = m0 + wm * WTM + i * 32 + li;
     if (mrow >= p.m) continue;
-    uint16_t* orow = out + (int64_t)mrow * p.n;
+    uint16_t* orow = out + (int64_t)mrow * p.out_pitch();
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
 #pragma unroll
@@ -259,13 +261,20 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
   const int chunk_tiles = (total + 7) >> 3;
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, slots = gridDim.x >> 3;
   const int range_end = min((xcd + 1) * chunk_tiles, total);
-  const bool blocked = (tiles_m & 7) == 0 && (tiles_n & 3) == 0;
+  // (n-tiles past the last multiple of 4: blocks of 8 (m) x 1..3 (n) after all the others; 8192 x 29440 x 8192, 115
+  // n-tiles: 2.33 -> 2.7 PFLOP/s against the plain m-major order)
+  const bool blocked = (tiles_m & 7) == 0 && tiles_n >= 4;
+  const int bulk_tiles = tiles_m * (tiles_n & ~3);
   auto tile_coords = [&](int t, int& m0, int& n0) {
     int mt, nt;
-    if (blocked) {
+    if (blocked && t < bulk_tiles) {
       const int sb = t >> 5, w = t & 31;
       mt = (sb % (tiles_m >> 3)) * 8 + (w & 7);
       nt = (sb / (tiles_m >> 3)) * 4 + (w >> 3);
+    } else if (blocked) {
+      const int u = t - bulk_tiles, bs = 8 * (tiles_n & 3), sb = u / bs, w = u - sb * bs;
+      mt = sb * 8 + (w & 7);
+      nt = (tiles_n & ~3) + (w >> 3);
     } else {
       mt = t % tiles_m;
       nt = t / tiles_m;
@@ -463,8 +472,9 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
     uint8_t* stage = reinterpret_cast<uint8_t*>(lds + 2 * BUF_UNITS) + wave * 4608;
     uint8_t* wr = stage + (elane & 31) * 144 + (elane >> 5) * 8;
     const uint8_t* rd = stage + (elane >> 3) * 144 + (elane & 7) * 16;
-    const uint32_t ooff = ((uint32_t)(elane >> 3) * (uint32_t)p.n + (uint32_t)(elane & 7) * 8u) * 2u;
-    uint8_t* obase = reinterpret_cast<uint8_t*>(static_cast<uint16_t*>(p.out) + (int64_t)(m0 + wm * (32 * TM)) * p.n + n0 + wn * 128);
+    const int ldc = p.out_pitch();
+    const uint32_t ooff = ((uint32_t)(elane >> 3) * (uint32_t)ldc + (uint32_t)(elane & 7) * 8u) * 2u;
+    uint8_t* obase = reinterpret_cast<uint8_t*>(static_cast<uint16_t*>(p.out) + (int64_t)(m0 + wm * (32 * TM)) * ldc + n0 + wn * 128);
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
@@ -484,7 +494,7 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
           const u32x4 v = *reinterpret_cast<const u32x4*>(rd + t * 1152);
-          u32x4* dst = reinterpret_cast<u32x4*>(obase + ((int64_t)(i * 32 + 8 * t) * p.n + jh * 64) * 2 + ooff);
+          u32x4* dst = reinterpret_cast<u32x4*>(obase + ((int64_t)(i * 32 + 8 * t) * ldc + jh * 64) * 2 + ooff);
           if constexpr (STREAM_OUT) __builtin_nontemporal_store(v, dst);
           else *dst = v;
         }
@@ -688,7 +698,7 @@ __global__ __launch_bounds__(512) void mxfp8_skinny_kernel(const Params p) {
       u32x2 v;
       v[0] = pack2(s[0] * alpha, s[1] * alpha, OUT_BF16);
       v[1] = pack2(s[2] * alpha, s[3] * alpha, OUT_BF16);
-      *reinterpret_cast<u32x2*>(out + (int64_t)(m_base + tok) * p.n + n0 + rt * 16 + 4 * (l >> 4)) = v;
+      *reinterpret_cast<u32x2*>(out + (int64_t)(m_base + tok) * p.out_pitch() + n0 + rt * 16 + 4 * (l >> 4)) = v;
     }
   }
 }
@@ -832,6 +842,23 @@ int launch_sized(const Params& p, hipStream_t stream) {
     case Plan::kTiles128: return launch_fast<2, OUT_BF16>(p, stream);
     case Plan::kOther: break;
   }
+  // N not a multiple of 256 (29568, 1408) with enough rows for the persistent kernel: the columns up to the last
+  // multiple of 256 go to whatever kernel that shape gets, the remaining columns (weight rows) to a launch of their
+  // own that writes into the same rows of the result (8192 x 29568 x 8192: 4.1 -> 1.3 ms).
+  if ((p.n & 255) != 0 && p.n > 256 && (p.n & 15) == 0 && p.m >= 512 && (p.k & 127) == 0 && p.k >= 256 &&
+      mxfp8_plan(p.m & ~127, p.n & ~255, p.k, cus) != Plan::kOther) {
+    if (mxfp8_plan(p.m & ~127, p.n & ~255, p.k, cus) == Plan::kStream) return launch_skinny<OUT_BF16>(p, stream);  // (takes any N % 16 == 0)
+    Params main = p, rest = p;
+    main.n = p.n & ~255;
+    rest.n = p.n - main.n;
+    main.ldc = rest.ldc = p.out_pitch();
+    const int64_t sf_padded = ((int64_t)(p.k >> 5) + 3) & ~(int64_t)3;
+    rest.b = p.b + (int64_t)main.n * p.k;
+    rest.sfb = p.sfb + (int64_t)main.n * sf_padded;
+    rest.out = static_cast<uint8_t*>(p.out) + (int64_t)main.n * 2;
+    if (const int rc = launch_sized<OUT_BF16>(main, stream)) return rc;
+    return launch_sized<OUT_BF16>(rest, stream);
+  }
   // M not a multiple of 128 (a prefill of any token count) and too many rows for the skinny kernel: the rows up to
   // the last multiple of 128 go to whatever kernel that shape gets, the remaining rows (at most 127, a whole number
   // of 128-row scale tiles further on) to the skinny kernel in a launch of their own (4000 x 4096 x 4096: 197 -> 77 us;
@@ -854,7 +881,7 @@ int launch_sized(const Params& p, hipStream_t stream) {
       const int64_t sf_padded = ((int64_t)(p.k >> 5) + 3) & ~(int64_t)3;
       rest.a = p.a + (int64_t)cut * p.k;
       rest.sfa = p.sfa + (int64_t)cut * sf_padded;
-      rest.out = static_cast<uint8_t*>(p.out) + (int64_t)cut * p.n * 2;
+      rest.out = static_cast<uint8_t*>(p.out) + (int64_t)cut * p.out_pitch() * 2;
       if (const int rc = launch_sized<OUT_BF16>(main, stream)) return rc;
       return launch_sized<OUT_BF16>(rest, stream);
     }

@@ -82,6 +82,7 @@ struct Gemm16Args {
   // layout), gnorm = the result's global scale on the device
   void* out_sf = nullptr;
   const float* gnorm = nullptr;
+  int64_t ldc = 0;  // dense NVFP4, 16-bit result: elements between rows of the result (0: n); set by the N cut's launches
 };
 constexpr int kDtypeFp4BlockScaled = 100;  // internal result type code of launch_gemm16, next to nvf_dtype
 int launch_gemm16(int op, const Gemm16Args& args, hipStream_t stream);

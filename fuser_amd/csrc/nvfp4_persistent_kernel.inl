@@ -91,7 +91,9 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   const int chunk_tiles = (total + 7) >> 3;
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, slots = gridDim.x >> 3;
   const int range_end = min((xcd + 1) * chunk_tiles, total);
-  const bool blocked = (tiles_m & 7) == 0 && (tiles_n & 3) == 0;
+  // (n-tiles past the last multiple of 4: blocks of 8 (m) x 1..3 (n) after all the others)
+  const bool blocked = (tiles_m & 7) == 0 && tiles_n >= 4;
+  const int bulk_tiles = tiles_m * (tiles_n & ~3);
   // tile -> group, first row of the tile among all rows of A (m0), among the rows of the group (gm0), n0
   struct Where { int g; int64_t m0; int gm0, n0, valid; };  // valid: rows of the tile that exist (grouped: the last tile of a group)
   auto tile_where = [&](int t) {
@@ -117,10 +119,14 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
       w.valid = min(BM, m_g - w.gm0);
     } else {
       int mt, nt;
-      if (blocked) {
+      if (blocked && t < bulk_tiles) {
         const int sb = t >> 5, q = t & 31;
         mt = (sb % (tiles_m >> 3)) * 8 + (q & 7);
         nt = (sb / (tiles_m >> 3)) * 4 + (q >> 3);
+      } else if (blocked) {
+        const int u = t - bulk_tiles, bs = 8 * (tiles_n & 3), sb = u / bs, q = u - sb * bs;
+        mt = sb * 8 + (q & 7);
+        nt = (tiles_n & ~3) + (q >> 3);
       } else {
         mt = t % tiles_m;
         nt = t / tiles_m;
@@ -457,8 +463,9 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
       uint8_t* stage = reinterpret_cast<uint8_t*>(lds + 2 * BUF_UNITS) + wave * 2560;
       uint8_t* wr = stage + (elane & 31) * 80 + (elane >> 5) * 8;
       const uint8_t* rd = stage + (elane >> 2) * 80 + (elane & 3) * 16;
-      const uint32_t ooff = ((uint32_t)(elane >> 2) * (uint32_t)p.n + (uint32_t)(elane & 3) * 8u) * 2u;
-      uint8_t* obase = reinterpret_cast<uint8_t*>(static_cast<uint16_t*>(p.out) + (cw.m0 + wm * (32 * TM)) * p.n + cw.n0 + wn * 64);
+      const int ldc = p.out_pitch();
+      const uint32_t ooff = ((uint32_t)(elane >> 2) * (uint32_t)ldc + (uint32_t)(elane & 3) * 8u) * 2u;
+      uint8_t* obase = reinterpret_cast<uint8_t*>(static_cast<uint16_t*>(p.out) + (cw.m0 + wm * (32 * TM)) * ldc + cw.n0 + wn * 64);
       const int erow = elane >> 2;
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
@@ -477,7 +484,7 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
             const int brow = i * 32 + 16 * t;  // first of the 16 rows of this piece, in the wavefront's tile
             const u32x4 v = *reinterpret_cast<const u32x4*>(rd + t * 1280);
             if (!GROUPED || wm * (32 * TM) + brow + erow < cw.valid)
-              *reinterpret_cast<u32x4*>(obase + ((int64_t)brow * p.n + j * 32) * 2 + ooff) = v;
+              *reinterpret_cast<u32x4*>(obase + ((int64_t)brow * ldc + j * 32) * 2 + ooff) = v;
           }
           asm volatile("" ::: "memory");
         }

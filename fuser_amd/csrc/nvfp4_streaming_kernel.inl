@@ -173,7 +173,7 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
             u32x2 v;
             v[0] = pack2(acc[rt][tt][0] * alpha, acc[rt][tt][1] * alpha, OUT_BF16);
             v[1] = pack2(acc[rt][tt][2] * alpha, acc[rt][tt][3] * alpha, OUT_BF16);
-            *reinterpret_cast<u32x2*>(out + (a_row0 + tok) * p.n + n0 + rt * 16 + 4 * g) = v;
+            *reinterpret_cast<u32x2*>(out + (a_row0 + tok) * p.out_pitch() + n0 + rt * 16 + 4 * g) = v;
           }
         }
       }
@@ -205,9 +205,10 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
         for (int w = 1; w < W; ++w) s += red[w * units + u];
         const int tok = tt * 16 + (l & 15);
         if (tok < m_loc) {
-          const int64_t at = (a_row0 + tok) * p.n + n0 + (round * RPR + r2) * 16 + 4 * (l >> 4);
+          const int col = n0 + (round * RPR + r2) * 16 + 4 * (l >> 4);
+          const int64_t at = (a_row0 + tok) * p.out_pitch() + col;
           if (!GROUPED && p.partial != nullptr) {  // this K range's sums as they are; the reduction applies alpha
-            *reinterpret_cast<f32x4*>(p.partial + (int64_t)blockIdx.z * p.m * p.n + at) = s;
+            *reinterpret_cast<f32x4*>(p.partial + ((int64_t)blockIdx.z * p.m + a_row0 + tok) * p.n + col) = s;
           } else {
             u32x2 v;
             v[0] = pack2(s[0] * alpha, s[1] * alpha, OUT_BF16);

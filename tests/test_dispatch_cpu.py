@@ -106,6 +106,15 @@ def test_dense_m_not_a_multiple_of_128_is_cut_into_a_main_part_and_a_remainder(o
     assert "; " not in plan(op, 4096, 4096, 4096) and "; " not in plan(op, 300, 4096, 4096)
 
 
+@pytest.mark.parametrize("op", ["nvfp4_scaled_mm", "mxfp8_scaled_mm"])
+def test_dense_n_not_a_multiple_of_256_is_cut_into_a_main_part_and_the_remaining_columns(op):
+    got = plan(op, 8192, 29568, 8192).split("; ")
+    assert len(got) == 2 and "gemm_256_kernel<" in got[0] and "TM=4" in got[0] and "grid=256" in got[0] and "skinny" in got[1], got
+    # few rows: the weight-streaming kernel takes any N % 16 == 0 in one launch
+    got = plan(op, 300, 29568, 4096).split("; ")
+    assert len(got) == 1 and "skinny" in got[0], got
+
+
 def test_nvfp4_8192_cubed_takes_the_persistent_256x256_kernel():
     assert plan("nvfp4_scaled_mm", 8192, 8192, 8192).startswith("nvfp4_gemm_256_kernel<grouped=0,TM=4,f32=0,pairs=1> grid=256")
 

@@ -329,6 +329,41 @@ def test_dense_gemms_with_m_not_a_multiple_of_128(dev, shape):
     assert all("; " in p for p in plans) or shape == (1000, 2048, 256), plans  # (the last shape: cut for MXFP8 only)
 
 
+@pytest.mark.parametrize("shape", [(2048, 2432, 256), (2100, 2368, 384), (1536, 4128, 256), (640, 4224, 2048), (2048, 4224, 2048)])
+def test_dense_gemms_with_n_not_a_multiple_of_256(dev, shape):
+    """N > 256 and not a multiple of 256 with 512 rows or more: the columns up to the last multiple of 256 go to the
+    persistent kernel, the remaining 32..224 columns to a launch of their own (tile kernel or weight-streaming kernel)
+    that writes into the same rows of the result at the full row pitch; the second shape is cut along M as well.  Both
+    ops, both output types, every element against the oracle (a launch writing at the wrong pitch would show), run-to-run
+    bit equality."""
+    from fuser_amd import capi
+
+    m, n, k = shape
+    gen = torch.Generator().manual_seed(m + n + k)
+    a, sa, ga = _nvfp4_operand(m, k, 1.0, gen)
+    b, sb, gb = _nvfp4_operand(n, k, 0.02, gen)
+    alpha = 1.0 / (ga * gb)
+    ref = O.ref_nvfp4_scaled_mm(a, b, sa, sb, alpha)
+    plans = [capi.describe_dispatch("nvfp4_scaled_mm", m, n, k)]
+    for dtype in (torch.bfloat16, torch.float16):
+        out = _run_nvfp4(a, b, sa, sb, alpha, dtype, dev)
+        assert out.shape == (m, n) and max_rel_rowwise(out, ref) <= GEMM_MAX_REL, (shape, dtype, plans[-1])
+        assert torch.equal(out, _run_nvfp4(a, b, sa, sb, alpha, dtype, dev))
+    a8, sa8 = _mxfp8_operand(m, k, gen, 1.0)
+    b8, sb8 = _mxfp8_operand(n, k, gen, 1.0)
+    ref = O.ref_mxfp8_scaled_mm(a8, b8, sa8, sb8, 0.75)
+    scale = ref.abs().amax(dim=1, keepdim=True).clamp(min=1e-30)
+    plans.append(capi.describe_dispatch("mxfp8_scaled_mm", m, n, k))
+    for dtype in (torch.bfloat16, torch.float16):
+        if dtype == torch.float16 and ref.abs().max() > 6e4:
+            continue
+        out = _run_mxfp8(a8, b8, sa8, sb8, 0.75, dtype, dev)
+        assert out.shape == (m, n)
+        assert ((out.float().cpu() - ref).abs() / scale).max().item() <= GEMM_MAX_REL, (shape, dtype, plans[-1])
+        assert torch.equal(out, _run_mxfp8(a8, b8, sa8, sb8, 0.75, dtype, dev))
+    assert any("; " in p for p in plans), plans
+
+
 @pytest.mark.parametrize("shape", [(128, 1024, 8224), (100, 256, 8224), (200, 512, 10272), (65, 160, 9248), (300, 2048, 14368),
                                    (80, 6144, 8192), (70, 8192, 7168), (72, 4736, 10752), (65, 4096, 14336)])
 def test_nvfp4_gemm_split_k_with_workspace(dev, shape):
@@ -461,14 +496,16 @@ def test_mxfp8_gemm_ragged_shapes_alpha_and_scale_spread(dev, shape):
 
 @pytest.mark.parametrize("shape", [(4096, 3072, 512), (3328, 3840, 384), (2048, 6144, 256), (8192, 1536, 1152),
                                    (4096, 8192, 256), (8192, 4096, 384), (4608, 5120, 128 * 5),
-                                   (4096, 2048, 512), (4352, 4096, 384), (1920, 4096, 256), (1024, 2048, 384)])
+                                   (4096, 2048, 512), (4352, 4096, 384), (1920, 4096, 256), (1024, 2048, 384),
+                                   (4096, 1536, 256), (2048, 3840, 256), (4096, 1280, 256)])
 def test_nvfp4_gemm_persistent_256_tile_kernel_full_compare(dev, shape):
     """Dense shapes with M % 128 == N % 256 == K % 128 == 0 take the persistent kernel that converts the
     operands to fp16 between its MFMAs, with 256x256 tiles (192, 195, 192, 192, 512, 512 and 360 tiles on 256
     compute units: blocked and unblocked tile grids, one and several tiles per workgroup with two, three, five
     and nine 128-deep spans per tile) or with 128x256 tiles where those fill the compute units better
     ((4096, 2048): 256 tiles; (4352, 4096): 544, i.e. two and three per workgroup; (1920, 4096): 240, M no
-    multiple of 256); (1024, 2048) with 64 such tiles falls to the 128x128 tile kernel.  Every output element
+    multiple of 256); (1024, 2048) with 64 such tiles falls to the 128x128 tile kernel; the last three: 6, 15 and 5
+    n-tiles, i.e. blocks of 8 (m) x 2, 3 and 1 (n) after the 8 x 4 blocks of the tile walk.  Every output element
     is compared with the oracle."""
     m, n, k = shape
     gen = torch.Generator().manual_seed(k + 1)
@@ -589,7 +626,8 @@ def test_mxfp8_gemm_many_rows_small_n_deep_k(dev, shape):
 
 @pytest.mark.parametrize("shape", [(4096, 2048, 512), (2560, 3328, 384), (2048, 4096, 256), (8192, 1024, 1152),
                                    (4096, 8192, 256), (8192, 4096, 384), (4352, 4096, 640), (1152, 2048, 384),
-                                   (256, 13312, 256), (128, 28672, 384), (256, 10240, 512)])
+                                   (256, 13312, 256), (128, 28672, 384), (256, 10240, 512),
+                                   (4096, 1536, 256), (2048, 3840, 256), (4096, 1280, 256)])
 def test_mxfp8_gemm_persistent_256_tile_kernel_full_compare(dev, shape):
     """Shapes with N % 256 == K % 128 == 0 and M % 128 == 0 take the persistent LDS-direct kernel with
     256x256 tiles ((2560, 3328): a tile grid that is not a multiple of the 8 x 4 blocking; the two 512-tile
