@@ -205,6 +205,26 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
     lp.sb = wrap ? np.sb : lp.sb;
   };
 
+  // ---- the thread's LDS byte addresses: per operand, one for each half scale block it stages and one for each of the
+  // four 16-deep sub-steps it reads fragments of (the swizzle makes those differ by an exclusive or, not by a sum).
+  // They pass through empty asm statements, so that the compiler keeps exactly these twelve registers and reaches
+  // buffer, row tile and second staging row through the instructions' immediate offsets.
+  uint8_t* const lds_b = reinterpret_cast<uint8_t*>(lds);
+  uint32_t stage_at[2][2], frag_at[2][4];
+#pragma unroll
+  for (int op = 0; op < 2; ++op) {
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc) {
+      stage_at[op][cc] = (uint32_t)(tile_units(0, op) + lds_pos2(srow, spiece * 2 + cc)) * 16u;
+      asm volatile("" : "+v"(stage_at[op][cc]));
+    }
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      frag_at[op][kk] = (uint32_t)(tile_units(0, op) + lds_pos2((op ? wn * 64 : wm * (32 * TM)) + li, kk * 2 + lg)) * 16u;
+      asm volatile("" : "+v"(frag_at[op][kk]));
+    }
+  }
+
   // ---- conversion for a step of parity P: unit u (0..7) = operand u>>2, row (u>>1)&1, half block u&1 (with 128
   // rows of A, its second row does not exist: conversion unit v of the NCU real ones is unit v + 2 from v = 2 on).
   // A unit is cut into three parts of about 3 VALU instructions each.
@@ -230,7 +250,7 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
     } else {
       ch[2] = ch[2] * sv[op][i];
       ch[3] = ch[3] * sv[op][i];
-      lds[tile_units(wbuf, op) + lds_pos2(srow + 128 * i, spiece * 2 + cc)] =
+      *reinterpret_cast<u32x4*>(lds_b + stage_at[op][cc] + (wbuf * (op ? TILE_UNITS : A_UNITS) + i * 1024) * 16) =
           u32x4{__builtin_bit_cast(uint32_t, ch[0]), __builtin_bit_cast(uint32_t, ch[1]), __builtin_bit_cast(uint32_t, ch[2]),
                 __builtin_bit_cast(uint32_t, ch[3])};
     }
@@ -242,8 +262,7 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   auto load_frag_unit = [&](int buf, int kk, int q, Frag& f) {
     const int op = (q == 1 || q == 2) ? 1 : 0;
     const int t = op ? q - 1 : (q == 0 ? 0 : q - 2);
-    const int row = (op ? wn * 64 : wm * (32 * TM)) + t * 32 + li;
-    const u32x4 v = lds[tile_units(buf, op) + lds_pos2(row, kk * 2 + lg)];
+    const u32x4 v = *reinterpret_cast<const u32x4*>(lds_b + frag_at[op][kk] + (buf * (op ? TILE_UNITS : A_UNITS) + t * 256) * 16);
     if (op) f.b[t] = v; else f.a[t] = v;
   };
 
