@@ -111,13 +111,14 @@ __global__ __launch_bounds__(512) void nvfp4_group_panel_kernel(const Params p) 
   auto load_b = [&](uint32_t c) {  // chunk c lives in slot c % BSLOTS
     const uint32_t bslot = bslot0 + (c % BSLOTS) * BSLOT;
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt) lds_dma16(bslot + rt * 1024, b_base, b_off[rt] + c * 64u);
+    for (int rt = 0; rt < RT; ++rt) lds_dma16(bslot + rt * 1024, b_base + c * 64u, b_off[rt]);
 #pragma unroll
-    for (int j = 0; j < B_SC; ++j) lds_dma16(bslot + (RT + j) * 1024, bsf_base, bsf_off[j] + c * 1024u);
+    for (int j = 0; j < B_SC; ++j) lds_dma16(bslot + (RT + j) * 1024, bsf_base + c * 1024u, bsf_off[j]);
   };
+  // (the chunk moves the wave-uniform base address, not the lanes' offsets: scalar additions)
   auto load_a = [&](uint32_t c) {
-    lds_dma16(aslot, a_base, a_off + c * 64u);
-    lds_dma16(aslot + 1024, asf_base, asf_off + c * 1024u);
+    lds_dma16(aslot, a_base + c * 64u, a_off);
+    lds_dma16(aslot + 1024, asf_base + c * 1024u, asf_off);
   };
   // s_waitcnt vmcnt(n) for a wave-uniform n (the operand is an immediate)
   auto wait_loads = [&](int n) {
@@ -179,8 +180,17 @@ __global__ __launch_bounds__(512) void nvfp4_group_panel_kernel(const Params p) 
     // ---- before the loop: chunk 0's activation tile is converted, its weights are read out and their first
     // operands converted; then in flight, in this order (BSLOTS = 2: weight part 1 first): activation tile 1,
     // weight part 1 (BSLOTS = 2: weight part 2)
-    u32x4 q[RT];            // packed weights of the current chunk
-    f16x2 sv[RT][2];        // their scales
+    // packed weights of a chunk and their scales: two sets that take turns as "current" and "next", so that no
+    // register moves from one to the other at the end of a chunk
+    struct Weights { u32x4 q[RT]; f16x2 sv[RT][2]; };
+    Weights w0, w1;
+    u32x4 (&q)[RT] = w0.q;
+    f16x2 (&sv)[RT][2] = w0.sv;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      w1.q[rt] = u32x4{0, 0, 0, 0};
+      w1.sv[rt][0] = w1.sv[rt][1] = f16x2{0, 0};
+    }
     u32x4 fb[RT];           // weight operands of the current MFMA step
     load_b(0);
     load_a(0);
@@ -206,7 +216,18 @@ __global__ __launch_bounds__(512) void nvfp4_group_panel_kernel(const Params p) 
       }
     }
 
-    for (int c = 0; c < chunks; ++c) {
+    // raw activation tile and weight scales of the next chunk: read out only while there is a next chunk, and what
+    // the last chunk converts from the stale values goes to a buffer nobody reads
+    u32x4 aq = {0, 0, 0, 0};
+    uint32_t as = 0;
+    uint32_t scn[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) scn[rt] = 0;
+    auto chunk = [&](int c, Weights& cur, Weights& nxt) {
+      u32x4 (&q)[RT] = cur.q;
+      f16x2 (&sv)[RT][2] = cur.sv;
+      u32x4 (&qn)[RT] = nxt.q;
+      f16x2 (&svn)[RT][2] = nxt.sv;
       const int buf = c & 1;
       const bool has1 = c + 1 < chunks, has2 = c + 2 < chunks;
       const bool has_b_next = c + BSLOTS < chunks;          // weight part issued during the previous chunk
@@ -228,22 +249,13 @@ __global__ __launch_bounds__(512) void nvfp4_group_panel_kernel(const Params p) 
       for (int gi = 0; gi < kAhead; ++gi) fetch(gi);
       // this wavefront's raw activation tile of chunk c+1: behind it in flight only the weight part issued during
       // the previous chunk
-      u32x4 aq = {0, 0, 0, 0};
-      uint32_t as = 0;
       f16x2 asv[2];
       if (has1) {
         wait_loads(has_b_next ? LB : 0);
         aq = *reinterpret_cast<const u32x4*>(asp + rd_payload);
         as = *reinterpret_cast<const uint32_t*>(asp + rd_asc) >> sc_shift;
       }
-      u32x4 fbn[RT], qn[RT];
-      uint32_t scn[RT];
-      f16x2 svn[RT][2];
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        qn[rt] = q[rt];
-        scn[rt] = 0;
-      }
+      u32x4 fbn[RT];
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
         // The work between the groups of MFMA step t, one part per group (what is left over after the last group):
@@ -303,13 +315,13 @@ __global__ __launch_bounds__(512) void nvfp4_group_panel_kernel(const Params p) 
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) fb[rt] = fbn[rt];
       }
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        q[rt] = qn[rt];
-        sv[rt][0] = svn[rt][0];
-        sv[rt][1] = svn[rt][1];
-      }
+    };
+    int c = 0;
+    for (; c + 1 < chunks; c += 2) {
+      chunk(c, w0, w1);
+      chunk(c + 1, w1, w0);
     }
+    if (c < chunks) chunk(c, w0, w1);
 
     // every wavefront holds finished sums: element e of lane l = weight row 4*(l/16) + e, activation row l%16
 #pragma unroll
