@@ -235,7 +235,11 @@ __device__ __forceinline__ void lds_dma16(uint32_t lds_byte_addr, const uint8_t*
 // TM = 32-row accumulator tiles of a wavefront along M: 4 -> 256x256 workgroup tile, 2 -> 128x256 (for shapes
 // whose 256x256 tiles would leave compute units idle).  The statement order for TM = 4 is the one the 8192^3
 // measurements were made with.
-template <int TM, bool OUT_BF16, bool STREAM_OUT>
+// RAGGED_K: K is a multiple of 32 but not of 128.  The last K step of a tile then holds K % 128 elements per row: the
+// lanes whose 16 bytes lie past the end of the row write zeros to their LDS unit instead of loading (the bytes there
+// belong to the next row), and the scale bytes of the blocks past K - padding columns of the scale layout, whose content
+// is not defined - are replaced by 2^0, so that the step adds exact zeros.
+template <int TM, bool OUT_BF16, bool STREAM_OUT, bool RAGGED_K = false>
 __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) {
   constexpr int BM = 64 * TM, BN = 256;
   constexpr int A_UNITS = BM * 8;             // 16-byte units of the A tile (BM rows x 8 chunks)
@@ -285,8 +289,9 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
   const int first_tile = xcd * chunk_tiles + slot;
   if (first_tile >= range_end) return;
 
-  const int nk = p.k >> 7;
-  const int sf_tiles_k = (p.k >> 5) >> 2;  // 512-byte scale tiles per 128-row tile (K % 128 == 0)
+  const int nk = (p.k + 127) >> 7;
+  const int sf_tiles_k = ((p.k >> 5) + 3) >> 2;  // 512-byte scale tiles per 128-row tile
+  const int k_tail = p.k & 127;                  // elements of the last step (RAGGED_K: 32, 64 or 96)
 
   // ---- LDS-direct load addressing.  Wave w issues 8 loads per operand per K step; load j covers LDS
   // units [(w*8+j)*64, +64) = rows (w*8+j)*8 .. +7; lane L lands at unit +L, i.e. row +(L>>3), chunk
@@ -296,6 +301,9 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
   const uint32_t voff_odd = row_off + (uint32_t)(((lane & 7) ^ ((lane >> 4) | 4)) << 4);
   const uint32_t lds_base = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)lds);
   const uint32_t step8 = 8u * (uint32_t)p.k;  // 8 rows
+  // RAGGED_K: does this lane's chunk of an even / odd load unit exist in the last step?
+  const bool tail_even = (((lane & 7) ^ (lane >> 4)) << 4) < k_tail;
+  const bool tail_odd = (((lane & 7) ^ ((lane >> 4) | 4)) << 4) < k_tail;
 
   // ---- load stream state: the (tile, K step) the next loads are issued for
   // ---- load stream: the loads of step g+2 are issued while step g is computed, so the stream runs
@@ -329,6 +337,11 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
     const int j = q < 4 * TM ? (q >> 1) : q - 2 * TM;
     const uint32_t l = lds_base + (uint32_t)(buf * BUF_UNITS + (op ? A_UNITS + wave * 512 : wave * (BM * 2))) * 16u + j * 1024u;
     const uint8_t* gp = (op ? lp.b : lp.a) + ((int64_t)l_ks << 7);
+    if (RAGGED_K && l_ks == nk - 1) {
+      if ((j & 1) ? tail_odd : tail_even) lds_dma16(l, gp, ((j & 1) ? voff_odd : voff_even) + (uint32_t)j * step8);
+      else *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(lds) + (l - lds_base) + lane * 16) = u32x4{0, 0, 0, 0};
+      return;
+    }
     lds_dma16(l, gp, ((j & 1) ? voff_odd : voff_even) + (uint32_t)j * step8);
   };
   // After the 16 units: the step's scale loads, then advance the stream (selects only).
@@ -399,7 +412,16 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   // scale word of accumulator row tile i: rows {li + 32 c} of a 128-row scale tile are component c of the load;
   // with 64 rows per wavefront (TM == 2) the wavefront's half of the tile is components 2 wm, 2 wm + 1
-  auto take_scales = [&]() {
+  // (tail: the scales are those of a tile's last step, RAGGED_K only)
+  auto take_scales = [&](bool tail = false) {
+    if (RAGGED_K && tail) {
+      const uint32_t keep = (1u << (k_tail >> 2)) - 1u, fill = 0x7f7f7f7fu & ~keep;  // k_tail / 32 bytes stay
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        na[c] = (na[c] & keep) | fill;
+        nb[c] = (nb[c] & keep) | fill;
+      }
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i) wa[i] = (TM == 4 ? na[i] : (wm ? na[2 + (i & 1)] : na[i & 1])) >> sh;
 #pragma unroll
@@ -454,7 +476,7 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
         __builtin_amdgcn_sched_barrier(0);
       }
       NVF_PIN_ACC();
-      take_scales();
+      take_scales(c_ks + 2 == nk);  // the scales of the next step
     }
     // ---- epilogue of this tile; the loads of the next tile's first two steps are already in flight.
     // acc[i][j][r] = C[m = li][n = (r/4)*8 + lg*4 + r%4] of its 32x32 sub-tile.
@@ -507,14 +529,14 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
 #undef NVF_PIN_ACC
 }
 
-template <int TM, bool OUT_BF16, bool STREAM_OUT>
+template <int TM, bool OUT_BF16, bool STREAM_OUT, bool RAGGED_K>
 int launch_fast_cfg(const Params& p, hipStream_t stream) {
-  auto kern = mxfp8_gemm_256_kernel<TM, OUT_BF16, STREAM_OUT>;
+  auto kern = mxfp8_gemm_256_kernel<TM, OUT_BF16, STREAM_OUT, RAGGED_K>;
   constexpr int lds_bytes = 2 * (64 * TM + 256) * 128 + 4 * 4608;  // 128 KiB / 96 KiB of tiles + the epilogue's 18 KiB
   const int64_t tiles = (int64_t)(p.m / (64 * TM)) * (p.n / 256);
   const int cus = cu_count() & ~7;  // workgroup ids are dealt round-robin to the 8 XCDs
   const unsigned grid = (unsigned)(tiles >= cus ? cus : ((tiles + 7) / 8) * 8);
-  if (note_launch("mxfp8_gemm_256_kernel<TM=%d,stream_out=%d> grid=%u", TM, (int)STREAM_OUT, grid)) return NVF_OK;
+  if (note_launch("mxfp8_gemm_256_kernel<TM=%d,stream_out=%d%s> grid=%u", TM, (int)STREAM_OUT, RAGGED_K ? ",ragged_k" : "", grid)) return NVF_OK;
   static std::atomic<uint64_t> configured{0};  // one bit per device
   if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_bytes, stream, p);
@@ -527,7 +549,8 @@ int launch_fast(const Params& p, hipStream_t stream) {
   // operand panels out of it (and out of the L2s) on its way to memory, so it leaves with non-temporal stores
   // (8192^3: +5 %, 16384 x 16384 x 2048: +17 %; smaller problems lose 1-5 % that way).
   const bool stream_out = ((int64_t)p.m + p.n) * p.k + 2 * (int64_t)p.m * p.n > (int64_t)224 << 20;
-  return stream_out ? launch_fast_cfg<TM, OUT_BF16, true>(p, stream) : launch_fast_cfg<TM, OUT_BF16, false>(p, stream);
+  if ((p.k & 127) != 0) return stream_out ? launch_fast_cfg<TM, OUT_BF16, true, true>(p, stream) : launch_fast_cfg<TM, OUT_BF16, false, true>(p, stream);
+  return stream_out ? launch_fast_cfg<TM, OUT_BF16, true, false>(p, stream) : launch_fast_cfg<TM, OUT_BF16, false, false>(p, stream);
 }
 
 // -------------------------------------------------------------------------------------------------
@@ -802,12 +825,13 @@ enum class Plan { kStream, kTiles256, kTiles128, kOther };
 Plan mxfp8_plan(int64_t m, int64_t n, int64_t k, int64_t cus, int64_t* ns = nullptr) {
   if (ns) *ns = INT64_MAX;
   const bool skinny_ok = (k & 127) == 0 && (n & 15) == 0 && k * 64 < (1ll << 31);  // 32-bit lane offsets
-  const bool fast_ok = (k & 127) == 0 && k >= 256 && (m & 127) == 0 && (n & 255) == 0 && k * 256 < (1ll << 31);
+  // (the persistent kernel takes any K % 32 == 0: its last step may be short)
+  const bool fast_ok = (k & 31) == 0 && k >= 256 && (m & 127) == 0 && (n & 255) == 0 && k * 256 < (1ll << 31);
   const int64_t t256 = fast_ok && (m & 255) == 0 ? (m / 256) * (n / 256) : 0, t128 = fast_ok ? (m / 128) * (n / 256) : 0;
   const int64_t cost256 = t256 >= 128 ? 100 * ceil_div(t256, cus) : INT64_MAX;
   const int64_t cost128 = t128 >= 48 ? 61 * ceil_div(t128, cus) : INT64_MAX;
   const bool fast = cost256 != INT64_MAX || cost128 != INT64_MAX;
-  const int64_t fast_ns = fast ? 5000 + std::min(cost256, cost128) * 113 * k / 1024 : INT64_MAX;
+  const int64_t fast_ns = fast ? 5000 + std::min(cost256, cost128) * 113 * ((k + 127) & ~127ll) / 1024 : INT64_MAX;
   if (skinny_ok) {
     const int64_t skinny_ns = mxfp8_skinny_best(m, n, k, cus, nullptr, nullptr) * 963 / 1000;
     if (ns) *ns = skinny_ns;
@@ -845,7 +869,7 @@ int launch_sized(const Params& p, hipStream_t stream) {
   // N not a multiple of 256 (29568, 1408) with enough rows for the persistent kernel: the columns up to the last
   // multiple of 256 go to whatever kernel that shape gets, the remaining columns (weight rows) to a launch of their
   // own that writes into the same rows of the result (8192 x 29568 x 8192: 4.1 -> 1.3 ms).
-  if ((p.n & 255) != 0 && p.n > 256 && (p.n & 15) == 0 && p.m >= 512 && (p.k & 127) == 0 && p.k >= 256 &&
+  if ((p.n & 255) != 0 && p.n > 256 && (p.n & 15) == 0 && p.m >= 512 && (p.k & 31) == 0 && p.k >= 256 &&
       mxfp8_plan(p.m & ~127, p.n & ~255, p.k, cus) != Plan::kOther) {
     if (mxfp8_plan(p.m & ~127, p.n & ~255, p.k, cus) == Plan::kStream) return launch_skinny<OUT_BF16>(p, stream);  // (takes any N % 16 == 0)
     Params main = p, rest = p;
