@@ -555,7 +555,7 @@ int launch_fast(const Params& p, hipStream_t stream) {
 
 // -------------------------------------------------------------------------------------------------
 // Skinny path: slabs of up to 128 activation rows (decode-sized activations; more rows as several slabs, the
-// whole ones side by side in one launch, blockIdx.y = slab), K % 128 == 0, N % (16*RT) == 0.  A slab streams
+// whole ones side by side in one launch, blockIdx.y = slab), K % 32 == 0, N % (16*RT) == 0.  A slab streams
 // the weight matrix exactly once, so the op is bound by HBM (by the last-level cache for the slabs after the
 // first):
 //   * A workgroup owns 16*RT weight rows for the whole of K and all M activation rows; its 8 wavefronts
@@ -595,8 +595,13 @@ __global__ __launch_bounds__(512) void mxfp8_skinny_kernel(const Params p) {
   const int m_base = p.m_base + (int)blockIdx.y * (16 * TT);
   const int m_loc = min(p.m - m_base, 16 * TT);
   const int tt_count = (m_loc + 15) >> 4;
-  const int chunks = p.k >> 7;
-  const int sf_padded = p.k >> 5;  // K % 128 == 0: no padding columns
+  // K % 128 = 32, 64 or 96: the last chunk is short.  Lanes whose 16 bytes lie past the end of the row write zeros to
+  // their LDS unit instead of loading, and the scale bytes of the blocks past K (padding columns of the scale layout,
+  // content not defined) are replaced by 2^0, so that the chunk adds exact zeros for them.
+  const int chunks = (p.k + 127) >> 7;
+  const int k_tail = p.k & 127;
+  const int tail_chunk = k_tail ? chunks - 1 : -1;
+  const int sf_padded = ((p.k >> 5) + 3) & ~3;  // scale columns with the layout's padding
 
   // ---- load side (memory order).  Payload: tile t, load j (rows 8j..8j+7): lane L = row 8j + L/8, piece
   // (L & 7) ^ ((4j + L/16) & 7).  Scales: lane L = tile L/16, row L%16: the 16 bytes that hold the scale
@@ -604,10 +609,12 @@ __global__ __launch_bounds__(512) void mxfp8_skinny_kernel(const Params p) {
   const uint8_t* b_base = p.b + (int64_t)n0 * p.k;
   const uint8_t* bsf_base = p.sfb + (int64_t)(n0 >> 7) * ((int64_t)sf_padded << 7);
   uint32_t b_off[RT][2], a_off[TT][2];
+  bool in_tail[2];  // does the lane's piece of load j exist in a short last chunk?
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     const int row = 8 * j + (lane >> 3);
     const uint32_t piece = (uint32_t)((lane & 7) ^ ((4 * j + (lane >> 4)) & 7)) * 16u;
+    in_tail[j] = (int)piece < k_tail;
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) b_off[rt][j] = (uint32_t)(rt * 16 + row) * (uint32_t)p.k + piece;
 #pragma unroll
@@ -624,14 +631,25 @@ __global__ __launch_bounds__(512) void mxfp8_skinny_kernel(const Params p) {
     if (c_in >= chunks) return;
     const uint32_t c = (uint32_t)c_in;
     const uint32_t sb = ring_base + (uint32_t)slot * SLOT_BYTES;
+    if (c_in == tail_chunk) {
+      char* const zp = reinterpret_cast<char*>(lds) + (sb - lds_base) + lane * 16;
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
+      for (int t = 0; t < NT; ++t)
 #pragma unroll
-      for (int j = 0; j < 2; ++j) lds_dma16(sb + rt * 2048 + j * 1024, b_base, b_off[rt][j] + c * 128u);
+        for (int j = 0; j < 2; ++j) {
+          if (in_tail[j]) lds_dma16(sb + t * 2048 + j * 1024, t < RT ? b_base : a_base, (t < RT ? b_off[t][j] : a_off[t - RT][j]) + c * 128u);
+          else *reinterpret_cast<u32x4*>(zp + t * 2048 + j * 1024) = u32x4{0, 0, 0, 0};
+        }
+    } else {
 #pragma unroll
-    for (int tt = 0; tt < TT; ++tt)
+      for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-      for (int j = 0; j < 2; ++j) lds_dma16(sb + (RT + tt) * 2048 + j * 1024, a_base, a_off[tt][j] + c * 128u);
+        for (int j = 0; j < 2; ++j) lds_dma16(sb + rt * 2048 + j * 1024, b_base, b_off[rt][j] + c * 128u);
+#pragma unroll
+      for (int tt = 0; tt < TT; ++tt)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) lds_dma16(sb + (RT + tt) * 2048 + j * 1024, a_base, a_off[tt][j] + c * 128u);
+    }
     // one load each for the scales of all weight tiles / all activation tiles (lanes of tiles that do not
     // exist stay off: a disabled lane writes nothing)
     if (lane < 16 * RT) lds_dma16(sb + NT * 2048, bsf_base, bsf_off + c * 512u);
@@ -679,6 +697,10 @@ __global__ __launch_bounds__(512) void mxfp8_skinny_kernel(const Params p) {
     for (int rt = 0; rt < RT; ++rt) sc[rt] = *reinterpret_cast<const uint32_t*>(sp + rd_bsc[rt]) >> sc_shift;
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) sc[RT + tt] = *reinterpret_cast<const uint32_t*>(sp + rd_asc[tt]) >> sc_shift;
+    if (c == tail_chunk && g * 32 >= k_tail) {  // this lane's K-block lies past K
+#pragma unroll
+      for (int t = 0; t < NT; ++t) sc[t] = 0x7f;
+    }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // read out: the slot may be refilled
     issue_chunk(c + DEPTH * W, slot);
     slot = (slot + 1 == DEPTH) ? 0 : slot + 1;
@@ -763,7 +785,7 @@ int64_t mxfp8_skinny_cost(int64_t m, int64_t n, int64_t k, int slab, int rt, int
   const int tt = m <= slab ? (m <= 16 ? 1 : m <= 32 ? 2 : m <= 64 ? 4 : 8) : slab / 16;
   if (tt == 8 && rt != 1) return INT64_MAX;
   const int64_t wgs = slabs * (n / (16 * rt));
-  const int64_t chunks = ceil_div(k >> 7, 8);
+  const int64_t chunks = ceil_div((k + 127) >> 7, 8);
   const int64_t per_chunk = (rt + tt) * 145 + rt * tt * 10 + 100;
   const int64_t wg_time = chunks * per_chunk + rt * tt * 193 + 2493;
   const int64_t full = wgs / cus, rest = wgs - full * cus;
@@ -824,7 +846,7 @@ enum class Plan { kStream, kTiles256, kTiles128, kOther };
 // (ns: the estimated duration, where there is an estimate)
 Plan mxfp8_plan(int64_t m, int64_t n, int64_t k, int64_t cus, int64_t* ns = nullptr) {
   if (ns) *ns = INT64_MAX;
-  const bool skinny_ok = (k & 127) == 0 && (n & 15) == 0 && k * 64 < (1ll << 31);  // 32-bit lane offsets
+  const bool skinny_ok = (k & 31) == 0 && (n & 15) == 0 && k * 64 < (1ll << 31);  // 32-bit lane offsets (a short last chunk is fine)
   // (the persistent kernel takes any K % 32 == 0: its last step may be short)
   const bool fast_ok = (k & 31) == 0 && k >= 256 && (m & 127) == 0 && (n & 255) == 0 && k * 256 < (1ll << 31);
   const int64_t t256 = fast_ok && (m & 255) == 0 ? (m / 256) * (n / 256) : 0, t128 = fast_ok ? (m / 128) * (n / 256) : 0;

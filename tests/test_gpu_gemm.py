@@ -391,6 +391,33 @@ def test_mxfp8_gemm_k_not_a_multiple_of_128_on_the_persistent_kernel(dev, shape)
         assert torch.equal(out, _run_mxfp8(a8, b8, sa8_p, sb8_p, 0.75, dtype, dev))
 
 
+@pytest.mark.parametrize("shape", [(16, 4096, 2880), (128, 5760, 2880), (300, 4096, 2880), (64, 512, 96), (7, 256, 32), (100, 1024, 4192),
+                                   (33, 2048, 160), (2048, 5760, 2880)])
+def test_mxfp8_gemm_k_not_a_multiple_of_128_on_the_streaming_kernel(dev, shape):
+    """The same on the weight-streaming kernel (decode sizes, ragged M, and - last shape - the columns that the persistent
+    kernel leaves over): the last 128-deep chunk of a row is short.  NaN codes in all scale padding."""
+    from fuser_amd import capi
+
+    m, n, k = shape
+    gen = torch.Generator().manual_seed(m + n + k)
+    a8, sa8 = _mxfp8_operand(m, k, gen, 1.0)
+    b8, sb8 = _mxfp8_operand(n, k, gen, 1.0)
+    ref = O.ref_mxfp8_scaled_mm(a8, b8, sa8, sb8, 0.75)
+    scale = ref.abs().amax(dim=1, keepdim=True).clamp(min=1e-30)
+    sa8_p, sb8_p = sa8.clone(), sb8.clone()
+    sa8_p[O.linear_to_swizzled_128_4(torch.ones(m, k // 32, dtype=torch.uint8)) == 0] = 0xFF
+    sb8_p[O.linear_to_swizzled_128_4(torch.ones(n, k // 32, dtype=torch.uint8)) == 0] = 0xFF
+    plan = capi.describe_dispatch("mxfp8_scaled_mm", m, n, k)
+    assert "mxfp8_skinny_kernel" in plan, plan
+    for dtype in (torch.bfloat16, torch.float16):
+        if dtype == torch.float16 and ref.abs().max() > 6e4:
+            continue
+        out = _run_mxfp8(a8, b8, sa8_p, sb8_p, 0.75, dtype, dev)
+        assert out.shape == (m, n) and torch.isfinite(out.float()).all()
+        assert ((out.float().cpu() - ref).abs() / scale).max().item() <= GEMM_MAX_REL, (shape, dtype, plan)
+        assert torch.equal(out, _run_mxfp8(a8, b8, sa8_p, sb8_p, 0.75, dtype, dev))
+
+
 @pytest.mark.parametrize("shape", [(128, 1024, 8224), (100, 256, 8224), (200, 512, 10272), (65, 160, 9248), (300, 2048, 14368),
                                    (80, 6144, 8192), (70, 8192, 7168), (72, 4736, 10752), (65, 4096, 14336)])
 def test_nvfp4_gemm_split_k_with_workspace(dev, shape):
