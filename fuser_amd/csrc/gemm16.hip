@@ -173,7 +173,7 @@ struct DensePlan {
   int64_t ns;  // estimated duration (INT64_MAX: no estimate)
 };
 DensePlan nvfp4_dense_plan(int64_t m, int64_t n, int64_t k, int cus) {
-  const bool stream_ok = (k & 127) == 0 && (n & 15) == 0 && k * 64 < (1ll << 31);  // 32-bit lane offsets
+  const bool stream_ok = (k & 31) == 0 && (n & 15) == 0 && k * 64 < (1ll << 31);  // 32-bit lane offsets (a short last chunk is fine)
   const bool persistent_ok = (m & 127) == 0 && (n & 255) == 0 && (k & 127) == 0 && k >= 256;
   int64_t cost256 = INT64_MAX, cost128 = INT64_MAX, cost_tile = INT64_MAX;
   if (persistent_ok) {

@@ -575,7 +575,7 @@ int launch_fast(const Params& p, hipStream_t stream) {
 // -------------------------------------------------------------------------------------------------
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-template <int RT, int TT, bool OUT_BF16, int DEPTH>
+template <int RT, int TT, bool OUT_BF16, int DEPTH, bool RAGGED_K = false>
 __global__ __launch_bounds__(512) void mxfp8_skinny_kernel(const Params p) {
   constexpr int W = 8;
   constexpr int NT = RT + TT;
@@ -600,7 +600,7 @@ __global__ __launch_bounds__(512) void mxfp8_skinny_kernel(const Params p) {
   // content not defined) are replaced by 2^0, so that the chunk adds exact zeros for them.
   const int chunks = (p.k + 127) >> 7;
   const int k_tail = p.k & 127;
-  const int tail_chunk = k_tail ? chunks - 1 : -1;
+  const int tail_chunk = RAGGED_K ? chunks - 1 : -1;  // (a kernel of its own: K % 128 != 0)
   const int sf_padded = ((p.k >> 5) + 3) & ~3;  // scale columns with the layout's padding
 
   // ---- load side (memory order).  Payload: tile t, load j (rows 8j..8j+7): lane L = row 8j + L/8, piece
@@ -631,7 +631,7 @@ __global__ __launch_bounds__(512) void mxfp8_skinny_kernel(const Params p) {
     if (c_in >= chunks) return;
     const uint32_t c = (uint32_t)c_in;
     const uint32_t sb = ring_base + (uint32_t)slot * SLOT_BYTES;
-    if (c_in == tail_chunk) {
+    if (RAGGED_K && c_in == tail_chunk) {
       char* const zp = reinterpret_cast<char*>(lds) + (sb - lds_base) + lane * 16;
 #pragma unroll
       for (int t = 0; t < NT; ++t)
@@ -697,7 +697,7 @@ __global__ __launch_bounds__(512) void mxfp8_skinny_kernel(const Params p) {
     for (int rt = 0; rt < RT; ++rt) sc[rt] = *reinterpret_cast<const uint32_t*>(sp + rd_bsc[rt]) >> sc_shift;
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) sc[RT + tt] = *reinterpret_cast<const uint32_t*>(sp + rd_asc[tt]) >> sc_shift;
-    if (c == tail_chunk && g * 32 >= k_tail) {  // this lane's K-block lies past K
+    if (RAGGED_K && c == tail_chunk && g * 32 >= k_tail) {  // this lane's K-block lies past K
 #pragma unroll
       for (int t = 0; t < NT; ++t) sc[t] = 0x7f;
     }
@@ -752,13 +752,13 @@ template <int RT, int TT, bool OUT_BF16>
 int launch_skinny_cfg(const Params& p, hipStream_t stream, int slabs = 1) {
   constexpr int SLOT = (RT + TT) * 2048 + RT * 256 + (TT < 2 ? TT : 2) * 256;
   constexpr int DEPTH = 8 * 3 * SLOT <= 160 * 1024 ? 3 : (8 * 2 * SLOT <= 160 * 1024 ? 2 : 1);
-  auto kern = mxfp8_skinny_kernel<RT, TT, OUT_BF16, DEPTH>;
+  auto kern = (p.k & 127) != 0 ? mxfp8_skinny_kernel<RT, TT, OUT_BF16, DEPTH, true> : mxfp8_skinny_kernel<RT, TT, OUT_BF16, DEPTH>;
   constexpr int ring = 8 * DEPTH * SLOT, red = 8 * RT * TT * 1024;
   constexpr int lds_bytes = ring > red ? ring : red;
   static_assert(lds_bytes <= 160 * 1024, "LDS");
   if (note_launch("mxfp8_skinny_kernel<RT=%d,TT=%d> grid=%ux%d m_base=%d", RT, TT, (unsigned)(p.n / (16 * RT)), slabs, p.m_base)) return NVF_OK;
-  static std::atomic<uint64_t> configured{0};  // one bit per device
-  if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
+  static std::atomic<uint64_t> configured[2] = {{0}, {0}};  // per kernel, one bit per device
+  if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured[(p.k & 127) != 0])) return rc;
   hipLaunchKernelGGL(kern, dim3((unsigned)(p.n / (16 * RT)), (unsigned)slabs), dim3(512), lds_bytes, stream, p);
   return check_launch("mxfp8_skinny_kernel");
 }

@@ -2,7 +2,7 @@
 // cost estimate that picks slab height and weight tiles per workgroup.
 // -------------------------------------------------------------------------------------------------
 // NVFP4 skinny path: dense, up to 128 activation rows per launch (decode-sized activations; up to 256 rows in
-// two launches), K % 128 == 0, N % (16*RT) == 0.  A launch streams the weight matrix exactly once, so the op
+// two launches), K % 32 == 0, N % (16*RT) == 0.  A launch streams the weight matrix exactly once, so the op
 // is bound by HBM and by the conversion work, not by the MFMAs:
 //   * A workgroup owns 16*RT weight rows for the whole of K and all M activation rows; its 8
 //     wavefronts split K in interleaved 128-element chunks and their partial sums are added in a fixed
@@ -49,7 +49,8 @@ __device__ __forceinline__ void dequant_frags(const u32x4 q, uint32_t s2, u32x4 
 // NSPLIT (grouped only, where the groups supply enough workgroups): the 8 wavefronts own 8 different blocks of
 // 16*RT weight rows and each walks all of K on its own - a long pipeline per wavefront and no reduction -
 // instead of sharing one block and splitting K.
-template <int RT, int TT, bool OUT_BF16, int DEPTH, bool GROUPED = false, bool NSPLIT = false>
+// RAGGED_K: K % 128 != 0 (a kernel of its own: the tests for the short chunk cost the others 4-8 %).
+template <int RT, int TT, bool OUT_BF16, int DEPTH, bool GROUPED = false, bool NSPLIT = false, bool RAGGED_K = false>
 __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) {
   static_assert(GROUPED || !NSPLIT, "the dense op has too few row blocks to give every wavefront its own");
   constexpr int W = 8;
@@ -66,14 +67,34 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, g = lane >> 4;
   const int kbytes = p.k >> 1;
-  int chunks = p.k >> 7;
-  const int sf_padded = p.k >> 4;  // K % 128 == 0: no padding columns
+  // K % 128 = 32, 64 or 96: the last chunk is short.  A zero scale makes an NVFP4 block count as zero whatever its
+  // payload, so it is enough that the lanes whose 32 elements lie past K (a) fetch bytes that exist - their own row's
+  // first piece and the chunk's first scale column tile instead of the next row's bytes and a column tile that the
+  // layout may not have - and (b) use zero for the scales of their two blocks, whatever the layout's padding holds.
+  int chunks = (p.k + 127) >> 7;
+  const int k_tail = p.k & 127;
+  const int sf_padded = ((p.k >> 4) + 3) & ~3;  // scale columns with the layout's padding
   // dense with a workspace: blockIdx.z owns the chunks [c_lo, c_lo + chunks) of K and leaves an fp32 partial result
   int c_lo = 0;
   if (!GROUPED && p.partial != nullptr) {
     c_lo = (int)blockIdx.z * p.spans_per_split;
     chunks = min(chunks - c_lo, p.spans_per_split);
   }
+  const int tail_chunk = ((p.k + 127) >> 7) - 1 - c_lo;  // the short chunk, counted like this workgroup's chunks
+  auto is_tail = [&](int c) { return RAGGED_K && c == tail_chunk; };
+  // (worked out where they are used, from a lane number the compiler cannot trace: no registers held for them)
+  auto tail_subs = [&](uint32_t& ld_sub, uint32_t& sc_sub) {
+    int tl = threadIdx.x & 63;
+    asm volatile("" : "+v"(tl));
+    const int piece = (tl & 3) ^ ((tl >> 4) & 3);
+    ld_sub = piece * 32 < k_tail ? 0u : (uint32_t)piece * 16u;  // back to the row's first piece
+    sc_sub = ((tl >> 4) & 1) * 64 < k_tail ? 0u : 512u;         // back to the chunk's first column tile
+  };
+  auto tail_keep = [&]() {  // read side: all ones if the lane's blocks 2g, 2g+1 of the chunk exist
+    int tl = threadIdx.x & 63;
+    asm volatile("" : "+v"(tl));
+    return (tl >> 4) * 32 < k_tail ? 0xffffffffu : 0u;
+  };
   int n0, m_loc, grp = 0, asf_word0 = 0;  // asf_word0: which 32-row group of its 128-row scale tile the slab starts in
   int64_t a_row0 = p.m_base, asf_row0 = p.m_base, b_row0 = 0;  // first activation row, its scale row, first weight row
   if constexpr (GROUPED) {
@@ -128,6 +149,21 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
     if (c_in >= chunks) return;
     const uint32_t c = (uint32_t)c_in;
     const uint32_t sb = ring_base + (uint32_t)slot * SLOT_BYTES;
+    if (is_tail(c_in)) {
+      uint32_t ld_sub, sc_sub;
+      tail_subs(ld_sub, sc_sub);
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) lds_dma16(sb + rt * 1024, b_base, b_off[rt] - ld_sub + c * 64u);
+#pragma unroll
+      for (int tt = 0; tt < TT; ++tt)
+        if (DEPTH == 2 || tt < tt_count) lds_dma16(sb + (RT + tt) * 1024, a_base, a_off[tt] - ld_sub + c * 64u);
+#pragma unroll
+      for (int j = 0; j < B_SC; ++j) lds_dma16(sb + (NT + j) * 1024, bsf_base, bsf_off[j] - sc_sub + c * 1024u);
+#pragma unroll
+      for (int j = 0; j < A_SC; ++j)
+        if (DEPTH == 2 || 2 * j < tt_count) lds_dma16(sb + (NT + B_SC + j) * 1024, asf_base, asf_off[j] - sc_sub + c * 1024u);
+      return;
+    }
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) lds_dma16(sb + rt * 1024, b_base, b_off[rt] + c * 64u);
 #pragma unroll
@@ -228,6 +264,15 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
   constexpr bool kFineRing = TT > 2 && DEPTH == 1;
   if constexpr (kFineRing) {
     auto load_b_part = [&](uint32_t c) {
+      if (is_tail((int)c)) {
+        uint32_t ld_sub, sc_sub;
+        tail_subs(ld_sub, sc_sub);
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) lds_dma16(ring_base + rt * 1024, b_base, b_off[rt] - ld_sub + c * 64u);
+#pragma unroll
+        for (int j = 0; j < B_SC; ++j) lds_dma16(ring_base + (NT + j) * 1024, bsf_base, bsf_off[j] - sc_sub + c * 1024u);
+        return;
+      }
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) lds_dma16(ring_base + rt * 1024, b_base, b_off[rt] + c * 64u);
 #pragma unroll
@@ -236,13 +281,21 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
     int fine_lrow = lrow;  // re-derived per use: eight row offsets kept in registers would not fit
     auto load_a_tile = [&](uint32_t c, int tt) {
       asm volatile("" : "+v"(fine_lrow));
-      lds_dma16(ring_base + (RT + tt) * 1024, a_base, (uint32_t)min(tt * 16 + fine_lrow, m_loc - 1) * (uint32_t)kbytes + lpiece * 16 + c * 64u);
+      uint32_t ld_sub = 0, sc_sub;
+      if (is_tail((int)c)) tail_subs(ld_sub, sc_sub);
+      lds_dma16(ring_base + (RT + tt) * 1024, a_base,
+                (uint32_t)min(tt * 16 + fine_lrow, m_loc - 1) * (uint32_t)kbytes + lpiece * 16 - ld_sub + c * 64u);
     };
-    auto load_a_scales = [&](uint32_t c, int j) { lds_dma16(ring_base + (NT + B_SC + j) * 1024, asf_base, asf_off[j] + c * 1024u); };
+    auto load_a_scales = [&](uint32_t c, int j) {
+      uint32_t ld_sub, sc_sub = 0;
+      if (is_tail((int)c)) tail_subs(ld_sub, sc_sub);
+      lds_dma16(ring_base + (NT + B_SC + j) * 1024, asf_base, asf_off[j] - sc_sub + c * 1024u);
+    };
     const char* sp = reinterpret_cast<const char*>(red) + wave * SLOT_BYTES;
-    auto read_a_tile = [&](int tt, u32x4& aq, uint32_t& as) {
+    auto read_a_tile = [&](uint32_t c, int tt, u32x4& aq, uint32_t& as) {
       aq = *reinterpret_cast<const u32x4*>(sp + (RT + tt) * 1024 + rd_payload);
       as = *reinterpret_cast<const uint32_t*>(sp + rd_asc[tt]) >> sc_shift;
+      if (is_tail((int)c)) as &= tail_keep();
     };
     // e4m3 scales of a lane's two blocks -> fp16 pairs; one dword (8 values of one block) -> one MFMA operand
     auto scale_pairs = [&](uint32_t s2, f16x2 sv[2]) {
@@ -272,7 +325,12 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) sc[rt] = *reinterpret_cast<const uint32_t*>(sp + rd_bsc[rt]) >> sc_shift;
 #pragma unroll
-      for (int tt = 0; tt < TTC; ++tt) read_a_tile(tt, aq[tt], as[tt]);
+      for (int tt = 0; tt < TTC; ++tt) read_a_tile(c, tt, aq[tt], as[tt]);
+      if (is_tail((int)c)) {
+        const uint32_t keep = tail_keep();
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) sc[rt] &= keep;
+      }
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // read out: may be refilled
       if (c + CSTEP < (uint32_t)chunks) {
         load_b_part(c + CSTEP);
@@ -330,6 +388,11 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
       for (int rt = 0; rt < RT; ++rt) q[rt] = *reinterpret_cast<const u32x4*>(sp + rt * 1024 + rd_payload);
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) sc[rt] = *reinterpret_cast<const uint32_t*>(sp + rd_bsc[rt]) >> sc_shift;
+      if (is_tail((int)c)) {
+        const uint32_t keep = tail_keep();
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) sc[rt] &= keep;
+      }
       u32x4 fb[RT][4];
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) dequant_frags(q[rt], sc[rt], fb[rt]);
@@ -338,7 +401,7 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
         __builtin_amdgcn_sched_barrier(0);
         u32x4 aq;
         uint32_t as;
-        read_a_tile(tt, aq, as);
+        read_a_tile(c, tt, aq, as);
         if (tt + 1 == TTC) {
           asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the last read of the slot is complete
           if (c + CSTEP < (uint32_t)chunks) {
@@ -408,10 +471,15 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
       for (int rt = 0; rt < RT; ++rt) q[rt] = *reinterpret_cast<const u32x4*>(sp + rt * 1024 + rd_payload);
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) sc[rt] = *reinterpret_cast<const uint32_t*>(sp + rd_bsc[rt]) >> sc_shift;
+      if (is_tail((int)c)) {
+        const uint32_t keep = tail_keep();
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) sc[rt] &= keep;
+      }
       wait_loads(after_tile(0));
       u32x4 aq, aqn = {0, 0, 0, 0};
       uint32_t as, asn = 0;
-      read_a_tile(0, aq, as);
+      read_a_tile(c, 0, aq, as);
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // read out: may be refilled
       if (has_next) {
         load_b_part(c + CSTEP);
@@ -437,7 +505,7 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
         if (tt + 1 < TTC) {
           // pending behind tile tt+1: the rest of this chunk's tiles, the next chunk's weight part and its tiles 0..tt
           wait_loads(after_tile(tt + 1) + (has_next ? LB + (tt + 1) + ((tt + 1) >> 1) : 0));
-          read_a_tile(tt + 1, aqn, asn);
+          read_a_tile(c, tt + 1, aqn, asn);
         }
         // K steps 0 and 1 of tile tt; behind every MFMA one dword of the operands of its steps 2 and 3
 #pragma unroll
@@ -536,6 +604,13 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
       if constexpr (!kLazyA) {
 #pragma unroll
         for (int tt = 0; tt < TT; ++tt) sc[RT + tt] = *reinterpret_cast<const uint32_t*>(sp + rd_asc[tt]) >> sc_shift;
+      }
+      if (is_tail(c)) {
+        const uint32_t keep = tail_keep();
+#pragma unroll
+        for (int t = 0; t < NQ; ++t) sc[t] &= keep;
+      }
+      if constexpr (!kLazyA) {
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // read out: the slot may be refilled
         issue_chunk(c + DEPTH * CSTEP, slot);
       }
@@ -550,6 +625,7 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
           if constexpr (kLazyA) {
             aq = *reinterpret_cast<const u32x4*>(sp + (RT + tt) * 1024 + rd_payload);
             as = *reinterpret_cast<const uint32_t*>(sp + rd_asc[tt]) >> sc_shift;
+            if (is_tail(c)) as &= tail_keep();
             if (tt + 1 == tt_count) {
               asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the last read of the slot is complete
               issue_chunk(c + DEPTH * CSTEP, slot);
@@ -579,7 +655,7 @@ int launch_nvfp4_skinny_ring_cfg(const Params& p, hipStream_t stream, int slabs 
   constexpr int SLOT_KIB = RT + TT + (RT + 1) / 2 + (TT + 1) / 2;
   // one slot per wavefront also where two would fit (M=16, N=14336, K=4096: 8.0 -> 7.5 us; K=14336: 9.6 -> 9.2 us)
   constexpr int DEPTH = 1;
-  auto kern = nvfp4_skinny_ring_kernel<RT, TT, OUT_BF16, DEPTH>;
+  auto kern = (p.k & 127) != 0 ? nvfp4_skinny_ring_kernel<RT, TT, OUT_BF16, DEPTH, false, false, true> : nvfp4_skinny_ring_kernel<RT, TT, OUT_BF16, DEPTH>;
   // the ring; the reduction reuses it and needs 8 KiB per partial tile of a round
   constexpr int red_kib = 8 * (RT * TT <= 8 ? RT * TT : TT);
   constexpr int ring_kib = 8 * DEPTH * SLOT_KIB;
@@ -590,8 +666,8 @@ int launch_nvfp4_skinny_ring_cfg(const Params& p, hipStream_t stream, int slabs 
                                (unsigned)(p.n / (16 * RT)), slabs, splits)
                  : note_launch("nvfp4_skinny_ring_kernel<RT=%d,TT=%d> grid=%ux%d", RT, TT, (unsigned)(p.n / (16 * RT)), slabs))
     return NVF_OK;
-  static std::atomic<uint64_t> configured{0};  // one bit per device
-  if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
+  static std::atomic<uint64_t> configured[2] = {{0}, {0}};  // per kernel, one bit per device
+  if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured[(p.k & 127) != 0])) return rc;
   hipLaunchKernelGGL(kern, dim3((unsigned)(p.n / (16 * RT)), (unsigned)slabs, (unsigned)splits), dim3(512), lds_bytes, stream, p);
   if (const int rc = check_launch("nvfp4_skinny_ring_kernel")) return rc;
   if (p.partial == nullptr) return NVF_OK;
@@ -651,7 +727,7 @@ int64_t nvfp4_skinny_cost(int64_t m, int64_t n, int64_t k, int slab, int rt, int
   if (rt * tt > 16) per_cu = 1;                 // (their accumulators take the registers)
   else if (rt * tt > 6) per_cu = std::min<int64_t>(per_cu, 2);
   if (per_cu < 1) per_cu = 1;
-  const int64_t chunks = ceil_div(k >> 7, 8);
+  const int64_t chunks = ceil_div((k + 127) >> 7, 8);
   const int64_t resident = std::min(per_cu, ceil_div(wgs, cus));
   const int64_t rounds = ceil_div(wgs, cus * per_cu);
   const int64_t per_chunk = (rt + tt) * 183 + rt * tt * 18 + 100;

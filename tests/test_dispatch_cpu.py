@@ -50,12 +50,14 @@ def test_deep_k_with_a_workspace_splits_k_only_where_it_wins():
     got = plan("nvfp4_scaled_mm", 96, 4096, 14336, ws=need - 1)
     assert got.startswith("nvfp4_skinny_ring_kernel<") and "split_k" not in got, got
     assert lib.nvf_nvfp4_scaled_mm_workspace_bytes(96, 4096, 4096) == 0
-    # few tiles and a deep K: the streaming kernel where it runs (K % 128 == 0), else the tile kernel's split
-    assert lib.nvf_nvfp4_scaled_mm_workspace_bytes(128, 1024, 8192) == 0
-    assert plan("nvfp4_scaled_mm", 128, 1024, 8192).startswith("nvfp4_skinny_ring_kernel<")
-    need = lib.nvf_nvfp4_scaled_mm_workspace_bytes(128, 1024, 8224)
-    assert need == 8 * 128 * 1024 * 4
-    assert plan("nvfp4_scaled_mm", 128, 1024, 8224, ws=need).startswith("nvfp4_tile_kernel<128,128,split_k>")
+    # few tiles and a deep K: the streaming kernel where it runs (up to 256 rows, K % 32 == 0: a short last chunk is
+    # fine), else the tile kernel's split
+    for k in (8192, 8224):
+        assert lib.nvf_nvfp4_scaled_mm_workspace_bytes(128, 1024, k) == 0
+        assert plan("nvfp4_scaled_mm", 128, 1024, k).startswith("nvfp4_skinny_ring_kernel<")
+    need = lib.nvf_nvfp4_scaled_mm_workspace_bytes(384, 4224, 8224)
+    assert need == 5 * 384 * 4224 * 4
+    assert plan("nvfp4_scaled_mm", 384, 4224, 8224, ws=need).startswith("nvfp4_tile_kernel<128,128,split_k>")
 
 
 @pytest.mark.parametrize("m,n,k,kernel", [

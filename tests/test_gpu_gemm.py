@@ -418,12 +418,40 @@ def test_mxfp8_gemm_k_not_a_multiple_of_128_on_the_streaming_kernel(dev, shape):
         assert torch.equal(out, _run_mxfp8(a8, b8, sa8_p, sb8_p, 0.75, dtype, dev))
 
 
-@pytest.mark.parametrize("shape", [(128, 1024, 8224), (100, 256, 8224), (200, 512, 10272), (65, 160, 9248), (300, 2048, 14368),
+@pytest.mark.parametrize("shape", [(16, 4096, 2880), (128, 5760, 2880), (300, 4096, 2880), (64, 512, 96), (7, 256, 32), (100, 1024, 4192),
+                                   (128, 1024, 8224), (100, 256, 8224), (200, 512, 10272), (65, 160, 9248), (300, 2048, 14368)])
+def test_nvfp4_gemm_k_not_a_multiple_of_128_on_the_streaming_kernel(dev, shape):
+    """K % 128 = 32, 64 or 96 on the weight-streaming kernel (all of its forms: 1, 2, 4 and 8 row tiles, several slabs,
+    ragged M): the last 128-deep chunk of a row is short; the bytes past the end of a row are the next row's and the
+    scale column tile past K may not exist.  NaN codes in all scale padding; every element against the oracle, both
+    output types, run-to-run bit equality."""
+    from fuser_amd import capi
+
+    m, n, k = shape
+    gen = torch.Generator().manual_seed(m + n + k)
+    a, sa, ga = _nvfp4_operand(m, k, 1.0, gen)
+    b, sb, gb = _nvfp4_operand(n, k, 0.02, gen)
+    alpha = 1.0 / (ga * gb)
+    ref = O.ref_nvfp4_scaled_mm(a, b, sa, sb, alpha)
+    sa_p, sb_p = sa.clone(), sb.clone()
+    sa_p[O.linear_to_swizzled_128_4(torch.ones(m, k // 16, dtype=torch.uint8)) == 0] = 0x7F
+    sb_p[O.linear_to_swizzled_128_4(torch.ones(n, k // 16, dtype=torch.uint8)) == 0] = 0x7F
+    plan = capi.describe_dispatch("nvfp4_scaled_mm", m, n, k)
+    assert plan.startswith("nvfp4_skinny_ring_kernel<") and ";" not in plan, plan
+    for dtype in (torch.bfloat16, torch.float16):
+        out = _run_nvfp4(a, b, sa_p, sb_p, alpha, dtype, dev)
+        assert out.shape == (m, n) and torch.isfinite(out.float()).all()
+        assert max_rel_rowwise(out, ref) <= GEMM_MAX_REL, (shape, dtype, plan)
+        assert torch.equal(out, _run_nvfp4(a, b, sa_p, sb_p, alpha, dtype, dev))
+
+
+@pytest.mark.parametrize("shape", [(384, 4224, 8224), (384, 5152, 10272), (384, 6176, 14368), (384, 4224, 8192),
                                    (80, 6144, 8192), (70, 8192, 7168), (72, 4736, 10752), (65, 4096, 14336)])
 def test_nvfp4_gemm_split_k_with_workspace(dev, shape):
-    """Few 128x128 output tiles and a deep K that the weight-streaming kernel cannot take (K % 128 != 0): with the
-    scratch memory that nvf_nvfp4_scaled_mm_workspace_bytes asks for, K is split over workgroups of the tile kernel
-    and fp32 partial tiles are added in a fixed order.  Ragged M / N / K (splits that do not divide the spans), both
+    """Fewer 128x128 output tiles than compute units and a deep K where neither the weight-streaming kernel (more than
+    256 rows in too many rounds of workgroups) nor the persistent kernel (N % 256 != 0) runs: with the scratch memory
+    that nvf_nvfp4_scaled_mm_workspace_bytes asks for, K is split over workgroups of the tile kernel and fp32 partial
+    tiles are added in a fixed order.  Ragged N / K (splits that do not divide the spans), both
     output types, against the oracle; run-to-run bit equality; a workspace that is too small, NULL or misaligned falls
     back to the kernels without one.  The last four shapes (one slab of 65..96 rows, N / 64 workgroups covering half
     the chip or less, K % 128 == 0, 28+ chunks per split, 48 Mi weights or more) split K over workgroups of the

@@ -20,8 +20,8 @@ def test_chain_replays_bit_exactly(dev):
     x = torch.randn(m, k, device=dev, generator=gen).bfloat16()
     w = (torch.randn(n, k, device=dev, generator=gen) * 0.05).bfloat16()
     xs = torch.randn(16, k, device=dev, generator=gen).bfloat16()            # decode-sized activations
-    xd = torch.randn(128, 8224, device=dev, generator=gen).bfloat16()        # few tiles, deep ragged K: split K
-    wd = (torch.randn(256, 8224, device=dev, generator=gen) * 0.05).bfloat16()
+    xd = torch.randn(72, 8192, device=dev, generator=gen).bfloat16()         # one slab of 65..96 rows, deep K: split K
+    wd = (torch.randn(6144, 8192, device=dev, generator=gen) * 0.05).bfloat16()
     sizes = [100, 0, 300, 112]
     eo = start_offsets(sizes).to(dev)
     so = start_offsets([O.round_up(t, 128) for t in sizes]).to(dev)
@@ -46,7 +46,7 @@ def test_chain_replays_bit_exactly(dev):
         # its first call per device, which looks the array's address up, is the eager run below, outside the capture)
         static = torch.empty_like(split)
         capi.check(capi.lib().nvf_nvfp4_scaled_mm_static_ws(dq.data_ptr(), wdq.data_ptr(), dsf.data_ptr(), wdsf.data_ptr(), one.data_ptr(),
-                                                            static.data_ptr(), 128, 256, 8224, capi.F16,
+                                                            static.data_ptr(), 72, 6144, 8192, capi.F16,
                                                             torch.cuda.current_stream().cuda_stream))
         gq, gsf = ops.nv_grouped_block_quantize(x, eo, so, None, 16)
         wgq = torch.stack([ops.nv_block_quantize(wg[e], None, True, 16)[0].view(torch.uint8) for e in range(len(sizes))])
@@ -66,7 +66,7 @@ def test_chain_replays_bit_exactly(dev):
                 rq.view(torch.uint8), rsf.view(torch.uint8)]
 
     eager = [t.clone() for t in chain()]  # also the warm-up: function attributes are set outside the capture
-    assert capi.lib().nvf_nvfp4_scaled_mm_workspace_bytes(128, 256, 8224) > 0 and torch.equal(eager[3], eager[4])
+    assert capi.lib().nvf_nvfp4_scaled_mm_workspace_bytes(72, 6144, 8192) > 0 and torch.equal(eager[3], eager[4])
     torch.cuda.synchronize()
     side = torch.cuda.Stream()
     with torch.cuda.stream(side):

@@ -22,8 +22,9 @@ def test_static_scratch_entry_point_equals_the_workspace_entry_point(dev):
     from fuser_amd import capi
 
     lib = capi.lib()
-    # two split-K shapes, the second smaller in every dimension (ragged M / N / K); then the first again
-    for call, (m, n, k) in enumerate([(200, 512, 10272), (100, 256, 8224), (80, 6144, 8192), (200, 512, 10272)]):
+    # two split-K shapes of the tile kernel, the second smaller in every dimension (ragged N / K), one of the
+    # weight-streaming kernel; then the first again
+    for call, (m, n, k) in enumerate([(384, 6176, 10272), (384, 4224, 8224), (80, 6144, 8192), (384, 6176, 10272)]):
         gen = torch.Generator().manual_seed(100 + call)
         a, sa, ga = _operand(m, k, 1.0, gen)
         b, sb, gb = _operand(n, k, 0.02, gen)
@@ -62,13 +63,13 @@ def test_static_scratch_entry_point_equals_the_workspace_entry_point(dev):
     # The largest scratch any split asks for on 256 compute units is exactly the static array (at most 2 x 256 work
     # items of 128 x 128 fp32): such a shape is accepted and runs; the size check itself is exercised on the CPU
     # side of the C ABI only where a device reports more compute units.
-    m, n, k = 256, 8192, 16416  # (K % 128 != 0: the tile kernel's split; K / 16 = 1026 scale columns, padded to 1028)
+    m, n, k = 512, 4096, 8224  # (the tile kernel's split, 4 x 128 tiles; K / 16 = 514 scale columns, padded to 516)
     assert lib.nvf_nvfp4_scaled_mm_workspace_bytes(m, n, k) == capi.STATIC_SCRATCH_BYTES
     g = torch.Generator(device=dev).manual_seed(3)
     ad = torch.randint(0, 256, (m, k // 2), dtype=torch.uint8, device=dev, generator=g)
     bd = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device=dev, generator=g)
-    sad = torch.randint(0x20, 0x40, (m, 1028), dtype=torch.uint8, device=dev, generator=g)
-    sbd = torch.randint(0x20, 0x40, (n, 1028), dtype=torch.uint8, device=dev, generator=g)
+    sad = torch.randint(0x20, 0x40, (m, 516), dtype=torch.uint8, device=dev, generator=g)
+    sbd = torch.randint(0x20, 0x40, (n, 516), dtype=torch.uint8, device=dev, generator=g)
     al = torch.tensor(2.0 ** -6, dtype=torch.float32, device=dev)
     ws = torch.full((capi.STATIC_SCRATCH_BYTES,), 0xFF, dtype=torch.uint8, device=dev)
     want = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
