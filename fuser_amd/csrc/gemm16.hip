@@ -174,7 +174,7 @@ struct DensePlan {
 };
 DensePlan nvfp4_dense_plan(int64_t m, int64_t n, int64_t k, int cus) {
   const bool stream_ok = (k & 31) == 0 && (n & 15) == 0 && k * 64 < (1ll << 31);  // 32-bit lane offsets (a short last chunk is fine)
-  const bool persistent_ok = (m & 127) == 0 && (n & 255) == 0 && (k & 127) == 0 && k >= 256;
+  const bool persistent_ok = (m & 127) == 0 && (n & 255) == 0 && (k & 31) == 0 && k >= 256;  // (a short last span is fine)
   int64_t cost256 = INT64_MAX, cost128 = INT64_MAX, cost_tile = INT64_MAX;
   if (persistent_ok) {
     const int64_t t256 = (m & 255) == 0 ? (m / 256) * (n / 256) : 0, t128 = (m / 128) * (n / 256);
@@ -184,7 +184,7 @@ DensePlan nvfp4_dense_plan(int64_t m, int64_t n, int64_t k, int cus) {
     cost_tile = full * 68 + (rest == 0 ? 0 : rest > cus ? 68 : full ? 45 : 22 + 25 * rest / cus);
   }
   const int64_t cost_min = std::min(cost256, std::min(cost128, cost_tile));
-  const int64_t rest_ns = persistent_ok ? 6000 + cost_min * 240 * k / 1024 : INT64_MAX;
+  const int64_t rest_ns = persistent_ok ? 6000 + cost_min * 240 * ((k + 127) & ~127ll) / 1024 : INT64_MAX;
   if (stream_ok) {
     // the streaming kernel's estimate is in ns within 0.8 (K = 2048) .. 1.1 (K = 14336)
     const int64_t stream_ns = nvfp4_skinny_best(m, n, k, cus, nullptr, nullptr) * (k < 3072 ? 82 : k < 6144 ? 96 : k < 10240 ? 103 : 110) / 100;
@@ -505,7 +505,7 @@ int launch_gemm16(int op, const Gemm16Args& a, hipStream_t stream) {
     // Dense with N not a multiple of 256 (29568, 1408) and enough rows for the persistent kernel: the columns up to the
     // last multiple of 256 go to whatever kernel that shape gets, the remaining columns (weight rows) to a launch of
     // their own that writes into the same rows of the result.
-    if (op == 0 && (p.n & 255) != 0 && p.n > 256 && p.m >= 512 && (p.k & 127) == 0 && p.k >= 256) {
+    if (op == 0 && (p.n & 255) != 0 && p.n > 256 && p.m >= 512 && (p.k & 31) == 0 && p.k >= 256) {
       const DensePlan::Kernel main_kernel = nvfp4_dense_plan(p.m & ~127, p.n & ~255, p.k, cus).kernel;
       if (main_kernel == DensePlan::kStream)  // (takes any M and any N % 16 == 0)
         return bf16 ? launch_nvfp4_skinny<true>(p, cus, stream) : launch_nvfp4_skinny<false>(p, cus, stream);

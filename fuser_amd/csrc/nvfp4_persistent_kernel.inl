@@ -1,6 +1,7 @@
 // Persistent 256x256 / 128x256 NVFP4 kernel of gemm16.hip (included there, inside namespace nvf).
 // -------------------------------------------------------------------------------------------------
-// NVFP4 fast path: 256x256 (or 128x256) tile, N % 256 == 0, K % 128 == 0, K >= 256; dense with M % 256 (128) == 0,
+// NVFP4 fast path: 256x256 (or 128x256) tile, N % 256 == 0, K % 128 == 0 (dense with a 16-bit result: K % 32 == 0),
+// K >= 256; dense with M % 256 (128) == 0,
 // or the whole 256-row tiles of every group of the grouped op; 16-bit or fp32 result.
 //   * 512 threads: 8 wavefronts as 2 (m) x 4 (n), each with a 128x64 (64x64) accumulator tile, two per SIMD.
 //     A single wavefront issues at most one non-MFMA instruction per ~8 cycles, which is too little for
@@ -27,7 +28,10 @@
 // TM = 32-row accumulator tiles of a wavefront along M: 4 -> 256x256 workgroup tile, 2 -> 128x256 (dense shapes
 // whose 256x256 tiles would leave compute units idle; 1.5 times the conversion work per MFMA).  The statement
 // order for TM = 4 is the one the 8192^3 measurements were made with.
-template <bool OUT_BF16, bool GROUPED, int TM = 4, bool OUT_F32 = false, bool PAIRS = false, bool OUT_FP4 = false>
+// RAGGED_K (dense, 16-bit result): K % 128 = 32, 64 or 96.  A tile's last span is short: the threads whose 32 elements lie
+// past K fetch their row's first piece instead of the next row's bytes, and their scale load runs past the range of its
+// buffer resource on purpose, which makes it return zero - and a zero scale makes a block count as zero.
+template <bool OUT_BF16, bool GROUPED, int TM = 4, bool OUT_F32 = false, bool PAIRS = false, bool OUT_FP4 = false, bool RAGGED_K = false>
 __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   static_assert(TM == 4 || TM == 2, "tile height");
   constexpr int BM = 64 * TM, BN = 256;
@@ -143,8 +147,8 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   if (first_tile >= range_end) return;
 
   const int kbytes = p.k >> 1;
-  const int nmac = p.k >> 7;       // 128-deep load spans per tile (>= 2)
-  const int sf_padded = p.k >> 4;  // K % 128 == 0: no padding columns
+  const int nmac = (p.k + 127) >> 7;            // 128-deep load spans per tile (>= 2)
+  const int sf_padded = ((p.k >> 4) + 3) & ~3;  // scale columns with the layout's padding
   const int64_t row128 = (int64_t)128 * kbytes;       // payload distance of the thread's two rows
   const int64_t sfrow128 = (int64_t)128 * sf_padded;  // same for the scales (next 128-row tile)
 
@@ -169,8 +173,12 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
     r.sb = p.sfb + (int64_t)w.g * p.n * sf_padded + swizzle_128x4(w.n0, 0, sf_padded);
     return r;
   };
-  const uint32_t off_ab = (uint32_t)srow * (uint32_t)kbytes + (uint32_t)spiece * 16u;
-  const uint32_t off_sf = (uint32_t)swizzle_128x4(srow, 0, sf_padded) + (uint32_t)(spiece >> 1) * 512u + (uint32_t)(spiece & 1) * 2u;
+  const uint32_t off_ab_full = (uint32_t)srow * (uint32_t)kbytes + (uint32_t)spiece * 16u;
+  const uint32_t off_sf_full = (uint32_t)swizzle_128x4(srow, 0, sf_padded) + (uint32_t)(spiece >> 1) * 512u + (uint32_t)(spiece & 1) * 2u;
+  // RAGGED_K: the offsets for a tile's last span
+  const bool in_tail = spiece * 32 < (p.k & 127);
+  const uint32_t off_ab_tail = in_tail ? off_ab_full : off_ab_full - (uint32_t)spiece * 16u;
+  const uint32_t off_sf_tail = in_tail ? off_sf_full : 0x7fffffffu;
   RowPtrs lp = tile_ptrs(first_tile);
   RowPtrs np = lp;
   int l_mac = 0;
@@ -183,6 +191,8 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   };
   auto issue_load_unit = [&](Raw& r, int q) {
     const int o = l_mac * 64, so = l_mac * 1024;
+    const bool tail = RAGGED_K && l_mac == nmac - 1;  // wave-uniform
+    const uint32_t off_ab = tail ? off_ab_tail : off_ab_full, off_sf = tail ? off_sf_tail : off_sf_full;
     if (q == 0) r.a[0] = __builtin_amdgcn_raw_buffer_load_b128(rsrc(lp.a, lp.a_bytes), off_ab, o, 0);
     // (rows 128.. of the tile through a resource of their own, so that the range check that zeroes the rows past a
     // group never depends on whether the hardware counts the scalar offset)
@@ -514,17 +524,17 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
 #undef NVF_PIN_ACC
 }
 
-template <bool OUT_BF16, bool GROUPED, int TM, bool OUT_F32, bool PAIRS, bool OUT_FP4 = false>
+template <bool OUT_BF16, bool GROUPED, int TM, bool OUT_F32, bool PAIRS, bool OUT_FP4 = false, bool RAGGED_K = false>
 int launch_nvfp4_fast_cfg(const Params& p, int cus, hipStream_t stream) {
-  auto kern = nvfp4_gemm_256_kernel<OUT_BF16, GROUPED, TM, OUT_F32, PAIRS, OUT_FP4>;
+  auto kern = nvfp4_gemm_256_kernel<OUT_BF16, GROUPED, TM, OUT_F32, PAIRS, OUT_FP4, RAGGED_K>;
   constexpr int lds_bytes = 2 * (64 * TM + 256) * 128 + 8 * 2560;  // 128 KiB / 96 KiB of tiles + the epilogue's 20 KiB
   // grouped: an upper bound (128-row tiles: one per weight panel and group of at least rows_lo rows)
   const int64_t tiles_m = (GROUPED && TM == 2) ? std::min<int64_t>(p.groups, p.m / std::max(p.rows_lo, 1)) : p.m / (64 * TM);
   const int64_t tiles = tiles_m * (p.n / 256);
   const unsigned grid = (unsigned)(tiles >= cus ? (cus & ~7) : ((tiles + 7) / 8) * 8);
   if (grid == 0) return NVF_OK;  // fewer rows in the whole call than the smallest group this launch serves: no work
-  if (note_launch("nvfp4_gemm_256_kernel<grouped=%d,TM=%d,f32=%d,pairs=%d%s> grid=%u rows=%d..%d min_rows=%d", (int)GROUPED, TM, (int)OUT_F32,
-                  (int)PAIRS, OUT_FP4 ? ",fp4_blockscale" : "", grid, p.rows_lo, p.rows_hi, p.min_rows))
+  if (note_launch("nvfp4_gemm_256_kernel<grouped=%d,TM=%d,f32=%d,pairs=%d%s%s> grid=%u rows=%d..%d min_rows=%d", (int)GROUPED, TM, (int)OUT_F32,
+                  (int)PAIRS, OUT_FP4 ? ",fp4_blockscale" : "", RAGGED_K ? ",ragged_k" : "", grid, p.rows_lo, p.rows_hi, p.min_rows))
     return NVF_OK;
   static std::atomic<uint64_t> configured{0};  // one bit per device
   if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
@@ -535,6 +545,12 @@ int launch_nvfp4_fast_cfg(const Params& p, int cus, hipStream_t stream) {
 template <bool OUT_BF16, bool GROUPED, int TM = 4, bool OUT_F32 = false, bool OUT_FP4 = false>
 int launch_nvfp4_fast(const Params& p, int cus, hipStream_t stream) {
   // an even number of 128-deep spans per tile: the variant whose two in-flight spans swap names instead of being copied
+  if constexpr (!GROUPED && !OUT_F32 && !OUT_FP4) {
+    if ((p.k & 127) != 0) {  // a short last span: an even number of spans counts it
+      if ((((p.k + 127) >> 7) & 1) == 0) return launch_nvfp4_fast_cfg<OUT_BF16, GROUPED, TM, OUT_F32, true, OUT_FP4, true>(p, cus, stream);
+      return launch_nvfp4_fast_cfg<OUT_BF16, GROUPED, TM, OUT_F32, false, OUT_FP4, true>(p, cus, stream);
+    }
+  }
   if (((p.k >> 7) & 1) == 0) return launch_nvfp4_fast_cfg<OUT_BF16, GROUPED, TM, OUT_F32, true, OUT_FP4>(p, cus, stream);
   return launch_nvfp4_fast_cfg<OUT_BF16, GROUPED, TM, OUT_F32, false, OUT_FP4>(p, cus, stream);
 }

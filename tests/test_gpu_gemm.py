@@ -445,6 +445,32 @@ def test_nvfp4_gemm_k_not_a_multiple_of_128_on_the_streaming_kernel(dev, shape):
         assert torch.equal(out, _run_nvfp4(a, b, sa_p, sb_p, alpha, dtype, dev))
 
 
+@pytest.mark.parametrize("shape", [(2048, 4096, 4160), (2048, 4096, 2976), (4096, 5120, 2880), (4096, 4096, 1504), (2048, 5760, 2880),
+                                   (2100, 4096, 2880)])
+def test_nvfp4_gemm_k_not_a_multiple_of_128_on_the_persistent_kernel(dev, shape):
+    """K % 128 = 32, 64 or 96 on the persistent kernel (128x256 and 256x256 tiles, an odd and an even number of spans;
+    the last two shapes are cut along N and along M as well): a tile's last span is short.  NaN codes in all scale
+    padding; every element against the oracle, both output types, run-to-run bit equality."""
+    from fuser_amd import capi
+
+    m, n, k = shape
+    gen = torch.Generator().manual_seed(m + n + k)
+    a, sa, ga = _nvfp4_operand(m, k, 1.0, gen)
+    b, sb, gb = _nvfp4_operand(n, k, 0.02, gen)
+    alpha = 1.0 / (ga * gb)
+    ref = O.ref_nvfp4_scaled_mm(a, b, sa, sb, alpha)
+    sa_p, sb_p = sa.clone(), sb.clone()
+    sa_p[O.linear_to_swizzled_128_4(torch.ones(m, k // 16, dtype=torch.uint8)) == 0] = 0x7F
+    sb_p[O.linear_to_swizzled_128_4(torch.ones(n, k // 16, dtype=torch.uint8)) == 0] = 0x7F
+    plan = capi.describe_dispatch("nvfp4_scaled_mm", m, n, k)
+    assert "nvfp4_gemm_256_kernel<" in plan and "ragged_k" in plan, plan
+    for dtype in (torch.bfloat16, torch.float16):
+        out = _run_nvfp4(a, b, sa_p, sb_p, alpha, dtype, dev)
+        assert out.shape == (m, n) and torch.isfinite(out.float()).all()
+        assert max_rel_rowwise(out, ref) <= GEMM_MAX_REL, (shape, dtype, plan)
+        assert torch.equal(out, _run_nvfp4(a, b, sa_p, sb_p, alpha, dtype, dev))
+
+
 @pytest.mark.parametrize("shape", [(384, 4224, 8224), (384, 5152, 10272), (384, 6176, 14368), (384, 4224, 8192),
                                    (80, 6144, 8192), (70, 8192, 7168), (72, 4736, 10752), (65, 4096, 14336)])
 def test_nvfp4_gemm_split_k_with_workspace(dev, shape):
