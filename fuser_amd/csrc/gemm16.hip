@@ -335,6 +335,16 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int6
     // Grouped NVFP4: groups of up to 128 rows (MoE decode, the small experts of a prefill) stream their expert's
     // weights once through the skinny kernel; the launches below then skip them.  The group sizes live on
     // the device, so every kernel is always launched; workgroups without work return at once.
+    if (!dense && p.min_rows == 0 && (p.n & 63) == 0 && (p.k & 127) != 0 && (p.k & 31) == 0 && (int64_t)p.k * 64 < (1ll << 31)) {
+      // K % 128 = 32, 64 or 96: the groups of up to 128 rows on the streaming kernel's variant with a short last chunk
+      // (the form that splits K over the wavefronts), larger groups on the tile kernels
+      int rc = launch_nvfp4_skinny_grouped<4, 2, OUT_BF16, false>(p, 1, 32, stream);
+      if (rc == NVF_OK) rc = launch_nvfp4_skinny_grouped<4, 8, OUT_BF16, false>(p, 33, 128, stream);
+      if (rc != NVF_OK) return rc;
+      Params rest = p;
+      rest.min_rows = 129;
+      return launch_sized<NVFP4, BF16_MMA, OUT_BF16>(rest, m_hint, cus, workspace, workspace_bytes, stream);
+    }
     if (!dense && p.min_rows == 0 && (p.n & 63) == 0 && (p.k & 127) == 0 && (int64_t)p.k * 64 < (1ll << 31)) {
       // With a shallow K a split of K over the wavefronts leaves each only a chunk or two: they then own
       // different weight rows instead (K=2048, N=7168: 549 -> 464 us for 64 tokens x top-8; deeper K: slower).

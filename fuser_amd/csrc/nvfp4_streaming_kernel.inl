@@ -684,7 +684,8 @@ int launch_nvfp4_skinny_grouped(const Params& p0, int rows_lo, int rows_hi, hipS
   // over 256 experts, K=7168: 401 -> 375 us; K=2048: 432 -> 413 us).  Forcing the registers down to two
   // workgroups per compute unit on top of that costs more than it gains (450 us).
   constexpr int DEPTH = 1;
-  auto kern = nvfp4_skinny_ring_kernel<RT, TT, OUT_BF16, DEPTH, true, NSPLIT>;
+  auto kern = (p0.k & 127) != 0 ? nvfp4_skinny_ring_kernel<RT, TT, OUT_BF16, DEPTH, true, NSPLIT, true>
+                                : nvfp4_skinny_ring_kernel<RT, TT, OUT_BF16, DEPTH, true, NSPLIT>;
   constexpr int red_kib = NSPLIT ? 0 : 8 * (RT * TT <= 8 ? RT * TT : TT);
   constexpr int ring_kib = 8 * DEPTH * SLOT_KIB;
   constexpr int lds_bytes = (ring_kib > red_kib ? ring_kib : red_kib) * 1024;
@@ -697,8 +698,8 @@ int launch_nvfp4_skinny_grouped(const Params& p0, int rows_lo, int rows_hi, hipS
   if (note_launch("nvfp4_skinny_ring_kernel<RT=%d,TT=%d,grouped,nsplit=%d> grid=%lld rows=%d..%d", RT, TT, (int)NSPLIT, (long long)wgs, rows_lo,
                   rows_hi))
     return NVF_OK;
-  static std::atomic<uint64_t> configured{0};  // one bit per device
-  if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
+  static std::atomic<uint64_t> configured[2] = {{0}, {0}};  // per kernel, one bit per device
+  if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured[(p.k & 127) != 0])) return rc;
   hipLaunchKernelGGL(kern, dim3((unsigned)wgs), dim3(512), lds_bytes, stream, p);
   return check_launch("nvfp4_skinny_ring_kernel (grouped)");
 }

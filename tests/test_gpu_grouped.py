@@ -301,10 +301,11 @@ def test_nvfp4_grouped_mm_whole_tiles_and_group_ends(dev, sizes, n, k):
         assert ((out[:rows].float().cpu() - ref[:rows]).abs() / scale).max().item() <= GEMM_MAX_REL, (sizes, dtype)
 
 
-@pytest.mark.parametrize("n,k", [(128, 128), (384, 384), (256, 1152), (128, 2048), (256, 4096), (512, 5120)])
+@pytest.mark.parametrize("n,k", [(128, 128), (384, 384), (256, 1152), (128, 2048), (256, 4096), (512, 5120), (256, 320), (512, 2880), (128, 192)])
 def test_nvfp4_grouped_mm_small_groups_stream_their_weights(dev, n, k):
-    """K % 128 == 0: groups of 1..32 and of 33..128 rows each run on the weight-streaming kernel (one workgroup
-    per group and 64 weight rows), larger groups on the tile kernels, which skip the small ones.  Sizes on
+    """Groups of 1..32 and of 33..128 rows each run on the weight-streaming kernel (one workgroup
+    per group and 64 weight rows), larger groups on the tile kernels, which skip the small ones; the last three
+    shapes have K % 128 = 64 (a short last chunk).  Sizes on
     both sides of every class border, empty groups, a different alpha per group, poisoned padding of the
     activation scale slabs, one to forty 128-deep chunks (wavefronts without work); N % 256 == 0 with K < 4096
     takes the variant whose wavefronts own different weight rows, the rest the one that splits K; every
@@ -335,6 +336,8 @@ def test_nvfp4_grouped_mm_small_groups_stream_their_weights(dev, n, k):
     ref = O.ref_nvfp4_scaled_grouped_mm(aq, bq, valid, bsf, alphas, ps, eo, so)
     rows = sum(sizes)
     args = (fp4(aq.to(dev)), fp4(bq.to(dev)), e4m3(asf.to(dev)), e4m3(bsf.to(dev)), alphas.to(dev), st, ct, ps.to(dev), eo.to(dev), so.to(dev))
+    from fuser_amd import capi
+    assert "nvfp4_skinny_ring_kernel<" in capi.describe_dispatch("nvfp4_scaled_grouped_mm", m, n, k, g)
     for dtype in (torch.bfloat16, torch.float16):
         out = nvf_cutlass.nvfp4_scaled_grouped_mm(*args, dtype)
         torch.cuda.synchronize()
