@@ -397,7 +397,7 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int6
     // Grouped NVFP4 with room for whole 256-row tiles: those go to the 256x256 kernel (about 1.4 times as
     // fast per flop), the ends of the groups to the 128x128 tile kernel.  The group sizes live on the
     // device, so both kernels are always launched; one that finds no work returns at once.
-    if (!dense && (p.n & 255) == 0 && (p.k & 127) == 0 && p.k >= 256 && m_hint >= kPrefillRows) {
+    if (!dense && (p.n & 255) == 0 && (p.k & 31) == 0 && p.k >= 256 && m_hint >= kPrefillRows) {
       const int rc = launch_nvfp4_fast<OUT_BF16, true>(p, cus, stream);
       if (rc != NVF_OK || p.tail_done) return rc;
       Params rest = p;

@@ -28,7 +28,7 @@
 // TM = 32-row accumulator tiles of a wavefront along M: 4 -> 256x256 workgroup tile, 2 -> 128x256 (dense shapes
 // whose 256x256 tiles would leave compute units idle; 1.5 times the conversion work per MFMA).  The statement
 // order for TM = 4 is the one the 8192^3 measurements were made with.
-// RAGGED_K (dense, 16-bit result): K % 128 = 32, 64 or 96.  A tile's last span is short: the threads whose 32 elements lie
+// RAGGED_K (16-bit result; grouped: the 256x256 tiles): K % 128 = 32, 64 or 96.  A tile's last span is short: the threads whose 32 elements lie
 // past K fetch their row's first piece instead of the next row's bytes, and their scale load runs past the range of its
 // buffer resource on purpose, which makes it return zero - and a zero scale makes a block count as zero.
 template <bool OUT_BF16, bool GROUPED, int TM = 4, bool OUT_F32 = false, bool PAIRS = false, bool OUT_FP4 = false, bool RAGGED_K = false>
@@ -545,7 +545,7 @@ int launch_nvfp4_fast_cfg(const Params& p, int cus, hipStream_t stream) {
 template <bool OUT_BF16, bool GROUPED, int TM = 4, bool OUT_F32 = false, bool OUT_FP4 = false>
 int launch_nvfp4_fast(const Params& p, int cus, hipStream_t stream) {
   // an even number of 128-deep spans per tile: the variant whose two in-flight spans swap names instead of being copied
-  if constexpr (!GROUPED && !OUT_F32 && !OUT_FP4) {
+  if constexpr ((!GROUPED || TM == 4) && !OUT_F32 && !OUT_FP4) {
     if ((p.k & 127) != 0) {  // a short last span: an even number of spans counts it
       if ((((p.k + 127) >> 7) & 1) == 0) return launch_nvfp4_fast_cfg<OUT_BF16, GROUPED, TM, OUT_F32, true, OUT_FP4, true>(p, cus, stream);
       return launch_nvfp4_fast_cfg<OUT_BF16, GROUPED, TM, OUT_F32, false, OUT_FP4, true>(p, cus, stream);
