@@ -168,6 +168,10 @@ int launch_nvfp4_tile(const Params& p, int grid, hipStream_t stream) {
 // K): a round of 128-row tiles costs 58 (half the flops at 86 % of the rate); the tile kernels run their 128x128 tiles
 // two to a compute unit: 68 per such round, 45 for a last round of one tile per compute unit, and 22..47 when there
 // is no more than that in all (all measured: M = 128..1024, N = 2048..14336, K = 4096 and 14336).
+// the streaming kernel's cost estimate is in ns within 0.8 (K = 2048) .. 1.1 (K = 14336)
+int64_t nvfp4_stream_ns(int64_t m, int64_t n, int64_t k, int cus) {
+  return nvfp4_skinny_best(m, n, k, cus, nullptr, nullptr) * (k < 3072 ? 82 : k < 6144 ? 96 : k < 10240 ? 103 : 110) / 100;
+}
 struct DensePlan {
   enum Kernel { kStream, kTiles256, kTiles128, kOther } kernel;
   int64_t ns;  // estimated duration (INT64_MAX: no estimate)
@@ -186,10 +190,9 @@ DensePlan nvfp4_dense_plan(int64_t m, int64_t n, int64_t k, int cus) {
   const int64_t cost_min = std::min(cost256, std::min(cost128, cost_tile));
   const int64_t rest_ns = persistent_ok ? 6000 + cost_min * 240 * ((k + 127) & ~127ll) / 1024 : INT64_MAX;
   if (stream_ok) {
-    // the streaming kernel's estimate is in ns within 0.8 (K = 2048) .. 1.1 (K = 14336)
-    const int64_t stream_ns = nvfp4_skinny_best(m, n, k, cus, nullptr, nullptr) * (k < 3072 ? 82 : k < 6144 ? 96 : k < 10240 ? 103 : 110) / 100;
+    const int64_t stream_ns = nvfp4_stream_ns(m, n, k, cus);
     bool stream;
-    if (m <= 256) {
+    if (m <= 128 || (m <= 256 && !(persistent_ok && k >= 2048))) {
       stream = true;  // at most two passes over the weights (256 x 14336 x 4096: 38 instead of 58 us on tiles)
     } else if (persistent_ok && k >= 2048) {
       // by estimated duration (measured: 512 x 4096 x 14336 115 -> 57 us, 384 x 8192 x 7168 82 -> 57 us,
@@ -212,18 +215,58 @@ DensePlan nvfp4_dense_plan(int64_t m, int64_t n, int64_t k, int cus) {
   return {DensePlan::kOther, rest_ns};
 }
 
+// What a dense call does about an N that is no multiple of 256 (29568, 1408): 0 nothing; 1 the whole call goes to the
+// weight-streaming kernel (which takes any N % 16 == 0); 2 the columns up to the last multiple of 256 go to whatever
+// kernel that shape gets and the remaining columns (weight rows) to a launch of their own that writes into the same rows
+// of the result.  A cut competes with the kernel the whole shape gets: the tile kernels (no estimate) lose to any cut;
+// the weight-streaming kernel loses to one whose main part runs on the persistent kernel and is estimated 5 % faster.
+// (ns: the estimated duration of what is returned, where there is one)
+int nvfp4_n_cut(int64_t m, int64_t n, int64_t k, int cus, int64_t* ns = nullptr) {
+  if (ns) *ns = INT64_MAX;
+  if ((n & 255) == 0 || n <= 256 || m <= 128 || (k & 31) != 0 || k < 256) return 0;
+  const DensePlan whole = nvfp4_dense_plan(m, n, k, cus);
+  const DensePlan main_plan = nvfp4_dense_plan(m & ~127, n & ~255, k, cus), rest_plan = nvfp4_dense_plan(m, n & 255, k, cus);
+  const bool whole_other = whole.kernel == DensePlan::kOther;
+  if (main_plan.kernel == DensePlan::kOther) return 0;
+  const bool have_cut_ns = rest_plan.kernel == DensePlan::kStream && main_plan.ns != INT64_MAX;
+  const int64_t cut_ns = have_cut_ns ? main_plan.ns + rest_plan.ns : INT64_MAX;
+  if (whole_other) {
+    if (main_plan.kernel != DensePlan::kStream) {
+      if (ns) *ns = cut_ns;
+      return 2;
+    }
+    // all columns to the streaming kernel, or - a few columns past a whole number of rounds of its workgroups cost a
+    // round - those in a launch of their own (512 x 4224 x 8224: 264 workgroups at once, or 256 and then 8)
+    const int64_t stream_ns = (k & 31) == 0 && (n & 15) == 0 ? nvfp4_stream_ns(m, n, k, cus) : INT64_MAX;
+    const bool cut = have_cut_ns && cut_ns < stream_ns - stream_ns / 20;
+    if (ns) *ns = cut ? cut_ns : stream_ns;
+    return cut ? 2 : 1;
+  }
+  if (whole.kernel == DensePlan::kStream && main_plan.kernel != DensePlan::kStream && have_cut_ns && cut_ns < whole.ns - whole.ns / 20) {
+    if (ns) *ns = cut_ns;
+    return 2;
+  }
+  return 0;
+}
+
 // Dense shapes whose M is not a multiple of 128 and that only the tile kernels would take whole: the number of rows
 // (the last multiple of 128) that go to a launch of their own, if that shape gets a better kernel; else 0.  If that
 // kernel is the weight-streaming one, which takes any number of rows, the answer is m: no cut, all rows to it.
 int64_t nvfp4_rows_before_remainder(int64_t m, int64_t n, int64_t k, int cus) {
   if (m <= 128 || (m & 127) == 0 || (k & 15) != 0) return 0;
-  if (nvfp4_dense_plan(m, n, k, cus).kernel != DensePlan::kOther) return 0;
+  // Against the kernel the whole shape gets: the tile kernels (no estimate) lose to any cut; the weight-streaming kernel
+  // loses to a cut whose first part runs on the persistent kernel and is estimated 5 % faster or more (192 rows against
+  // 28672 weight rows: 128 of them on 128x256 tiles).
+  const DensePlan whole = nvfp4_dense_plan(m, n, k, cus);
+  const bool whole_other = whole.kernel == DensePlan::kOther;
+  if (!whole_other && whole.kernel != DensePlan::kStream) return 0;
   // the cut is the last multiple of 128 or of 256 (which allows 256x256 tiles), whichever is estimated faster
-  int64_t best = INT64_MAX, cut = 0;
+  int64_t best = whole_other ? INT64_MAX : whole.ns - whole.ns / 20, cut = 0;
   for (const int64_t c : {m & ~(int64_t)127, m & ~(int64_t)255}) {
     if (c < 128) continue;
     const DensePlan main = nvfp4_dense_plan(c, n, k, cus), rest = nvfp4_dense_plan(m - c, n, k, cus);
     if (main.kernel == DensePlan::kOther || rest.kernel != DensePlan::kStream || main.ns == INT64_MAX) continue;
+    if (!whole_other && main.kernel == DensePlan::kStream) continue;  // (the whole shape is on that kernel already)
     if (main.ns + rest.ns < best) best = main.ns + rest.ns, cut = main.kernel == DensePlan::kStream ? m : c;
   }
   return cut;
@@ -242,7 +285,13 @@ int nvfp4_splits(int64_t m, int64_t n, int64_t k, int cus) {
   int64_t s = (2 * (int64_t)cus) / tiles;
   if (s > nspans / 8) s = nspans / 8;
   if (s > 32) s = 32;
-  return s < 2 ? 1 : (int)s;
+  if (s < 2) return 1;
+  // N no multiple of 256: the split has to be estimated faster (25 us + 2 us per span of an item, two items to a compute
+  // unit) than what the call does otherwise - all columns, or those up to the last multiple of 256, on another kernel
+  // (384 x 4224 x 8224 50 us against 42 us streamed, 384 x 6176 x 14368 100 against 122 us)
+  int64_t other_ns;
+  if (nvfp4_n_cut(m, n, k, cus, &other_ns) != 0 && other_ns < 25000 + 2000 * ceil_div(nspans, s) * ceil_div(tiles * s, 2 * (int64_t)cus)) return 1;
+  return (int)s;
 }
 
 // Split of K over workgroups for the weight-streaming kernel with one slab of 65..96 activation rows: every
@@ -517,11 +566,11 @@ int launch_gemm16(int op, const Gemm16Args& a, hipStream_t stream) {
     // Dense with N not a multiple of 256 (29568, 1408) and enough rows for the persistent kernel: the columns up to the
     // last multiple of 256 go to whatever kernel that shape gets, the remaining columns (weight rows) to a launch of
     // their own that writes into the same rows of the result.
-    if (op == 0 && (p.n & 255) != 0 && p.n > 256 && p.m >= 512 && (p.k & 31) == 0 && p.k >= 256) {
-      const DensePlan::Kernel main_kernel = nvfp4_dense_plan(p.m & ~127, p.n & ~255, p.k, cus).kernel;
-      if (main_kernel == DensePlan::kStream)  // (takes any M and any N % 16 == 0)
-        return bf16 ? launch_nvfp4_skinny<true>(p, cus, stream) : launch_nvfp4_skinny<false>(p, cus, stream);
-      if (main_kernel != DensePlan::kOther) {
+    const bool split_wins = op == 0 && a.workspace != nullptr && nvfp4_splits(p.m, p.n, p.k, cus) > 1 &&
+                            a.workspace_bytes >= (int64_t)nvfp4_splits(p.m, p.n, p.k, cus) * p.m * p.n * 4;
+    if (const int n_cut = op == 0 && !split_wins ? nvfp4_n_cut(p.m, p.n, p.k, cus) : 0) {
+      if (n_cut == 1) return bf16 ? launch_nvfp4_skinny<true>(p, cus, stream) : launch_nvfp4_skinny<false>(p, cus, stream);
+      {
         Gemm16Args main = a, rest = a;
         main.n = p.n & ~255;
         rest.n = p.n - main.n;

@@ -779,7 +779,10 @@ int launch_skinny_rt(const Params& p, int rt, hipStream_t stream, int slabs) {
 // partly filled costs 70 % of a full one plus its share of the rest; the weight stream bounds the whole from below.
 // Constants fitted to a sweep of the seven forms over 140 shapes (M 48..256, N 1024..14336, K 2048..14336): the form
 // picked is within 7 % of the best everywhere.
-int64_t mxfp8_skinny_cost(int64_t m, int64_t n, int64_t k, int slab, int rt, int64_t cus) {
+// (duration: the estimate is compared with another kernel's; then a round of workgroups streams the weight rows it
+// covers, not all of them - with 28672 weight rows a slab takes two rounds, which made the other floor twice the
+// measured time; the choice of the form keeps the floor it was fitted with)
+int64_t mxfp8_skinny_cost(int64_t m, int64_t n, int64_t k, int slab, int rt, int64_t cus, bool duration = false) {
   if ((slab == 128 && rt != 1) || n % (16 * rt) != 0) return INT64_MAX;
   const int64_t slabs = m <= slab ? 1 : ceil_div(m, slab);
   const int tt = m <= slab ? (m <= 16 ? 1 : m <= 32 ? 2 : m <= 64 ? 4 : 8) : slab / 16;
@@ -791,7 +794,7 @@ int64_t mxfp8_skinny_cost(int64_t m, int64_t n, int64_t k, int slab, int rt, int
   const int64_t full = wgs / cus, rest = wgs - full * cus;
   // every round of workgroups streams the weights again, out of the last-level cache at best: 5.6 TB/s
   // (256 x 14336 x 14336 as 4 slabs in 3.5 rounds: 123 us for 4 x 205 MB)
-  const int64_t stream = ceil_div(wgs, cus) * n * k / 5400;
+  const int64_t stream = ceil_div(wgs, cus) * (duration ? std::min<int64_t>(n, cus * 16 * rt) : n) * k / 5400;
   return std::max((full * 100 + (rest ? 70 + 30 * rest / cus : 0)) * wg_time / 100, stream);
 }
 
@@ -807,6 +810,12 @@ int64_t mxfp8_skinny_best(int64_t m, int64_t n, int64_t k, int64_t cus, int* sla
   if (slab_out) *slab_out = slab;
   if (rt_out) *rt_out = rt;
   return best;
+}
+// estimated duration of the form that mxfp8_skinny_best picks, in ns
+int64_t mxfp8_skinny_ns(int64_t m, int64_t n, int64_t k, int64_t cus) {
+  int slab, rt;
+  if (mxfp8_skinny_best(m, n, k, cus, &slab, &rt) == INT64_MAX) return INT64_MAX;
+  return mxfp8_skinny_cost(m, n, k, slab, rt, cus, true) * 963 / 1000;
 }
 
 template <bool OUT_BF16>
@@ -855,7 +864,7 @@ Plan mxfp8_plan(int64_t m, int64_t n, int64_t k, int64_t cus, int64_t* ns = null
   const bool fast = cost256 != INT64_MAX || cost128 != INT64_MAX;
   const int64_t fast_ns = fast ? 5000 + std::min(cost256, cost128) * 113 * ((k + 127) & ~127ll) / 1024 : INT64_MAX;
   if (skinny_ok) {
-    const int64_t skinny_ns = mxfp8_skinny_best(m, n, k, cus, nullptr, nullptr) * 963 / 1000;
+    const int64_t skinny_ns = mxfp8_skinny_ns(m, n, k, cus);
     if (ns) *ns = skinny_ns;
     if (m <= 32) return Plan::kStream;
     if (fast) {
@@ -882,42 +891,51 @@ template <bool OUT_BF16>
 int launch_sized(const Params& p, hipStream_t stream) {
   auto tiles = [&](int bm, int bn) { return ceil_div(p.m, bm) * ceil_div(p.n, bn); };
   const int64_t cus = cu_count();
-  switch (mxfp8_plan(p.m, p.n, p.k, cus)) {
-    case Plan::kStream: return launch_skinny<OUT_BF16>(p, stream);
-    case Plan::kTiles256: return launch_fast<4, OUT_BF16>(p, stream);
-    case Plan::kTiles128: return launch_fast<2, OUT_BF16>(p, stream);
-    case Plan::kOther: break;
+  int64_t whole_ns;
+  const Plan whole = mxfp8_plan(p.m, p.n, p.k, cus, &whole_ns);
+  // A cut along N or M competes with the kernel the whole shape gets: the tile kernels (no estimate) lose to any cut
+  // that works; the weight-streaming kernel loses to a cut whose main part runs on the persistent kernel and is
+  // estimated 5 % faster or more (384 x 29568 x 8192: 291 us on tiles, 256 x 29568 x 8192: 169 us streamed).
+  const bool whole_other = whole == Plan::kOther;
+  const int64_t bar = whole_other ? INT64_MAX : whole == Plan::kStream ? whole_ns - whole_ns / 20 : 0;
+  auto is_tiles = [](Plan q) { return q == Plan::kTiles256 || q == Plan::kTiles128; };
+  // N not a multiple of 256 (29568, 1408): the columns up to the last multiple of 256 go to whatever kernel that shape
+  // gets, the remaining columns (weight rows) to a launch of their own that writes into the same rows of the result
+  // (8192 x 29568 x 8192: 4.1 -> 1.3 ms).
+  if ((p.n & 255) != 0 && p.n > 256 && (p.n & 15) == 0 && p.m > 128 && (p.k & 31) == 0 && p.k >= 256) {
+    int64_t main_ns, rest_ns;
+    const Plan main_plan = mxfp8_plan(p.m & ~127, p.n & ~255, p.k, cus, &main_ns), rest_plan = mxfp8_plan(p.m, p.n & 255, p.k, cus, &rest_ns);
+    if (whole_other && main_plan == Plan::kStream) return launch_skinny<OUT_BF16>(p, stream);  // (takes any N % 16 == 0)
+    if (main_plan != Plan::kOther && (whole_other || (is_tiles(main_plan) && rest_plan == Plan::kStream && main_ns != INT64_MAX &&
+                                                       rest_ns != INT64_MAX && main_ns + rest_ns < bar))) {
+      Params main = p, rest = p;
+      main.n = p.n & ~255;
+      rest.n = p.n - main.n;
+      main.ldc = rest.ldc = p.out_pitch();
+      const int64_t sf_padded = ((int64_t)(p.k >> 5) + 3) & ~(int64_t)3;
+      rest.b = p.b + (int64_t)main.n * p.k;
+      rest.sfb = p.sfb + (int64_t)main.n * sf_padded;
+      rest.out = static_cast<uint8_t*>(p.out) + (int64_t)main.n * 2;
+      if (const int rc = launch_sized<OUT_BF16>(main, stream)) return rc;
+      return launch_sized<OUT_BF16>(rest, stream);
+    }
   }
-  // N not a multiple of 256 (29568, 1408) with enough rows for the persistent kernel: the columns up to the last
-  // multiple of 256 go to whatever kernel that shape gets, the remaining columns (weight rows) to a launch of their
-  // own that writes into the same rows of the result (8192 x 29568 x 8192: 4.1 -> 1.3 ms).
-  if ((p.n & 255) != 0 && p.n > 256 && (p.n & 15) == 0 && p.m >= 512 && (p.k & 31) == 0 && p.k >= 256 &&
-      mxfp8_plan(p.m & ~127, p.n & ~255, p.k, cus) != Plan::kOther) {
-    if (mxfp8_plan(p.m & ~127, p.n & ~255, p.k, cus) == Plan::kStream) return launch_skinny<OUT_BF16>(p, stream);  // (takes any N % 16 == 0)
-    Params main = p, rest = p;
-    main.n = p.n & ~255;
-    rest.n = p.n - main.n;
-    main.ldc = rest.ldc = p.out_pitch();
-    const int64_t sf_padded = ((int64_t)(p.k >> 5) + 3) & ~(int64_t)3;
-    rest.b = p.b + (int64_t)main.n * p.k;
-    rest.sfb = p.sfb + (int64_t)main.n * sf_padded;
-    rest.out = static_cast<uint8_t*>(p.out) + (int64_t)main.n * 2;
-    if (const int rc = launch_sized<OUT_BF16>(main, stream)) return rc;
-    return launch_sized<OUT_BF16>(rest, stream);
-  }
-  // M not a multiple of 128 (a prefill of any token count) and too many rows for the skinny kernel: the rows up to
-  // the last multiple of 128 go to whatever kernel that shape gets, the remaining rows (at most 127, a whole number
-  // of 128-row scale tiles further on) to the skinny kernel in a launch of their own (4000 x 4096 x 4096: 197 -> 77 us;
-  // 8100 x 8192 x 8192: 1475 -> 390 us).
+  // M not a multiple of 128 (a prefill of any token count): the rows up to the last multiple of 128 go to whatever kernel
+  // that shape gets, the remaining rows (at most 127, a whole number of 128-row scale tiles further on) to the skinny
+  // kernel in a launch of their own (4000 x 4096 x 4096: 197 -> 77 us; 8100 x 8192 x 8192: 1475 -> 390 us).
   // The cut is the last multiple of 128 or of 256 (which allows 256x256 tiles), whichever is estimated faster
   // (8100 x 8192 x 8192: 546 us cut at 8064, 128x256 tiles; 390 us cut at 7936).
-  if (p.m > 128 && (p.m & 127) != 0 && (p.k & 31) == 0) {
-    int64_t best = INT64_MAX;
+  if (p.m > 128 && (p.m & 127) != 0 && (p.k & 31) == 0 && (whole_other || whole == Plan::kStream)) {
+    int64_t best = bar;
     int cut = 0;
     for (const int c : {p.m & ~127, p.m & ~255}) {
       int64_t ns_main, ns_rest;
-      if (c < 128 || mxfp8_plan(c, p.n, p.k, cus, &ns_main) == Plan::kOther || mxfp8_plan(p.m - c, p.n, p.k, cus, &ns_rest) != Plan::kStream) continue;
-      if (ns_main + ns_rest < best) best = ns_main + ns_rest, cut = mxfp8_plan(c, p.n, p.k, cus) == Plan::kStream ? p.m : c;
+      if (c < 128) continue;
+      const Plan main_plan = mxfp8_plan(c, p.n, p.k, cus, &ns_main);
+      if (main_plan == Plan::kOther || mxfp8_plan(p.m - c, p.n, p.k, cus, &ns_rest) != Plan::kStream) continue;
+      if (!whole_other && main_plan == Plan::kStream) continue;  // (the whole shape is on that kernel already)
+      if (ns_main == INT64_MAX || ns_rest == INT64_MAX) continue;
+      if (ns_main + ns_rest < best) best = ns_main + ns_rest, cut = main_plan == Plan::kStream ? p.m : c;
     }
     if (cut == p.m) return launch_skinny<OUT_BF16>(p, stream);  // (the skinny kernel takes any number of rows)
     if (cut) {
@@ -931,6 +949,12 @@ int launch_sized(const Params& p, hipStream_t stream) {
       if (const int rc = launch_sized<OUT_BF16>(main, stream)) return rc;
       return launch_sized<OUT_BF16>(rest, stream);
     }
+  }
+  switch (whole) {
+    case Plan::kStream: return launch_skinny<OUT_BF16>(p, stream);
+    case Plan::kTiles256: return launch_fast<4, OUT_BF16>(p, stream);
+    case Plan::kTiles128: return launch_fast<2, OUT_BF16>(p, stream);
+    case Plan::kOther: break;
   }
   if (tiles(256, 256) >= cus) return launch_cfg<256, 256, OUT_BF16>(p, stream);
   if (tiles(128, 128) >= cus) return launch_cfg<128, 128, OUT_BF16>(p, stream);

@@ -471,11 +471,11 @@ def test_nvfp4_gemm_k_not_a_multiple_of_128_on_the_persistent_kernel(dev, shape)
         assert torch.equal(out, _run_nvfp4(a, b, sa_p, sb_p, alpha, dtype, dev))
 
 
-@pytest.mark.parametrize("shape", [(384, 4224, 8224), (384, 5152, 10272), (384, 6176, 14368), (384, 4224, 8192),
+@pytest.mark.parametrize("shape", [(384, 6176, 8224), (512, 5152, 8224), (640, 4224, 12320), (512, 3104, 12320),
                                    (80, 6144, 8192), (70, 8192, 7168), (72, 4736, 10752), (65, 4096, 14336)])
 def test_nvfp4_gemm_split_k_with_workspace(dev, shape):
-    """Fewer 128x128 output tiles than compute units and a deep K where neither the weight-streaming kernel (more than
-    256 rows in too many rounds of workgroups) nor the persistent kernel (N % 256 != 0) runs: with the scratch memory
+    """Fewer 128x128 output tiles than compute units and a deep K where the weight-streaming kernel (more than 256 rows in
+    too many rounds of workgroups) and the persistent kernel behind a cut of N are estimated slower: with the scratch memory
     that nvf_nvfp4_scaled_mm_workspace_bytes asks for, K is split over workgroups of the tile kernel and fp32 partial
     tiles are added in a fixed order.  Ragged N / K (splits that do not divide the spans), both
     output types, against the oracle; run-to-run bit equality; a workspace that is too small, NULL or misaligned falls

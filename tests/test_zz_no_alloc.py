@@ -22,9 +22,9 @@ def test_static_scratch_entry_point_equals_the_workspace_entry_point(dev):
     from fuser_amd import capi
 
     lib = capi.lib()
-    # two split-K shapes of the tile kernel, the second smaller in every dimension (ragged N / K), one of the
+    # two split-K shapes of the tile kernel, the second smaller (fewer rows and columns; ragged N / K), one of the
     # weight-streaming kernel; then the first again
-    for call, (m, n, k) in enumerate([(384, 6176, 10272), (384, 4224, 8224), (80, 6144, 8192), (384, 6176, 10272)]):
+    for call, (m, n, k) in enumerate([(640, 4224, 12320), (512, 3104, 12320), (80, 6144, 8192), (640, 4224, 12320)]):
         gen = torch.Generator().manual_seed(100 + call)
         a, sa, ga = _operand(m, k, 1.0, gen)
         b, sb, gb = _operand(n, k, 0.02, gen)
@@ -61,5 +61,5 @@ def test_static_scratch_entry_point_equals_the_workspace_entry_point(dev):
     torch.cuda.synchronize()
     assert torch.equal(got, want)
     # The largest scratch any split asks for on 256 compute units is the static array (at most 2 x 256 work items of
-    # 128 x 128 fp32); the second shape above comes within 4 % of it (5 splits of 3 x 33 tiles).
-    assert lib.nvf_nvfp4_scaled_mm_workspace_bytes(384, 4224, 8224) > 0.96 * capi.STATIC_SCRATCH_BYTES
+    # 128 x 128 fp32); the first shape above comes within 4 % of it (3 splits of 5 x 33 tiles).
+    assert lib.nvf_nvfp4_scaled_mm_workspace_bytes(640, 4224, 12320) > 0.96 * capi.STATIC_SCRATCH_BYTES
