@@ -828,6 +828,10 @@ int launch_skinny(const Params& p, hipStream_t stream) {
   // 256 x 4096 x 14336: 49.9 -> 26.1 us; 128 x 8192 x 7168: 28.0 -> 16.6 us).
   int slab, rt;
   mxfp8_skinny_best(p.m, p.n, p.k, cu_count(), &slab, &rt);
+  // Decode sizes against weight rows a multiple of 8 KiB apart: 2 weight tiles per workgroup stream them slower than
+  // 1 or 4 do (measured, 8 rows: 8192 x 8192 15.8 us with 2, 14.3 with 1, 12.6 with 4; 7168 x 8192 13.6 / 12.5 / 11.4;
+  // other K: as estimated), so 4 where that still leaves 80 workgroups
+  if (p.m <= 32 && rt == 2 && (p.k & 8191) == 0 && (p.n & 63) == 0 && p.n / 64 >= 80) rt = 4;
   const int slabs = p.m <= slab ? 1 : (int)ceil_div(p.m, slab);
   const int rows = p.m <= slab ? p.m : slab;
   return rows <= 16 ? launch_skinny_rt<1, OUT_BF16>(p, rt, stream, slabs)
