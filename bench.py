@@ -401,6 +401,19 @@ def main():
             wbytes = int((d_sizes > 0).sum()) * n * k * 0.5625
             res[f"decode_512rows_K{k}_N{n}"] = {"us": round(ms_d * 1e3, 1), "active_experts": int((d_sizes > 0).sum()),
                                                 "weight_GB/s": round(wbytes / ms_d / 1e6, 1)}
+            # and with the prefill's skew of the routing (64 tokens x top-8 over Zipf(1.1) loads: a few experts get 33
+            # rows or more)
+            z_sizes = moe_zipf(64, 8, g, 1.1, 0).int()
+            z_pad = (z_sizes + 127) // 128 * 128
+            z_eo = (torch.cumsum(z_sizes, 0) - z_sizes).int().to(dev)
+            z_so = (torch.cumsum(z_pad, 0) - z_pad).int().to(dev)
+            z_q, z_sf = ops.nv_grouped_block_quantize(x[:512].contiguous(), z_eo, z_so, None, 16)
+            z_ps = torch.stack([z_sizes, torch.full_like(z_sizes, n), torch.full_like(z_sizes, k)], 1).int().to(dev)
+            ms_z, _ = timed(lambda: nvf_cutlass.nvfp4_scaled_grouped_mm(z_q, bq4, z_sf, bsf8, alphas, st, ct, z_ps, z_eo, z_so,
+                                                                        torch.bfloat16), 10, 2)
+            zbytes = int((z_sizes > 0).sum()) * n * k * 0.5625
+            res[f"decode_512rows_zipf_K{k}_N{n}"] = {"us": round(ms_z * 1e3, 1), "active_experts": int((z_sizes > 0).sum()),
+                                                     "largest_group": int(z_sizes.max()), "weight_GB/s": round(zbytes / ms_z / 1e6, 1)}
             del bq, bsf, bq4, bsf8, x, aq, asf
         extra["nvfp4_grouped_mm"] = res
 

@@ -58,6 +58,9 @@ struct Params {
   int m_base = 0;
   // grouped skinny kernel: the group sizes it serves; the tile kernel skips groups of fewer than min_rows rows
   int rows_lo = 0, rows_hi = 0, min_rows = 0;
+  // grouped skinny kernel: 0 = one block of workgroups per group (those of other sizes return at once); otherwise the
+  // launch has class_slots blocks and block i looks for the i-th group of rows_lo..rows_hi rows
+  int class_slots = 0;
   int tail_done = 0;  // grouped NVFP4 dispatch: the ends of the large groups have been computed by an earlier launch
   // block-scaled result (nvfp4_scaled_mm_blockscale): out = packed e2m1 [m, n/2], out_sf = e4m3 scales in the 128x4
   // layout of [roundUp(m,128), roundUp(n/16,4)], gnorm = the result's global (encode) scale on the device
@@ -403,10 +406,19 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int6
       else if (p.k < 4096 && (p.n & 255) == 0) rc = launch_nvfp4_skinny_grouped<2, 2, OUT_BF16, true>(p, 1, 32, stream);
       else rc = launch_nvfp4_skinny_grouped<4, 2, OUT_BF16, false>(p, 1, 32, stream);
       if (rc != NVF_OK) return rc;
-      if ((p.k < 4096 || m_hint < kPrefillRows) && (p.n & 255) == 0 && p.k >= 256) {
+      // Below the prefill size the groups of 33..128 rows are few: they stream their weights like the smaller ones,
+      // found by rank among the groups of their size (a launch with few workgroups when there are few rows in all).  A
+      // 128x256 tile of the persistent kernel walks all of K on one compute unit: with 64 or 256 experts, 512..5600
+      // rows and K = 4096..14336 the call is 5-40 % slower that way wherever such groups exist and 0-3 % faster where
+      // none does; with K < 4096 the tiles win from about 2048 rows on.  Kept on the tiles: many groups of near 128
+      // rows against wide weights (64 experts, 5600 rows, N=14336, K=4096: 0.97 against 1.05 ms).
+      const int64_t mid_tiles = std::min<int64_t>(p.groups, m_hint / 33) * (p.n / 256);
+      const bool mid_on_tiles = mid_tiles >= 12 * (int64_t)cus && m_hint >= 80 * (int64_t)p.groups;
+      if (m_hint <= 1024 || (p.k >= 4096 && m_hint < kPrefillRows && !mid_on_tiles)) {
+        rc = launch_nvfp4_skinny_grouped<4, 8, OUT_BF16, false>(p, 33, 128, stream);
+      } else if ((p.k < 4096 || m_hint < kPrefillRows) && (p.n & 255) == 0 && p.k >= 256) {
         // shallow K: one 128x256 tile of the persistent kernel per weight panel converts a group's rows once per 256
-        // weight rows; the streaming kernel whose wavefronts own rows converts them once per wavefront.  Few rows
-        // in all (a decode step): such groups are rare and the persistent kernel costs least when it finds none.
+        // weight rows; the streaming kernel whose wavefronts own rows converts them once per wavefront.
         Params mid = p;
         mid.rows_lo = 33;
         mid.rows_hi = 128;

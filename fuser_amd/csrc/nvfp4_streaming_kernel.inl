@@ -99,8 +99,34 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
   int64_t a_row0 = p.m_base, asf_row0 = p.m_base, b_row0 = 0;  // first activation row, its scale row, first weight row
   if constexpr (GROUPED) {
     const int nblocks = p.n / (16 * RT * (NSPLIT ? W : 1));
-    grp = blockIdx.x / nblocks;
-    n0 = ((blockIdx.x - grp * nblocks) * (NSPLIT ? W : 1) + (NSPLIT ? wave : 0)) * (16 * RT);
+    const int block = blockIdx.x / nblocks;
+    grp = block;
+    if (p.class_slots != 0) {
+      // the block-th group of the size class, in group order: every wavefront counts the groups, 256 at a time (four
+      // loads in flight: a workgroup that finds no group of its own is gone after one round trip to the L2)
+      grp = -1;
+      int before = 0;
+      for (int base = 0; base < p.groups && grp < 0; base += 256) {
+        int mg[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int gi = base + u * 64 + lane;
+          mg[u] = gi < p.groups ? p.problem_sizes[gi * 3] : 0;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          uint64_t in_class = __builtin_amdgcn_ballot_w64(mg[u] >= p.rows_lo && mg[u] <= p.rows_hi);
+          const int count = __builtin_popcountll(in_class);
+          if (grp < 0 && block < before + count) {
+            for (int skip = block - before; skip > 0; --skip) in_class &= in_class - 1;
+            grp = base + u * 64 + __builtin_ctzll(in_class);
+          }
+          before += count;
+        }
+      }
+      if (grp < 0) return;
+    }
+    n0 = ((blockIdx.x - block * nblocks) * (NSPLIT ? W : 1) + (NSPLIT ? wave : 0)) * (16 * RT);
     m_loc = __builtin_amdgcn_readfirstlane(p.problem_sizes[grp * 3]);
     if (m_loc < p.rows_lo || m_loc > p.rows_hi) return;
     a_row0 = __builtin_amdgcn_readfirstlane(p.expert_offsets[grp]);
@@ -693,7 +719,12 @@ int launch_nvfp4_skinny_grouped(const Params& p0, int rows_lo, int rows_hi, hipS
   Params p = p0;
   p.rows_lo = rows_lo;
   p.rows_hi = rows_hi;
-  const int64_t wgs = (int64_t)p.groups * (p.n / (16 * RT * (NSPLIT ? 8 : 1)));
+  // Groups of rows_lo rows or more: at most m / rows_lo of them exist (the groups are disjoint row ranges of the
+  // activations), so the launch has that many blocks of workgroups and each looks its group up.  One block per group
+  // costs a decode step with 256 experts 20-30 us of workgroups that return at once.
+  if (rows_lo > 1) p.class_slots = (int)std::min<int64_t>(p.groups, p.m / rows_lo);
+  if (rows_lo > 1 && p.class_slots == 0) return NVF_OK;  // fewer rows in all than one such group has
+  const int64_t wgs = (int64_t)(p.class_slots ? p.class_slots : p.groups) * (p.n / (16 * RT * (NSPLIT ? 8 : 1)));
   if (wgs >= ((int64_t)1 << 31)) return fail(NVF_ERR_UNSUPPORTED_SHAPE, "too many (group, row block) pairs for one launch");
   if (note_launch("nvfp4_skinny_ring_kernel<RT=%d,TT=%d,grouped,nsplit=%d> grid=%lld rows=%d..%d", RT, TT, (int)NSPLIT, (long long)wgs, rows_lo,
                   rows_hi))

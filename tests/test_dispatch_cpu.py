@@ -143,6 +143,27 @@ def test_config5_nvfp4_grouped(n, k):
     assert "nvfp4_tile_kernel" not in got, got
 
 
+@pytest.mark.parametrize("m,n,k,groups,streams,slots", [
+    (512, 2048, 7168, 256, True, 15),     # a decode step: 64 tokens x top-8 (the benchmark's decode-sized call)
+    (512, 7168, 2048, 256, True, 15),     # few rows in all: also against shallow weights
+    (4096, 2048, 7168, 256, True, 124),   # a short prefill against deep weights
+    (4096, 4096, 14336, 64, True, 64),
+    (4096, 7168, 2048, 256, False, 0),    # shallow weights from 1025 rows on: 128x256 tiles of the persistent kernel
+    (5600, 14336, 4096, 64, False, 0),    # many groups of near 128 rows against wide weights: tiles
+    (2048, 14336, 4096, 64, True, 62),
+])
+def test_nvfp4_grouped_below_the_prefill_size_streams_the_mid_sized_groups(m, n, k, groups, streams, slots):
+    got = plan("nvfp4_scaled_grouped_mm", m, n, k, groups=groups)
+    mid = [g for g in got.split("; ") if "rows=33..128" in g]
+    assert len(mid) == 1, got
+    if streams:
+        # one block of N/64 workgroups per group that can exist with 33 rows or more, not one per expert
+        assert mid[0].startswith("nvfp4_skinny_ring_kernel<RT=4,TT=8,grouped,nsplit=0>") and f"grid={slots * (n // 64)} " in mid[0], got
+    else:
+        assert mid[0].startswith("nvfp4_gemm_256_kernel<grouped=1,TM=2"), got
+    assert "nvfp4_group_panel_kernel" not in got, got
+
+
 def test_dry_run_reports_argument_errors_and_touches_no_device():
     buf = __import__("ctypes").create_string_buffer(64)
     assert capi.lib().nvf_describe_dispatch(b"mxfp8_scaled_mm", 128, 128, 40, 1, BF16, 0, buf, 64) == -2

@@ -392,6 +392,60 @@ def test_nvfp4_grouped_mm_mid_sized_groups_of_a_prefill(dev, n, k):
         assert torch.equal(out[:rows], nvf_cutlass.nvfp4_scaled_grouped_mm(*args, dtype)[:rows])
 
 
+@pytest.mark.parametrize("n,k,few_rows", [(256, 4096, False), (128, 4224, False), (256, 512, False), (256, 512, True), (128, 4096, True)])
+def test_nvfp4_grouped_mm_mid_sized_groups_below_the_prefill_size(dev, n, k, few_rows):
+    """300 experts, most of them with 0..3 rows, a few with 33..128 at indices on both sides of the borders at which
+    the streaming kernel counts the groups of a size class (63 | 64, 255 | 256, the last one), two large ones.  Up to
+    1024 rows in all, or below 6144 with K >= 4096, the mid-sized groups stream their weights from a launch with one
+    block of workgroups per group of 33 rows that the call could hold (the block finds its group by rank); otherwise
+    they run as 128x256 tiles of the persistent kernel.  A different alpha per group, poisoned padding of the activation
+    scale slabs; every element compared, rows after the last group untouched, run-to-run bit equality."""
+    from fuser_amd import capi, nvf_cutlass
+
+    g = 300
+    if few_rows:
+        sizes = [1 if i % 5 == 0 else 0 for i in range(g)]
+        for i, t in {63: 33, 64: 128, 256: 40, 299: 100, 130: 129}.items():
+            sizes[i] = t
+    else:
+        sizes = [i % 4 for i in range(g)]
+        for i, t in {2: 33, 63: 128, 64: 100, 70: 64, 255: 90, 256: 77, 257: 128, 299: 40, 130: 400, 131: 129}.items():
+            sizes[i] = t
+    m = sum(sizes) + 3
+    assert (m <= 1024) == few_rows and m < 6144
+    got = capi.describe_dispatch("nvfp4_scaled_grouped_mm", m, n, k, groups=g)
+    mid = [part for part in got.split("; ") if "rows=33..128" in part]
+    assert len(mid) == 1 and mid[0].startswith("nvfp4_skinny_ring_kernel<" if few_rows or k >= 4096 else "nvfp4_gemm_256_kernel<grouped=1,TM=2"), got
+    gen = torch.Generator().manual_seed(n + k + few_rows)
+    x = torch.randn(m, k, generator=gen).bfloat16()
+    w = (torch.randn(8, n, k, generator=gen) * 0.05).bfloat16()  # eight different experts, repeated
+    ps, eo, st, ct = _grouped_args(sizes, n, k, dev)
+    so = start_offsets([O.round_up(t, 128) for t in sizes])
+    aq, valid = O.grouped_block_quantize_nvfp4(x, eo, so, None)
+    lin = torch.zeros_like(valid, dtype=torch.bool)
+    for e, t in enumerate(sizes):
+        if t:
+            ones = O.linear_to_swizzled_128_4(torch.ones(t, k // 16, dtype=torch.uint8))
+            lin[int(so[e]) : int(so[e]) + ones.shape[0]] |= ones.bool()
+    asf = torch.where(lin, valid, torch.full_like(valid, 0x7F))  # NaN code wherever no row owns the byte
+    bq = torch.empty(g, n, k // 2, dtype=torch.uint8)
+    bsf = torch.empty(g, n, k // 16, dtype=torch.uint8)
+    alphas = torch.empty(g)
+    quantized = [O.block_quantize_nvfp4(w[e], gs_of(w[e]), True) for e in range(8)]
+    for e in range(g):
+        bq[e], bsf[e] = quantized[e % 8]
+        alphas[e] = (e % 11 + 1) / gs_of(w[e % 8])
+    ref = O.ref_nvfp4_scaled_grouped_mm(aq, bq, valid, bsf, alphas, ps, eo, so)
+    rows = sum(sizes)
+    args = (fp4(aq.to(dev)), fp4(bq.to(dev)), e4m3(asf.to(dev)), e4m3(bsf.to(dev)), alphas.to(dev), st, ct, ps.to(dev), eo.to(dev), so.to(dev))
+    for dtype in (torch.bfloat16, torch.float16):
+        out = nvf_cutlass.nvfp4_scaled_grouped_mm(*args, dtype)
+        torch.cuda.synchronize()
+        scale = ref[:rows].abs().amax(dim=1, keepdim=True).clamp(min=1e-30)
+        assert ((out[:rows].float().cpu() - ref[:rows]).abs() / scale).max().item() <= GEMM_MAX_REL, (n, k, dtype)
+        assert torch.equal(out[:rows], nvf_cutlass.nvfp4_scaled_grouped_mm(*args, dtype)[:rows])
+
+
 def _zipf_sizes(tokens, topk, experts, s, seed):
     gen = torch.Generator().manual_seed(seed)
     p = 1.0 / torch.arange(1, experts + 1).float() ** s
