@@ -55,8 +55,14 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
   static_assert(GROUPED || !NSPLIT, "the dense op has too few row blocks to give every wavefront its own");
   constexpr int W = 8;
   constexpr int NT = RT + TT;
-  constexpr int B_SC = (RT + 1) / 2, A_SC = (TT + 1) / 2;     // scale blocks (1 KiB) per operand
-  constexpr int SLOT_BYTES = (NT + B_SC + A_SC) * 1024;
+  // Scale blocks (1 KiB) per operand and chunk: one.  A block holds, for a pair of 16-row tiles, the 16-byte pieces of
+  // the 128x4 layout with the scale words of rows {row, row+32, row+64, row+96}: the pairs of an operand (rows 32 apart)
+  // find their words in the same pieces, so the block of the first pair serves them all.
+  constexpr int B_SC = 1, A_SC = 1;
+  // (two places for the activations' block where a chunk's tiles are read one by one while the next chunk's loads are
+  // already under way: the chunks of a wavefront alternate between them)
+  constexpr int A_SC_PLACES = TT > 2 ? 2 : 1;
+  constexpr int SLOT_BYTES = (NT + B_SC + A_SC_PLACES) * 1024;
   constexpr int NDMA = NT + B_SC + A_SC;                      // loads per chunk and wavefront
   // DEPTH 2: two chunks in flight per wavefront.  DEPTH 1 (many tiles per chunk): the next chunk is requested
   // as soon as the current one has been read out of LDS, and lands under its long conversion + MFMA phase.
@@ -211,11 +217,11 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
     const int rowgroup = (((n0 & 127) + rt * 16) >> 5) & 3;  // which of the 4 words of the 16 bytes
-    rd_bsc[rt] = (NT + (rt >> 1)) * 1024 + ((rt & 1) * 2 + (g >> 1)) * 256 + r * 16 + rowgroup * 4;
+    rd_bsc[rt] = NT * 1024 + ((rt & 1) * 2 + (g >> 1)) * 256 + r * 16 + rowgroup * 4;
   }
 #pragma unroll
   for (int tt = 0; tt < TT; ++tt)
-    rd_asc[tt] = (NT + B_SC + (tt >> 1)) * 1024 + ((tt & 1) * 2 + (g >> 1)) * 256 + r * 16 + (asf_word0 + ((tt * 16) >> 5)) * 4;
+    rd_asc[tt] = (NT + B_SC) * 1024 + ((tt & 1) * 2 + (g >> 1)) * 256 + r * 16 + (asf_word0 + ((tt * 16) >> 5)) * 4;
   const int sc_shift = (g & 1) * 16;
 
   const float alpha = p.alpha[grp];
@@ -312,15 +318,15 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
       lds_dma16(ring_base + (RT + tt) * 1024, a_base,
                 (uint32_t)min(tt * 16 + fine_lrow, m_loc - 1) * (uint32_t)kbytes + lpiece * 16 - ld_sub + c * 64u);
     };
-    auto load_a_scales = [&](uint32_t c, int j) {
+    auto load_a_scales = [&](uint32_t c, uint32_t place = 0) {
       uint32_t ld_sub, sc_sub = 0;
       if (is_tail((int)c)) tail_subs(ld_sub, sc_sub);
-      lds_dma16(ring_base + (NT + B_SC + j) * 1024, asf_base, asf_off[j] - sc_sub + c * 1024u);
+      lds_dma16(ring_base + (NT + B_SC) * 1024 + place * 1024u, asf_base, asf_off[0] - sc_sub + c * 1024u);
     };
     const char* sp = reinterpret_cast<const char*>(red) + wave * SLOT_BYTES;
-    auto read_a_tile = [&](uint32_t c, int tt, u32x4& aq, uint32_t& as) {
+    auto read_a_tile = [&](uint32_t c, int tt, u32x4& aq, uint32_t& as, uint32_t place = 0) {
       aq = *reinterpret_cast<const u32x4*>(sp + (RT + tt) * 1024 + rd_payload);
-      as = *reinterpret_cast<const uint32_t*>(sp + rd_asc[tt]) >> sc_shift;
+      as = *reinterpret_cast<const uint32_t*>(sp + rd_asc[tt] + place * 1024u) >> sc_shift;
       if (is_tail((int)c)) as &= tail_keep();
     };
     // e4m3 scales of a lane's two blocks -> fp16 pairs; one dword (8 values of one block) -> one MFMA operand
@@ -363,7 +369,7 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
 #pragma unroll
         for (int tt = 0; tt < TTC; ++tt) {
           load_a_tile(c + CSTEP, tt);
-          if ((tt & 1) || tt + 1 == TTC) load_a_scales(c + CSTEP, tt >> 1);
+          if (tt == (TTC > 1 ? 1 : 0)) load_a_scales(c + CSTEP);
         }
       }
       f16x2 sv[RT][2], asv[TTC][2];
@@ -435,7 +441,7 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
 #pragma unroll
             for (int t2 = 0; t2 < TTC; ++t2) {
               load_a_tile(c + CSTEP, t2);
-              if ((t2 & 1) || t2 + 1 == TTC) load_a_scales(c + CSTEP, t2 >> 1);
+              if (t2 == (TTC > 1 ? 1 : 0)) load_a_scales(c + CSTEP);
             }
           }
         }
@@ -483,12 +489,14 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
     // counts that follow from it.
     auto chunk_pipe = [&](auto ttc_c, uint32_t c, auto& acc) {
       constexpr int TTC = decltype(ttc_c)::value;
-      constexpr int NS = (TTC + 1) / 2, NA = TTC + NS, LB = RT + B_SC;
+      constexpr int NA = TTC + A_SC, LB = RT + B_SC;
       const bool has_next = c + CSTEP < (uint32_t)chunks;
+      // this chunk's block of activation scales: tiles 2.. read their words from it after the next chunk's block has
+      // been requested, which therefore goes to the other place
+      const uint32_t place = ((c - (uint32_t)c_first) / CSTEP) & 1u;
       // loads of this chunk still pending once tile tt and the scale block of its pair have landed
-      auto after_tile = [&](int tt) {
-        const int last_of_pair = (tt | 1) < TTC ? (tt | 1) : TTC - 1;
-        return NA - 1 - (last_of_pair + (last_of_pair >> 1) + 1);
+      auto after_tile = [&](int tt) {  // (the scale block follows tile 1, or tile 0 if that is the only one)
+        return NA - (tt <= 1 ? (TTC > 1 ? 3 : 2) : tt + 2);
       };
       wait_loads(NA);  // the weight part has landed
       u32x4 q[RT];
@@ -505,12 +513,12 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
       wait_loads(after_tile(0));
       u32x4 aq, aqn = {0, 0, 0, 0};
       uint32_t as, asn = 0;
-      read_a_tile(c, 0, aq, as);
+      read_a_tile(c, 0, aq, as, place);
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // read out: may be refilled
       if (has_next) {
         load_b_part(c + CSTEP);
         load_a_tile(c + CSTEP, 0);
-        if (TTC == 1) load_a_scales(c + CSTEP, 0);
+        if (TTC == 1) load_a_scales(c + CSTEP, place ^ 1u);
       }
       u32x4 fb[RT][4];
 #pragma unroll
@@ -530,8 +538,8 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
         __builtin_amdgcn_sched_barrier(0);
         if (tt + 1 < TTC) {
           // pending behind tile tt+1: the rest of this chunk's tiles, the next chunk's weight part and its tiles 0..tt
-          wait_loads(after_tile(tt + 1) + (has_next ? LB + (tt + 1) + ((tt + 1) >> 1) : 0));
-          read_a_tile(c, tt + 1, aqn, asn);
+          wait_loads(after_tile(tt + 1) + (has_next ? LB + (tt + 1) + (tt >= 1 ? 1 : 0) : 0));
+          read_a_tile(c, tt + 1, aqn, asn, place);
         }
         // K steps 0 and 1 of tile tt; behind every MFMA one dword of the operands of its steps 2 and 3
 #pragma unroll
@@ -548,7 +556,7 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
           asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // tile tt+1 is in registers: its slot may be refilled
           if (has_next) {
             load_a_tile(c + CSTEP, tt + 1);
-            if (((tt + 1) & 1) || tt + 2 == TTC) load_a_scales(c + CSTEP, (tt + 1) >> 1);
+            if (tt == 0) load_a_scales(c + CSTEP, place ^ 1u);
           }
           scale_pairs(asn, asvn);
         }
@@ -580,7 +588,7 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
 #pragma unroll
         for (int tt = 0; tt < TTC; ++tt) {
           load_a_tile((uint32_t)c_first, tt);
-          if ((tt & 1) || tt + 1 == TTC) load_a_scales((uint32_t)c_first, tt >> 1);
+          if (tt == (TTC > 1 ? 1 : 0)) load_a_scales((uint32_t)c_first);
         }
       }
       for (int c = c_first; c < chunks; c += CSTEP) {
