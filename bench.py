@@ -55,7 +55,7 @@ def main():
 
     import torch
 
-    from fuser_amd import nvf_cutlass, ops
+    from fuser_amd import capi, nvf_cutlass, ops
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = "cuda:0"
@@ -242,7 +242,7 @@ def main():
         ar, sar = a[:mr].contiguous(), sa[: 8192].contiguous()
         ms_r, _ = timed(lambda: nvf_cutlass.nvfp4_scaled_mm(ar, b, sar, sb, alpha, torch.bfloat16), 20, 3)
         extra["nvfp4_gemm_8100x8192x8192"] = {"ms": round(ms_r, 4), "TFLOP/s": round(2.0 * mr * n * k / ms_r / 1e9, 1),
-                                              "note": "M not a multiple of 128: two launches (7936 rows on 256x256 tiles, 164 rows streamed)"}
+                                              "launches": capi.describe_dispatch("nvfp4_scaled_mm", mr, n, k)}
         gn = torch.ones((), device=dev)
         ms_b, _ = timed(lambda: nvf_cutlass.nvfp4_scaled_mm_blockscale(a, b, sa, sb, alpha, gn), 20, 3)
         extra["nvfp4_gemm_blockscale_8192"] = {"ms": round(ms_b, 4), "TFLOP/s": round(2.0 * m * n * k / ms_b / 1e9, 1),
@@ -505,12 +505,12 @@ def main():
             vendor["hipblaslt_fp8_per_tensor_scale_TFLOP/s"] = None
             vendor["hipblaslt_fp8_error"] = str(exc)[:120]
         extra["vendor_library_8192"] = vendor
-        # a prefill of a token count that is no multiple of 128: rows up to the cut on the persistent kernel, the rest streamed
+        # a prefill of a token count that is no multiple of 128: one launch of 256x256 tiles, the last row tile with 164 rows
         mr = 8100
         qar = qa[:mr].contiguous()
         r_ms, _ = timed(lambda: nvf_cutlass.mxfp8_scaled_mm(qar, qb, sa, sb, one, torch.bfloat16), args.steps, args.warmup)
         extra["mxfp8_gemm_8100x8192x8192"] = {"ms": round(r_ms, 4), "TFLOP/s": round(2.0 * mr * n * k / r_ms / 1e9, 1),
-                                              "note": "M not a multiple of 128: two launches (7936 rows on 256x256 tiles, 164 rows streamed)"}
+                                              "launches": capi.describe_dispatch("mxfp8_scaled_mm", mr, n, k)}
 
     if not args.no_extra:
         for name in ("quant", "fused", "nvfp4", "llm", "grouped", "gnvfp4"):

@@ -239,8 +239,9 @@ __device__ __forceinline__ void lds_dma16(uint32_t lds_byte_addr, const uint8_t*
 // lanes whose 16 bytes lie past the end of the row write zeros to their LDS unit instead of loading (the bytes there
 // belong to the next row), and the scale bytes of the blocks past K - padding columns of the scale layout, whose content
 // is not defined - are replaced by 2^0, so that the step adds exact zeros.
-template <int TM, bool OUT_BF16, bool STREAM_OUT, bool RAGGED_K = false>
+template <int TM, bool OUT_BF16, bool STREAM_OUT, bool RAGGED_K = false, bool RAGGED_M = false>
 __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) {
+  static_assert(!(RAGGED_K && RAGGED_M), "one variant per kind of raggedness");
   constexpr int BM = 64 * TM, BN = 256;
   constexpr int A_UNITS = BM * 8;             // 16-byte units of the A tile (BM rows x 8 chunks)
   constexpr int TILE_UNITS = 2048;            // ... of the B tile
@@ -260,7 +261,10 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
   // contiguous tile range [x*chunk, (x+1)*chunk) and its workgroups take consecutive tiles of it in
   // each round: with the 8 (m) x 4 (n) blocked tile numbering below, the 32 tiles an XCD works on at
   // any time share 8 A panels and 4 B panels in that XCD's L2.
-  const int tiles_m = p.m / BM, tiles_n = p.n / BN;
+  // RAGGED_M: the last row tile holds fewer than BM rows (a kernel of its own: clamping the row of every activation
+  // load costs the others time).  Its missing rows load the last row again and are not stored; the scale layout is
+  // padded to 128 rows, so only a 256-row tile can ask for a scale tile that does not exist (it takes the last one).
+  const int tiles_m = RAGGED_M ? (p.m + BM - 1) / BM : p.m / BM, tiles_n = p.n / BN;
   const int total = tiles_m * tiles_n;
   const int chunk_tiles = (total + 7) >> 3;
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, slots = gridDim.x >> 3;
@@ -310,16 +314,20 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
   // ahead of the compute loop and crosses into the next tile two steps early.  All of its state is
   // wave-uniform and it advances without branches (the next tile's base pointers are prepared at the
   // top of the tile loop), so that the hot loop stays one basic block.
-  struct TilePtrs { const uint8_t *a, *b, *sa, *sb; };
+  struct TilePtrs { const uint8_t *a, *b, *sa, *sb; int valid; };
   auto tile_ptrs = [&](int t) {
     int m0, n0;
     tile_coords(t, m0, n0);
     TilePtrs r;
-    r.a = p.a + ((int64_t)m0 + wave * (BM / 4)) * p.k;
+    // (RAGGED_M: the tile's first row; the wavefront's share is part of the lane's clamped row)
+    r.a = p.a + ((int64_t)m0 + (RAGGED_M ? 0 : wave * (BM / 4))) * p.k;
     r.b = p.b + ((int64_t)n0 + wave * 64) * p.k;
+    r.valid = p.m - m0;  // rows of the tile that exist (RAGGED_M: possibly fewer than BM)
     // one 16-byte scale load per lane per K step: rows {li, li+32, li+64, li+96} of the wave's 128-row
     // scale tile x 4 K-blocks
-    r.sa = p.sfa + ((int64_t)((m0 >> 7) + (TM == 4 ? wm : 0)) * sf_tiles_k) * 512;
+    int sa_tile = (m0 >> 7) + (TM == 4 ? wm : 0);
+    if (RAGGED_M) sa_tile = min(sa_tile, ((p.m + 127) >> 7) - 1);
+    r.sa = p.sfa + ((int64_t)sa_tile * sf_tiles_k) * 512;
     r.sb = p.sfb + ((int64_t)((n0 >> 7) + wn) * sf_tiles_k) * 512;
     return r;
   };
@@ -342,6 +350,11 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
       else *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(lds) + (l - lds_base) + lane * 16) = u32x4{0, 0, 0, 0};
       return;
     }
+    if (RAGGED_M && op == 0) {
+      const uint32_t row = min((uint32_t)(wave * (BM / 4) + j * 8) + (uint32_t)(lane >> 3), (uint32_t)(lp.valid - 1));
+      lds_dma16(l, gp, row * (uint32_t)p.k + (((j & 1) ? voff_odd : voff_even) - row_off));
+      return;
+    }
     lds_dma16(l, gp, ((j & 1) ? voff_odd : voff_even) + (uint32_t)j * step8);
   };
   // After the 16 units: the step's scale loads, then advance the stream (selects only).
@@ -355,6 +368,7 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
     lp.b = wrap ? np.b : lp.b;
     lp.sa = wrap ? np.sa : lp.sa;
     lp.sb = wrap ? np.sb : lp.sb;
+    if (RAGGED_M) lp.valid = wrap ? np.valid : lp.valid;
   };
   // Fragment storage: [operand: 0 = A, 1 = B][sub-tile][half].  Unit q (0..NF-1) of a half step is one
   // ds_read_b128: the 2*TM units of A (sub-tile q/2, half q&1), then the 8 units of B.
@@ -497,6 +511,7 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
     const int ldc = p.out_pitch();
     const uint32_t ooff = ((uint32_t)(elane >> 3) * (uint32_t)ldc + (uint32_t)(elane & 7) * 8u) * 2u;
     uint8_t* obase = reinterpret_cast<uint8_t*>(static_cast<uint16_t*>(p.out) + (int64_t)(m0 + wm * (32 * TM)) * ldc + n0 + wn * 128);
+    const int rows_left = p.m - m0 - wm * (32 * TM) - (elane >> 3);  // RAGGED_M: rows from this lane's first one to the end
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
@@ -517,6 +532,7 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
         for (int t = 0; t < 4; ++t) {
           const u32x4 v = *reinterpret_cast<const u32x4*>(rd + t * 1152);
           u32x4* dst = reinterpret_cast<u32x4*>(obase + ((int64_t)(i * 32 + 8 * t) * ldc + jh * 64) * 2 + ooff);
+          if (RAGGED_M && i * 32 + 8 * t >= rows_left) continue;
           if constexpr (STREAM_OUT) __builtin_nontemporal_store(v, dst);
           else *dst = v;
         }
@@ -529,15 +545,18 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
 #undef NVF_PIN_ACC
 }
 
-template <int TM, bool OUT_BF16, bool STREAM_OUT, bool RAGGED_K>
+template <int TM, bool OUT_BF16, bool STREAM_OUT, bool RAGGED_K, bool RAGGED_M = false>
 int launch_fast_cfg(const Params& p, hipStream_t stream) {
-  auto kern = mxfp8_gemm_256_kernel<TM, OUT_BF16, STREAM_OUT, RAGGED_K>;
+  auto kern = mxfp8_gemm_256_kernel<TM, OUT_BF16, STREAM_OUT, RAGGED_K, RAGGED_M>;
   constexpr int lds_bytes = 2 * (64 * TM + 256) * 128 + 4 * 4608;  // 128 KiB / 96 KiB of tiles + the epilogue's 18 KiB
-  const int64_t tiles = (int64_t)(p.m / (64 * TM)) * (p.n / 256);
+  const int64_t tiles = ceil_div(p.m, 64 * TM) * (p.n / 256);
+  if (!RAGGED_M && p.m % (64 * TM) != 0) return fail(NVF_ERR_LAUNCH, "mxfp8_gemm_256_kernel: M = %d is no multiple of %d", p.m, 64 * TM);
   const int cus = cu_count() & ~7;  // workgroup ids are dealt round-robin to the 8 XCDs
   const unsigned grid = (unsigned)(tiles >= cus ? cus : ((tiles + 7) / 8) * 8);
-  if (note_launch("mxfp8_gemm_256_kernel<TM=%d,stream_out=%d%s> grid=%u", TM, (int)STREAM_OUT, RAGGED_K ? ",ragged_k" : "", grid)) return NVF_OK;
-  static std::atomic<uint64_t> configured{0};  // one bit per device
+  if (note_launch("mxfp8_gemm_256_kernel<TM=%d,stream_out=%d%s%s> grid=%u", TM, (int)STREAM_OUT, RAGGED_K ? ",ragged_k" : "",
+                  RAGGED_M ? ",ragged_m" : "", grid))
+    return NVF_OK;
+  static std::atomic<uint64_t> configured{0};  // one bit per device (and per instantiation of this launcher)
   if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_bytes, stream, p);
   return check_launch("mxfp8_gemm_256_kernel");
@@ -549,6 +568,7 @@ int launch_fast(const Params& p, hipStream_t stream) {
   // operand panels out of it (and out of the L2s) on its way to memory, so it leaves with non-temporal stores
   // (8192^3: +5 %, 16384 x 16384 x 2048: +17 %; smaller problems lose 1-5 % that way).
   const bool stream_out = ((int64_t)p.m + p.n) * p.k + 2 * (int64_t)p.m * p.n > (int64_t)224 << 20;
+  if (p.m % (64 * TM) != 0) return stream_out ? launch_fast_cfg<TM, OUT_BF16, true, false, true>(p, stream) : launch_fast_cfg<TM, OUT_BF16, false, false, true>(p, stream);
   if ((p.k & 127) != 0) return stream_out ? launch_fast_cfg<TM, OUT_BF16, true, true>(p, stream) : launch_fast_cfg<TM, OUT_BF16, false, true>(p, stream);
   return stream_out ? launch_fast_cfg<TM, OUT_BF16, true, false>(p, stream) : launch_fast_cfg<TM, OUT_BF16, false, false>(p, stream);
 }
@@ -861,8 +881,12 @@ Plan mxfp8_plan(int64_t m, int64_t n, int64_t k, int64_t cus, int64_t* ns = null
   if (ns) *ns = INT64_MAX;
   const bool skinny_ok = (k & 31) == 0 && (n & 15) == 0 && k * 64 < (1ll << 31);  // 32-bit lane offsets (a short last chunk is fine)
   // (the persistent kernel takes any K % 32 == 0: its last step may be short)
-  const bool fast_ok = (k & 31) == 0 && k >= 256 && (m & 127) == 0 && (n & 255) == 0 && k * 256 < (1ll << 31);
-  const int64_t t256 = fast_ok && (m & 255) == 0 ? (m / 256) * (n / 256) : 0, t128 = fast_ok ? (m / 128) * (n / 256) : 0;
+  // (a last row tile with fewer rows: the variant that clamps the rows of its activation loads, K % 128 == 0 only;
+  // the tile counts as a whole one.  640 x 14336 x 4096: 280 tiles of 128 rows in 2 rounds 60 us, 168 of 256 rows 43 us)
+  const bool fast_shape = (k & 31) == 0 && k >= 256 && (n & 255) == 0 && k * 256 < (1ll << 31);
+  const bool ok256 = fast_shape && ((m & 255) == 0 || ((k & 127) == 0 && m > 256));
+  const bool ok128 = fast_shape && ((m & 127) == 0 || ((k & 127) == 0 && m > 64));
+  const int64_t t256 = ok256 ? ceil_div(m, 256) * (n / 256) : 0, t128 = ok128 ? ceil_div(m, 128) * (n / 256) : 0;
   const int64_t cost256 = t256 >= 128 ? 100 * ceil_div(t256, cus) : INT64_MAX;
   const int64_t cost128 = t128 >= 48 ? 61 * ceil_div(t128, cus) : INT64_MAX;
   const bool fast = cost256 != INT64_MAX || cost128 != INT64_MAX;

@@ -99,8 +99,8 @@ def test_nvfp4_mid_sized_shapes(m, n, k, kernel):
     assert plan("nvfp4_scaled_mm", m, n, k).startswith(kernel), plan("nvfp4_scaled_mm", m, n, k)
 
 
-@pytest.mark.parametrize("op", ["nvfp4_scaled_mm", "mxfp8_scaled_mm"])
-def test_dense_m_not_a_multiple_of_128_is_cut_into_a_main_part_and_a_remainder(op):
+def test_nvfp4_dense_m_not_a_multiple_of_128_is_cut_into_a_main_part_and_a_remainder():
+    op = "nvfp4_scaled_mm"
     # a prefill of any token count: the rows up to a multiple of 128 / 256 on the persistent kernel, the rest streamed
     got = plan(op, 4000, 4096, 4096).split("; ")
     assert len(got) == 2 and "gemm_256_kernel<" in got[0] and "TM=4" in got[0] and "skinny" in got[1], got
@@ -111,6 +111,22 @@ def test_dense_m_not_a_multiple_of_128_is_cut_into_a_main_part_and_a_remainder(o
     assert len(got) == 1 and "skinny" in got[0], got
     # multiples of 128 and small shapes: as before
     assert "; " not in plan(op, 4096, 4096, 4096) and "; " not in plan(op, 300, 4096, 4096)
+
+
+def test_mxfp8_dense_m_not_a_multiple_of_the_tile_height_takes_the_persistent_kernel_with_a_short_last_row_tile():
+    op = "mxfp8_scaled_mm"
+    # a prefill of any token count: one launch, the last row tile with fewer rows
+    for m, n, k, tm, grid in ((4000, 4096, 4096, 4, 256), (8100, 8192, 8192, 4, 256), (320, 14336, 4096, 2, 168), (640, 14336, 4096, 4, 168),
+                              (96, 28672, 4096, 2, 112), (384, 28672, 4096, 4, 224)):
+        got = plan(op, m, n, k)
+        assert got.startswith(f"mxfp8_gemm_256_kernel<TM={tm},") and "ragged_m" in got and f"grid={grid}" in got and ";" not in got, (m, n, k, got)
+    # where the weight-streaming kernel is estimated faster it takes all rows, and multiples of the tile height are as before
+    got = plan(op, 1000, 4096, 14336)
+    assert "skinny" in got and ";" not in got, got
+    assert "ragged_m" not in plan(op, 4096, 4096, 4096) and "skinny" in plan(op, 300, 4096, 4096)
+    # K % 128 != 0 has its own variant of the kernel: such a shape is still cut at a multiple of 128 rows
+    got = plan(op, 4000, 4096, 2880).split("; ")
+    assert len(got) == 2 and "ragged_k" in got[0] and "skinny" in got[1], got
 
 
 @pytest.mark.parametrize("op", ["nvfp4_scaled_mm", "mxfp8_scaled_mm"])

@@ -756,6 +756,47 @@ def test_mxfp8_gemm_persistent_256_tile_kernel_full_compare(dev, shape):
     assert torch.equal(out, out2)
 
 
+@pytest.mark.parametrize("shape", [(300, 14336, 512), (136, 12288, 512), (80, 28672, 256), (520, 14336, 512), (640, 14336, 1024),
+                                   (700, 12288, 256), (2049, 4096, 512), (390, 8192, 1280)])
+def test_mxfp8_gemm_last_row_tile_with_fewer_rows_on_the_persistent_kernel(dev, shape):
+    """M no multiple of the tile height, N % 256 == K % 128 == 0 and enough tiles: the persistent kernel's variant whose
+    last row tile clamps the rows of its activation loads and stores only the rows that exist.  128-row tiles with 44,
+    8 and 80 rows in the last one (one tile row in all for the 80), 256-row tiles with 8 rows (the tile's second scale
+    tile does not exist: the last one is read instead), 128 (M % 256 == 128), 188 and 1 row; two to ten K steps.  NaN
+    code in every scale byte of the padding rows, both output types, every element compared, rows are written once
+    (a result buffer pre-filled with a pattern keeps it past row M), run-to-run determinism."""
+    from fuser_amd import capi
+
+    m, n, k = shape
+    plan = capi.describe_dispatch("mxfp8_scaled_mm", m, n, k)
+    assert plan.startswith("mxfp8_gemm_256_kernel<") and "ragged_m" in plan and ";" not in plan, plan
+    gen = torch.Generator().manual_seed(m * 31 + n)
+    a, sa = _mxfp8_operand(m, k, gen, 1.0)
+    b, sb = _mxfp8_operand(n, k, gen, 1.0)
+    ref = O.ref_mxfp8_scaled_mm(a, b, sa, sb, 0.75)
+    sa_p = sa.clone()
+    sa_p[O.linear_to_swizzled_128_4(torch.ones(m, k // 32, dtype=torch.uint8)) == 0] = 0xFF
+    scale = ref.abs().amax(dim=1, keepdim=True).clamp(min=1e-30)
+    for dtype in (torch.bfloat16, torch.float16):
+        if dtype == torch.float16 and ref.abs().max() > 6e4:
+            continue
+        out = _run_mxfp8(a, b, sa_p, sb, 0.75, dtype, dev)
+        assert out.shape == (m, n)
+        assert ((out.float().cpu() - ref).abs() / scale).max().item() <= GEMM_MAX_REL, (shape, dtype)
+        assert torch.equal(out, _run_mxfp8(a, b, sa_p, sb, 0.75, dtype, dev))
+    # through the C ABI into the first M rows of a larger buffer: the rows after them keep their contents
+    from fuser_amd import capi as C
+    buf = torch.full((m + 130, n), 7.0, dtype=torch.bfloat16, device=dev)
+    ad, bd = a.to(dev), b.to(dev)
+    sad, sbd = sa_p.to(dev), sb.to(dev)
+    alpha = torch.tensor(0.75, dtype=torch.float32, device=dev)
+    C.check(C.lib().nvf_mxfp8_scaled_mm(ad.data_ptr(), bd.data_ptr(), sad.data_ptr(), sbd.data_ptr(), alpha.data_ptr(), buf.data_ptr(),
+                                        m, n, k, C.BF16, None))
+    torch.cuda.synchronize()
+    assert ((buf[:m].float().cpu() - ref).abs() / scale).max().item() <= GEMM_MAX_REL
+    assert bool((buf[m:] == 7.0).all())
+
+
 def test_mxfp8_gemm_8192_cubed_sampled_against_oracle(dev):
     """BASELINE config 2 at full size.  The CPU oracle is applied to a sample of output rows/columns;
     determinism and the K-split additivity property are checked on the whole output."""
