@@ -181,10 +181,14 @@ struct DensePlan {
 };
 DensePlan nvfp4_dense_plan(int64_t m, int64_t n, int64_t k, int cus) {
   const bool stream_ok = (k & 31) == 0 && (n & 15) == 0 && k * 64 < (1ll << 31);  // 32-bit lane offsets (a short last chunk is fine)
-  const bool persistent_ok = (m & 127) == 0 && (n & 255) == 0 && (k & 31) == 0 && k >= 256;  // (a short last span is fine)
+  // (a short last span is fine; so is, with whole spans, a last row tile with fewer rows, which counts as a whole one:
+  // 384 x 28672 x 4096 as 224 tiles of 256 rows in one round instead of 336 of 128 rows in two)
+  const bool persistent_shape = (n & 255) == 0 && (k & 31) == 0 && k >= 256;
+  const bool ok256 = persistent_shape && ((m & 255) == 0 || ((k & 127) == 0 && m > 256));
+  const bool persistent_ok = persistent_shape && ((m & 127) == 0 || ((k & 127) == 0 && m > 128));
   int64_t cost256 = INT64_MAX, cost128 = INT64_MAX, cost_tile = INT64_MAX;
   if (persistent_ok) {
-    const int64_t t256 = (m & 255) == 0 ? (m / 256) * (n / 256) : 0, t128 = (m / 128) * (n / 256);
+    const int64_t t256 = ok256 ? ceil_div(m, 256) * (n / 256) : 0, t128 = ceil_div(m, 128) * (n / 256);
     cost256 = t256 ? 100 * ceil_div(t256, cus) : INT64_MAX;
     cost128 = 58 * ceil_div(t128, cus);
     const int64_t small = 2 * t128, full = small / (2 * cus), rest = small - full * 2 * cus;

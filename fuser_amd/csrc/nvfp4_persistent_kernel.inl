@@ -31,9 +31,15 @@
 // RAGGED_K (16-bit result; grouped: the 256x256 tiles): K % 128 = 32, 64 or 96.  A tile's last span is short: the threads whose 32 elements lie
 // past K fetch their row's first piece instead of the next row's bytes, and their scale load runs past the range of its
 // buffer resource on purpose, which makes it return zero - and a zero scale makes a block count as zero.
-template <bool OUT_BF16, bool GROUPED, int TM = 4, bool OUT_F32 = false, bool PAIRS = false, bool OUT_FP4 = false, bool RAGGED_K = false>
+// RAGGED_M (dense, 16-bit result): the last row tile holds fewer than BM rows.  As for the last tile of a group, the
+// buffer range of the activations ends with the last row, so the rows past it read as zero, and they are not stored;
+// the scale tile of a 256-row tile's second half may not exist and then reads as zero the same way.
+template <bool OUT_BF16, bool GROUPED, int TM = 4, bool OUT_F32 = false, bool PAIRS = false, bool OUT_FP4 = false, bool RAGGED_K = false,
+          bool RAGGED_M = false>
 __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   static_assert(TM == 4 || TM == 2, "tile height");
+  static_assert(!RAGGED_M || (!GROUPED && !OUT_F32 && !OUT_FP4), "a short last row tile: dense calls with a 16-bit result");
+  constexpr bool PARTIAL = GROUPED || RAGGED_M;  // tiles may hold fewer rows than BM
   constexpr int BM = 64 * TM, BN = 256;
   constexpr int A_UNITS = BM * 8;            // 16-byte units of the A tile (fp16, 64 of K per row)
   constexpr int TILE_UNITS = 2048;           // ... of the B tile
@@ -64,7 +70,7 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   // is left at the end of a group goes to the tile kernel.  With 128-row tiles (TM == 2) the list is instead one
   // tile per weight panel for every group of rows_lo..rows_hi (<= 128) rows and, if min_rows is set, for the end
   // (what rows_in_256_tiles() leaves) of every group of at least min_rows rows.
-  const int tiles_m = p.m / BM, tiles_n = p.n / BN;
+  const int tiles_m = (RAGGED_M ? p.m + BM - 1 : p.m) / BM, tiles_n = p.n / BN;
   int total = tiles_m * tiles_n;
   if constexpr (GROUPED) {
     if (wave == 0) {  // prefix sums of tiles per group, 64 groups per round
@@ -139,7 +145,7 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
       w.gm0 = mt * BM;
       w.m0 = w.gm0;
       w.n0 = nt * BN;
-      w.valid = BM;
+      w.valid = RAGGED_M ? min(BM, p.m - w.gm0) : BM;
     }
     return w;
   };
@@ -158,14 +164,15 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   // 2*spiece+1 of the span: 128x4 layout column tile spiece>>1, bytes 2*(spiece&1)..).  A tile's first row is
   // a multiple of 128, so the swizzled scale address splits into the tile's part and the thread's part.
   // a_bytes / a_bytes2: bytes of the existing A rows among the tile's rows 0..127 / 128..255 (buffer ranges)
-  struct RowPtrs { const uint8_t *a, *b, *sa, *sb; int a_bytes, a_bytes2; };
+  struct RowPtrs { const uint8_t *a, *b, *sa, *sb; int a_bytes, a_bytes2, sa_bytes2; };
   auto tile_ptrs = [&](int t) {
     const Where w = tile_where(t);
     RowPtrs r;
     r.a = p.a + w.m0 * kbytes;
     // the last tile of a group may have fewer rows than the tile: the rows past the group read as zero
-    r.a_bytes = GROUPED ? min(w.valid, 128) * kbytes : 0x7fffffff;
-    r.a_bytes2 = GROUPED ? max(w.valid - 128, 0) * kbytes : 0x7fffffff;
+    r.a_bytes = PARTIAL ? min(w.valid, 128) * kbytes : 0x7fffffff;
+    r.a_bytes2 = PARTIAL ? max(w.valid - 128, 0) * kbytes : 0x7fffffff;
+    r.sa_bytes2 = RAGGED_M && w.valid <= 128 ? 0 : 0x7fffffff;  // (no rows 128.. : their scale tile may not exist)
     r.b = p.b + ((int64_t)w.g * p.n + w.n0) * kbytes;
     // (a group's activation scales are a slab of their own, swizzled from its first row)
     const int64_t sa_slab = GROUPED ? (int64_t)__builtin_amdgcn_readfirstlane(p.sf_offsets[w.g]) * sf_padded : 0;
@@ -200,7 +207,10 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
     if (q == 2) r.b[0] = __builtin_amdgcn_raw_buffer_load_b128(rsrc(lp.b), off_ab, o, 0);
     if (q == 3) r.b[1] = __builtin_amdgcn_raw_buffer_load_b128(rsrc(lp.b), off_ab, o + (int)row128, 0);
     if (q == 4) r.sa[0] = __builtin_amdgcn_raw_buffer_load_b16(rsrc(lp.sa), off_sf, so, 0);
-    if (q == 5 && AR == 2) r.sa[1] = __builtin_amdgcn_raw_buffer_load_b16(rsrc(lp.sa), off_sf, so + (int)sfrow128, 0);
+    if (q == 5 && AR == 2) {
+      if constexpr (RAGGED_M) r.sa[1] = __builtin_amdgcn_raw_buffer_load_b16(rsrc(lp.sa + sfrow128, lp.sa_bytes2), off_sf, so, 0);
+      else r.sa[1] = __builtin_amdgcn_raw_buffer_load_b16(rsrc(lp.sa), off_sf, so + (int)sfrow128, 0);
+    }
     if (q == 6) r.sb[0] = __builtin_amdgcn_raw_buffer_load_b16(rsrc(lp.sb), off_sf, so, 0);
     if (q == 7) r.sb[1] = __builtin_amdgcn_raw_buffer_load_b16(rsrc(lp.sb), off_sf, so + (int)sfrow128, 0);
   };
@@ -210,6 +220,7 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
     lp.a = wrap ? np.a : lp.a;
     lp.a_bytes = wrap ? np.a_bytes : lp.a_bytes;
     lp.a_bytes2 = wrap ? np.a_bytes2 : lp.a_bytes2;
+    if (RAGGED_M) lp.sa_bytes2 = wrap ? np.sa_bytes2 : lp.sa_bytes2;
     lp.b = wrap ? np.b : lp.b;
     lp.sa = wrap ? np.sa : lp.sa;
     lp.sb = wrap ? np.sb : lp.sb;
@@ -512,7 +523,7 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
           for (int t = 0; t < 2; ++t) {
             const int brow = i * 32 + 16 * t;  // first of the 16 rows of this piece, in the wavefront's tile
             const u32x4 v = *reinterpret_cast<const u32x4*>(rd + t * 1280);
-            if (!GROUPED || wm * (32 * TM) + brow + erow < cw.valid)
+            if (!PARTIAL || wm * (32 * TM) + brow + erow < cw.valid)
               *reinterpret_cast<u32x4*>(obase + ((int64_t)brow * ldc + j * 32) * 2 + ooff) = v;
           }
           asm volatile("" ::: "memory");
@@ -524,17 +535,18 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
 #undef NVF_PIN_ACC
 }
 
-template <bool OUT_BF16, bool GROUPED, int TM, bool OUT_F32, bool PAIRS, bool OUT_FP4 = false, bool RAGGED_K = false>
+template <bool OUT_BF16, bool GROUPED, int TM, bool OUT_F32, bool PAIRS, bool OUT_FP4 = false, bool RAGGED_K = false, bool RAGGED_M = false>
 int launch_nvfp4_fast_cfg(const Params& p, int cus, hipStream_t stream) {
-  auto kern = nvfp4_gemm_256_kernel<OUT_BF16, GROUPED, TM, OUT_F32, PAIRS, OUT_FP4, RAGGED_K>;
+  auto kern = nvfp4_gemm_256_kernel<OUT_BF16, GROUPED, TM, OUT_F32, PAIRS, OUT_FP4, RAGGED_K, RAGGED_M>;
+  if (!GROUPED && !RAGGED_M && p.m % (64 * TM) != 0) return fail(NVF_ERR_LAUNCH, "nvfp4_gemm_256_kernel: M = %d is no multiple of %d", p.m, 64 * TM);
   constexpr int lds_bytes = 2 * (64 * TM + 256) * 128 + 8 * 2560;  // 128 KiB / 96 KiB of tiles + the epilogue's 20 KiB
   // grouped: an upper bound (128-row tiles: one per weight panel and group of at least rows_lo rows)
-  const int64_t tiles_m = (GROUPED && TM == 2) ? std::min<int64_t>(p.groups, p.m / std::max(p.rows_lo, 1)) : p.m / (64 * TM);
+  const int64_t tiles_m = (GROUPED && TM == 2) ? std::min<int64_t>(p.groups, p.m / std::max(p.rows_lo, 1)) : (p.m + (RAGGED_M ? 64 * TM - 1 : 0)) / (64 * TM);
   const int64_t tiles = tiles_m * (p.n / 256);
   const unsigned grid = (unsigned)(tiles >= cus ? (cus & ~7) : ((tiles + 7) / 8) * 8);
   if (grid == 0) return NVF_OK;  // fewer rows in the whole call than the smallest group this launch serves: no work
   if (note_launch("nvfp4_gemm_256_kernel<grouped=%d,TM=%d,f32=%d,pairs=%d%s%s> grid=%u rows=%d..%d min_rows=%d", (int)GROUPED, TM, (int)OUT_F32,
-                  (int)PAIRS, OUT_FP4 ? ",fp4_blockscale" : "", RAGGED_K ? ",ragged_k" : "", grid, p.rows_lo, p.rows_hi, p.min_rows))
+                  (int)PAIRS, OUT_FP4 ? ",fp4_blockscale" : (RAGGED_M ? ",ragged_m" : ""), RAGGED_K ? ",ragged_k" : "", grid, p.rows_lo, p.rows_hi, p.min_rows))
     return NVF_OK;
   static std::atomic<uint64_t> configured{0};  // one bit per device
   if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
@@ -549,6 +561,12 @@ int launch_nvfp4_fast(const Params& p, int cus, hipStream_t stream) {
     if ((p.k & 127) != 0) {  // a short last span: an even number of spans counts it
       if ((((p.k + 127) >> 7) & 1) == 0) return launch_nvfp4_fast_cfg<OUT_BF16, GROUPED, TM, OUT_F32, true, OUT_FP4, true>(p, cus, stream);
       return launch_nvfp4_fast_cfg<OUT_BF16, GROUPED, TM, OUT_F32, false, OUT_FP4, true>(p, cus, stream);
+    }
+  }
+  if constexpr (!GROUPED && !OUT_F32 && !OUT_FP4) {
+    if (p.m % (64 * TM) != 0) {  // a last row tile with fewer rows
+      if (((p.k >> 7) & 1) == 0) return launch_nvfp4_fast_cfg<OUT_BF16, GROUPED, TM, OUT_F32, true, OUT_FP4, false, true>(p, cus, stream);
+      return launch_nvfp4_fast_cfg<OUT_BF16, GROUPED, TM, OUT_F32, false, OUT_FP4, false, true>(p, cus, stream);
     }
   }
   if (((p.k >> 7) & 1) == 0) return launch_nvfp4_fast_cfg<OUT_BF16, GROUPED, TM, OUT_F32, true, OUT_FP4>(p, cus, stream);

@@ -99,18 +99,19 @@ def test_nvfp4_mid_sized_shapes(m, n, k, kernel):
     assert plan("nvfp4_scaled_mm", m, n, k).startswith(kernel), plan("nvfp4_scaled_mm", m, n, k)
 
 
-def test_nvfp4_dense_m_not_a_multiple_of_128_is_cut_into_a_main_part_and_a_remainder():
+def test_nvfp4_dense_m_not_a_multiple_of_the_tile_height_takes_the_persistent_kernel_with_a_short_last_row_tile():
     op = "nvfp4_scaled_mm"
-    # a prefill of any token count: the rows up to a multiple of 128 / 256 on the persistent kernel, the rest streamed
-    got = plan(op, 4000, 4096, 4096).split("; ")
-    assert len(got) == 2 and "gemm_256_kernel<" in got[0] and "TM=4" in got[0] and "skinny" in got[1], got
-    got = plan(op, 8100, 8192, 8192).split("; ")
-    assert len(got) == 2 and "gemm_256_kernel<" in got[0] and "TM=4" in got[0] and "grid=256" in got[0] and "skinny" in got[1], got
-    # where the main part would stream as well, one launch takes all rows
-    got = plan(op, 1000, 4096, 14336).split("; ")
-    assert len(got) == 1 and "skinny" in got[0], got
-    # multiples of 128 and small shapes: as before
-    assert "; " not in plan(op, 4096, 4096, 4096) and "; " not in plan(op, 300, 4096, 4096)
+    # a prefill of any token count: one launch, the last row tile with fewer rows
+    for m, n, k, tm, grid in ((4000, 4096, 4096, 4, 256), (8100, 8192, 8192, 4, 256), (384, 28672, 4096, 4, 224), (160, 28672, 4096, 2, 224)):
+        got = plan(op, m, n, k)
+        assert got.startswith(f"nvfp4_gemm_256_kernel<grouped=0,TM={tm},") and "ragged_m" in got and f"grid={grid} " in got and ";" not in got, (m, n, k, got)
+    # where the weight-streaming kernel is estimated faster it takes all rows, and multiples of the tile height are as before
+    got = plan(op, 1000, 4096, 14336)
+    assert "skinny" in got and ";" not in got, got
+    assert "ragged_m" not in plan(op, 4096, 4096, 4096) and "skinny" in plan(op, 300, 4096, 4096)
+    # K % 128 != 0 has its own variant of the kernel: such a shape is still cut at a multiple of 128 rows
+    got = plan(op, 4000, 4096, 2880).split("; ")
+    assert len(got) == 2 and "ragged_k" in got[0] and "skinny" in got[1], got
 
 
 def test_mxfp8_dense_m_not_a_multiple_of_the_tile_height_takes_the_persistent_kernel_with_a_short_last_row_tile():

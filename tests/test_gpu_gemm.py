@@ -471,6 +471,43 @@ def test_nvfp4_gemm_k_not_a_multiple_of_128_on_the_persistent_kernel(dev, shape)
         assert torch.equal(out, _run_nvfp4(a, b, sa_p, sb_p, alpha, dtype, dev))
 
 
+@pytest.mark.parametrize("shape", [(300, 14336, 512), (264, 12288, 256), (520, 14336, 512), (640, 14336, 384), (700, 12288, 256),
+                                   (2049, 4096, 512), (390, 28672, 384)])
+def test_nvfp4_gemm_last_row_tile_with_fewer_rows_on_the_persistent_kernel(dev, shape):
+    """M no multiple of the tile height, N % 256 == K % 128 == 0 and enough tiles: the persistent kernel's variant whose
+    last row tile reads the rows past M as zero (the range of its buffer ends with the last row) and does not store
+    them.  128-row tiles with 44 and 8 rows in the last one, 256-row tiles with 8 rows (the scale tile of the tile's
+    second half does not exist and is not read), 128 (M % 256 == 128), 188, 1 and 134 rows; two, three and four spans.
+    NaN code in all scale padding, both output types, every element against the oracle, run-to-run bit equality; through
+    the C ABI into the first M rows of a larger buffer, whose other rows keep their contents."""
+    from fuser_amd import capi
+
+    m, n, k = shape
+    plan = capi.describe_dispatch("nvfp4_scaled_mm", m, n, k)
+    assert plan.startswith("nvfp4_gemm_256_kernel<") and "ragged_m" in plan and ";" not in plan, plan
+    gen = torch.Generator().manual_seed(m + n + k)
+    a, sa, ga = _nvfp4_operand(m, k, 1.0, gen)
+    b, sb, gb = _nvfp4_operand(n, k, 0.02, gen)
+    alpha = 1.0 / (ga * gb)
+    ref = O.ref_nvfp4_scaled_mm(a, b, sa, sb, alpha)
+    sa_p, sb_p = sa.clone(), sb.clone()
+    sa_p[O.linear_to_swizzled_128_4(torch.ones(m, k // 16, dtype=torch.uint8)) == 0] = 0x7F
+    sb_p[O.linear_to_swizzled_128_4(torch.ones(n, k // 16, dtype=torch.uint8)) == 0] = 0x7F
+    for dtype in (torch.bfloat16, torch.float16):
+        out = _run_nvfp4(a, b, sa_p, sb_p, alpha, dtype, dev)
+        assert out.shape == (m, n) and torch.isfinite(out.float()).all()
+        assert max_rel_rowwise(out, ref) <= GEMM_MAX_REL, (shape, dtype, plan)
+        assert torch.equal(out, _run_nvfp4(a, b, sa_p, sb_p, alpha, dtype, dev))
+    buf = torch.full((m + 130, n), 7.0, dtype=torch.bfloat16, device=dev)
+    ad, bd, sad, sbd = a.to(dev), b.to(dev), sa_p.to(dev), sb_p.to(dev)
+    al = torch.tensor(float(alpha), dtype=torch.float32, device=dev)
+    capi.check(capi.lib().nvf_nvfp4_scaled_mm(ad.data_ptr(), bd.data_ptr(), sad.data_ptr(), sbd.data_ptr(), al.data_ptr(), buf.data_ptr(),
+                                              m, n, k, capi.BF16, None))
+    torch.cuda.synchronize()
+    assert max_rel_rowwise(buf[:m], ref) <= GEMM_MAX_REL
+    assert bool((buf[m:] == 7.0).all())
+
+
 @pytest.mark.parametrize("shape", [(384, 6176, 8224), (512, 5152, 8224), (640, 4224, 12320), (512, 3104, 12320),
                                    (80, 6144, 8192), (70, 8192, 7168), (72, 4736, 10752), (65, 4096, 14336)])
 def test_nvfp4_gemm_split_k_with_workspace(dev, shape):
