@@ -287,13 +287,15 @@ def test_nvfp4_gemm_many_rows_small_n_deep_k(dev, shape):
         assert torch.equal(out, _run_nvfp4(a, b, sa_p, sb, alpha, dtype, dev))
 
 
-@pytest.mark.parametrize("shape", [(2100, 4096, 2048), (2504, 2048, 2048), (1000, 14336, 2048), (2304 + 255, 4096, 2048), (4300, 2048, 2048), (1000, 2048, 256)])
+@pytest.mark.parametrize("shape", [(2100, 4096, 2048), (2504, 2048, 2048), (1000, 14336, 2048), (2304 + 255, 4096, 2048), (4300, 2048, 2048), (1000, 2048, 256),
+                                   (2100, 4096, 2080), (2504, 2048, 2144), (1000, 14336, 2080), (4300, 2048, 2080)])
 def test_dense_gemms_with_m_not_a_multiple_of_128(dev, shape):
-    """A prefill of any token count: M > 128 and not a multiple of 128 is cut at a multiple of 128 or 256; the rows
-    before the cut go to the persistent (or streaming) kernel, the 1..255 rows after it to the weight-streaming kernel
-    in a launch of its own, which reads its activation scales a whole number of 128-row scale tiles further on.  Both
-    ops, both output types, every element against the oracle, poisoned scale padding, rows of the two launches next to
-    the cut compared like all others, run-to-run bit equality."""
+    """A prefill of any token count, M > 128 and not a multiple of 128.  K % 128 == 0: one launch of the persistent
+    kernel whose last row tile holds fewer rows.  K % 128 != 0 (the last four shapes; that variant of the kernel wants
+    whole row tiles): cut at a multiple of 128 or 256; the rows before the cut go to the persistent kernel, the 1..255
+    rows after it to the weight-streaming kernel in a launch of its own, which reads its activation scales a whole
+    number of 128-row scale tiles further on.  Both ops, both output types, every element against the oracle, poisoned
+    scale padding, rows of the two launches next to the cut compared like all others, run-to-run bit equality."""
     from fuser_amd import capi
 
     m, n, k = shape
@@ -326,7 +328,10 @@ def test_dense_gemms_with_m_not_a_multiple_of_128(dev, shape):
         assert out.shape == (m, n)
         assert ((out.float().cpu() - ref).abs() / scale).max().item() <= GEMM_MAX_REL, (shape, dtype, plans[-1])
         assert torch.equal(out, _run_mxfp8(a8, b8, sa8_p, sb8, 0.75, dtype, dev))
-    assert all("; " in p for p in plans) or shape == (1000, 2048, 256), plans  # (the last shape: cut for MXFP8 only)
+    if k % 128 != 0:
+        assert all("; " in p and "ragged_k" in p for p in plans), plans
+    elif shape != (1000, 2048, 256):  # (too few tiles for the persistent kernel)
+        assert all("ragged_m" in p and "; " not in p for p in plans), plans
 
 
 @pytest.mark.parametrize("shape", [(2048, 2432, 256), (2100, 2368, 384), (1536, 4128, 256), (640, 4224, 2048), (2048, 4224, 2048)])
