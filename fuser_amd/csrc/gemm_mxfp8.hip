@@ -900,7 +900,10 @@ Plan mxfp8_plan(int64_t m, int64_t n, int64_t k, int64_t cus, int64_t* ns = null
       // about 5 us (so cost 100 = 11.3 us per 1024 of K), the skinny kernel what its estimate says (its unit is
       // 0.96 ns).  Measured: 256 x 14336 x 4096 31 (persistent) against 47 us, 512 x 4096 x 7168 51 against 30 us
       // (skinny), 1024 x 2048 x 14336 97 against 48 us, 1024 x 4096 x 4096 31 against 34 us.
-      if (skinny_ns <= fast_ns) return Plan::kStream;
+      // (129..192 rows are three slabs of 64, which the estimate puts 15-22 % low against a wide N: 160 and 192 x 14336
+      // x 4096 run 37 and 40 us streamed, estimated 31, and 31 us on 112 tiles of 128 rows)
+      const int64_t margin = m > 128 && m <= 192 ? skinny_ns / 5 : 0;
+      if (skinny_ns + margin <= fast_ns) return Plan::kStream;
     } else {
       // No persistent kernel for the shape (ragged M or N, or too few tiles): up to 256 rows, i.e. four passes over
       // the weights, the skinny kernel beats the tile kernels (128 x 4096 x 14336: 20 instead of 117 us); with more
