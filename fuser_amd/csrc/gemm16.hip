@@ -184,7 +184,7 @@ DensePlan nvfp4_dense_plan(int64_t m, int64_t n, int64_t k, int cus) {
   // (a short last span is fine; so is, with whole spans, a last row tile with fewer rows, which counts as a whole one:
   // 384 x 28672 x 4096 as 224 tiles of 256 rows in one round instead of 336 of 128 rows in two)
   const bool persistent_shape = (n & 255) == 0 && (k & 31) == 0 && k >= 256;
-  const bool ok256 = persistent_shape && ((m & 255) == 0 || ((k & 127) == 0 && m > 256));
+  const bool ok256 = persistent_shape && ((m & 255) == 0 || ((k & 127) == 0 && m > 128));
   const bool persistent_ok = persistent_shape && ((m & 127) == 0 || ((k & 127) == 0 && m > 128));
   int64_t cost256 = INT64_MAX, cost128 = INT64_MAX, cost_tile = INT64_MAX;
   if (persistent_ok) {
@@ -232,7 +232,7 @@ int nvfp4_n_cut(int64_t m, int64_t n, int64_t k, int cus, int64_t* ns = nullptr)
   if (ns) *ns = INT64_MAX;
   if ((n & 255) == 0 || n <= 256 || m <= 128 || (k & 31) != 0 || k < 256) return 0;
   const DensePlan whole = nvfp4_dense_plan(m, n, k, cus);
-  const DensePlan main_plan = nvfp4_dense_plan(m & ~127, n & ~255, k, cus), rest_plan = nvfp4_dense_plan(m, n & 255, k, cus);
+  const DensePlan main_plan = nvfp4_dense_plan(m, n & ~255, k, cus), rest_plan = nvfp4_dense_plan(m, n & 255, k, cus);
   const bool whole_other = whole.kernel == DensePlan::kOther;
   if (main_plan.kernel == DensePlan::kOther) return 0;
   const bool have_cut_ns = rest_plan.kernel == DensePlan::kStream && main_plan.ns != INT64_MAX;

@@ -884,7 +884,7 @@ Plan mxfp8_plan(int64_t m, int64_t n, int64_t k, int64_t cus, int64_t* ns = null
   // (a last row tile with fewer rows: the variant that clamps the rows of its activation loads, K % 128 == 0 only;
   // the tile counts as a whole one.  640 x 14336 x 4096: 280 tiles of 128 rows in 2 rounds 60 us, 168 of 256 rows 43 us)
   const bool fast_shape = (k & 31) == 0 && k >= 256 && (n & 255) == 0 && k * 256 < (1ll << 31);
-  const bool ok256 = fast_shape && ((m & 255) == 0 || ((k & 127) == 0 && m > 256));
+  const bool ok256 = fast_shape && ((m & 255) == 0 || ((k & 127) == 0 && m > 128));
   const bool ok128 = fast_shape && ((m & 127) == 0 || ((k & 127) == 0 && m > 64));
   const int64_t t256 = ok256 ? ceil_div(m, 256) * (n / 256) : 0, t128 = ok128 ? ceil_div(m, 128) * (n / 256) : 0;
   const int64_t cost256 = t256 >= 128 ? 100 * ceil_div(t256, cus) : INT64_MAX;
@@ -900,9 +900,10 @@ Plan mxfp8_plan(int64_t m, int64_t n, int64_t k, int64_t cus, int64_t* ns = null
       // about 5 us (so cost 100 = 11.3 us per 1024 of K), the skinny kernel what its estimate says (its unit is
       // 0.96 ns).  Measured: 256 x 14336 x 4096 31 (persistent) against 47 us, 512 x 4096 x 7168 51 against 30 us
       // (skinny), 1024 x 2048 x 14336 97 against 48 us, 1024 x 4096 x 4096 31 against 34 us.
-      // (129..192 rows are three slabs of 64, which the estimate puts 15-22 % low against a wide N: 160 and 192 x 14336
-      // x 4096 run 37 and 40 us streamed, estimated 31, and 31 us on 112 tiles of 128 rows)
-      const int64_t margin = m > 128 && m <= 192 ? skinny_ns / 5 : 0;
+      // (129..256 rows are three or four slabs of 64, which the estimate puts 15-22 % low against a wide N: 160 and 192 x
+      // 14336 x 4096 run 37 and 40 us streamed, estimated 31, and 31 us on 112 tiles of 128 rows; 256 x 11008 x 4096
+      // 38 against 31 us)
+      const int64_t margin = m > 128 && m <= 256 ? skinny_ns / 5 : 0;
       if (skinny_ns + margin <= fast_ns) return Plan::kStream;
     } else {
       // No persistent kernel for the shape (ragged M or N, or too few tiles): up to 256 rows, i.e. four passes over
@@ -933,9 +934,9 @@ int launch_sized(const Params& p, hipStream_t stream) {
   // N not a multiple of 256 (29568, 1408): the columns up to the last multiple of 256 go to whatever kernel that shape
   // gets, the remaining columns (weight rows) to a launch of their own that writes into the same rows of the result
   // (8192 x 29568 x 8192: 4.1 -> 1.3 ms).
-  if ((p.n & 255) != 0 && p.n > 256 && (p.n & 15) == 0 && p.m > 128 && (p.k & 31) == 0 && p.k >= 256) {
+  if ((p.n & 255) != 0 && p.n > 256 && (p.n & 15) == 0 && p.m > 64 && (p.k & 31) == 0 && p.k >= 256) {
     int64_t main_ns, rest_ns;
-    const Plan main_plan = mxfp8_plan(p.m & ~127, p.n & ~255, p.k, cus, &main_ns), rest_plan = mxfp8_plan(p.m, p.n & 255, p.k, cus, &rest_ns);
+    const Plan main_plan = mxfp8_plan(p.m, p.n & ~255, p.k, cus, &main_ns), rest_plan = mxfp8_plan(p.m, p.n & 255, p.k, cus, &rest_ns);
     if (whole_other && main_plan == Plan::kStream) return launch_skinny<OUT_BF16>(p, stream);  // (takes any N % 16 == 0)
     if (main_plan != Plan::kOther && (whole_other || (is_tiles(main_plan) && rest_plan == Plan::kStream && main_ns != INT64_MAX &&
                                                        rest_ns != INT64_MAX && main_ns + rest_ns < bar))) {

@@ -134,9 +134,13 @@ def test_mxfp8_dense_m_not_a_multiple_of_the_tile_height_takes_the_persistent_ke
 def test_dense_n_not_a_multiple_of_256_is_cut_into_a_main_part_and_the_remaining_columns(op):
     got = plan(op, 8192, 29568, 8192).split("; ")
     assert len(got) == 2 and "gemm_256_kernel<" in got[0] and "TM=4" in got[0] and "grid=256" in got[0] and "skinny" in got[1], got
-    # few rows: the weight-streaming kernel takes any N % 16 == 0 in one launch
-    got = plan(op, 100, 29568, 4096).split("; ")
+    # few rows: the weight-streaming kernel takes any N % 16 == 0 in one launch (MXFP8 from 65 rows on: one round of
+    # 128x256 tiles with 100 rows each for the columns up to the last multiple of 256 is estimated faster)
+    got = plan(op, 100 if op == "nvfp4_scaled_mm" else 48, 29568, 4096).split("; ")
     assert len(got) == 1 and "skinny" in got[0], got
+    if op == "mxfp8_scaled_mm":
+        got = plan(op, 100, 29568, 4096).split("; ")
+        assert len(got) == 2 and got[0].startswith("mxfp8_gemm_256_kernel<TM=2,") and "ragged_m" in got[0] and "skinny" in got[1], got
 
 
 def test_nvfp4_8192_cubed_takes_the_persistent_256x256_kernel():

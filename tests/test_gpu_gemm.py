@@ -334,12 +334,14 @@ def test_dense_gemms_with_m_not_a_multiple_of_128(dev, shape):
         assert all("ragged_m" in p and "; " not in p for p in plans), plans
 
 
-@pytest.mark.parametrize("shape", [(2048, 2432, 256), (2100, 2368, 384), (1536, 4128, 256), (640, 4224, 2048), (2048, 4224, 2048)])
+@pytest.mark.parametrize("shape", [(2048, 2432, 256), (2100, 2368, 384), (1536, 4128, 256), (640, 4224, 2048), (2048, 4224, 2048),
+                                   (100, 12416, 512), (200, 12352, 512), (200, 32896, 2048)])
 def test_dense_gemms_with_n_not_a_multiple_of_256(dev, shape):
-    """N > 256 and not a multiple of 256 with 512 rows or more: the columns up to the last multiple of 256 go to the
-    persistent kernel, the remaining 32..224 columns to a launch of their own (tile kernel or weight-streaming kernel)
-    that writes into the same rows of the result at the full row pitch; the second shape is cut along M as well.  Both
-    ops, both output types, every element against the oracle (a launch writing at the wrong pitch would show), run-to-run
+    """N > 256 and not a multiple of 256: the columns up to the last multiple of 256 go to the persistent kernel, the
+    remaining 32..224 columns to a launch of their own (tile kernel or weight-streaming kernel) that writes into the same
+    rows of the result at the full row pitch; the second shape is cut along M as well (K % 128 != 0), the last three
+    have a short last row tile in the main part (100 rows: MXFP8 only, NVFP4 streams; the last: both ops).  Both ops,
+    both output types, every element against the oracle (a launch writing at the wrong pitch would show), run-to-run
     bit equality."""
     from fuser_amd import capi
 
@@ -477,12 +479,13 @@ def test_nvfp4_gemm_k_not_a_multiple_of_128_on_the_persistent_kernel(dev, shape)
 
 
 @pytest.mark.parametrize("shape", [(300, 14336, 512), (264, 12288, 256), (520, 14336, 512), (640, 14336, 384), (700, 12288, 256),
-                                   (2049, 4096, 512), (390, 28672, 384)])
+                                   (2049, 4096, 512), (390, 28672, 384), (200, 49152, 2048)])
 def test_nvfp4_gemm_last_row_tile_with_fewer_rows_on_the_persistent_kernel(dev, shape):
     """M no multiple of the tile height, N % 256 == K % 128 == 0 and enough tiles: the persistent kernel's variant whose
     last row tile reads the rows past M as zero (the range of its buffer ends with the last row) and does not store
     them.  128-row tiles with 44 and 8 rows in the last one, 256-row tiles with 8 rows (the scale tile of the tile's
-    second half does not exist and is not read), 128 (M % 256 == 128), 188, 1 and 134 rows; two, three and four spans.
+    second half does not exist and is not read), 128 (M % 256 == 128), 188, 1 and 134 rows, and a single 256-row tile row
+    with 200 rows; 2 to 16 spans.
     NaN code in all scale padding, both output types, every element against the oracle, run-to-run bit equality; through
     the C ABI into the first M rows of a larger buffer, whose other rows keep their contents."""
     from fuser_amd import capi
@@ -799,12 +802,13 @@ def test_mxfp8_gemm_persistent_256_tile_kernel_full_compare(dev, shape):
 
 
 @pytest.mark.parametrize("shape", [(300, 14336, 512), (136, 12288, 512), (80, 28672, 256), (520, 14336, 512), (640, 14336, 1024),
-                                   (700, 12288, 256), (2049, 4096, 512), (390, 8192, 1280)])
+                                   (700, 12288, 256), (2049, 4096, 512), (390, 8192, 1280), (200, 65536, 256), (130, 65536, 256)])
 def test_mxfp8_gemm_last_row_tile_with_fewer_rows_on_the_persistent_kernel(dev, shape):
     """M no multiple of the tile height, N % 256 == K % 128 == 0 and enough tiles: the persistent kernel's variant whose
     last row tile clamps the rows of its activation loads and stores only the rows that exist.  128-row tiles with 44,
     8 and 80 rows in the last one (one tile row in all for the 80), 256-row tiles with 8 rows (the tile's second scale
-    tile does not exist: the last one is read instead), 128 (M % 256 == 128), 188 and 1 row; two to ten K steps.  NaN
+    tile does not exist: the last one is read instead), 128 (M % 256 == 128), 188 and 1 row, and a single 256-row tile row
+    with 200 and 130 rows; two to ten K steps.  NaN
     code in every scale byte of the padding rows, both output types, every element compared, rows are written once
     (a result buffer pre-filled with a pattern keeps it past row M), run-to-run determinism."""
     from fuser_amd import capi
