@@ -382,8 +382,10 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int6
     }
   }
   if constexpr (!NVFP4) {
-    // grouped_mm with groups of a few hundred rows on average: persistent LDS-direct kernel
-    if (!dense && m_hint >= 256 * (int64_t)p.groups && tiles(256, 256) >= cus / 2 && (p.n & 255) == 0 && (p.k & 63) == 0 &&
+    // grouped_mm with groups of 128 rows or more on average and tiles for half the compute units: persistent LDS-direct
+    // kernel (at 128..255 rows per group the 128x128 tile kernel used to run: 8 experts, 1536 rows, N=14336, K=4096 373 ->
+    // 272 us; 64 experts, 8192 rows, N=7168, K=2048 571 -> 449 us; below 128 rows per group it stays faster)
+    if (!dense && m_hint >= 128 * (int64_t)p.groups && tiles(256, 256) >= cus / 2 && (p.n & 255) == 0 && (p.k & 63) == 0 &&
         p.k >= 128 && (int64_t)p.k * 2 * 256 < (1ll << 31))
       return launch_grouped16_fast<BF16_MMA, OUT_BF16>(p, cus, stream);
   }

@@ -150,6 +150,11 @@ def test_nvfp4_8192_cubed_takes_the_persistent_256x256_kernel():
 def test_config4_bf16_grouped_takes_the_persistent_kernel_in_one_launch():
     got = plan("grouped_mm", 8192, 14336, 4096, groups=8)
     assert got.startswith("grouped16_gemm_256_kernel<") and ";" not in got, got
+    # from 128 rows per group on average, where its 256x256 tiles cover half the compute units; the tile kernels below
+    assert plan("grouped_mm", 1024, 14336, 4096, groups=8).startswith("grouped16_gemm_256_kernel<")
+    assert plan("grouped_mm", 8192, 2048, 7168, groups=64).startswith("grouped16_gemm_256_kernel<")
+    assert plan("grouped_mm", 1000, 14336, 4096, groups=8).startswith("gemm16_kernel<")
+    assert plan("grouped_mm", 1024, 4096, 14336, groups=8).startswith("gemm16_kernel<")  # 64 tiles of 256x256 only
 
 
 @pytest.mark.parametrize("n,k", [(2048, 7168), (7168, 2048)])

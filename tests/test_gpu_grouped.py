@@ -117,6 +117,34 @@ def test_grouped_mm_group_ends_inside_tiles(dev, n, k):
     assert ((out[:rows].float().cpu() - ref[:rows]).abs() / scale).max().item() <= GEMM_MAX_REL
 
 
+@pytest.mark.parametrize("n,k", [(14336, 192), (8192, 128)])
+def test_grouped_mm_persistent_kernel_from_128_rows_per_group(dev, n, k):
+    """128 to 255 rows per group on average and a wide N: the persistent kernel (most of its 256-row tiles are short,
+    one group is empty, two have a single tile of 1 and of 255 rows).  Every element compared, rows after the last
+    group untouched, both operand types."""
+    from fuser_amd import capi
+
+    sizes = [130, 0, 255, 1, 200, 128, 300, 129, 90, 257]
+    m = sum(sizes) + 5
+    assert 128 * len(sizes) <= m < 256 * len(sizes)
+    assert capi.describe_dispatch("grouped_mm", m, n, k, groups=len(sizes)).startswith("grouped16_gemm_256_kernel")
+    for tensor_dtype, dt in ((torch.bfloat16, capi.BF16), (torch.float16, capi.F16)):
+        gen = torch.Generator().manual_seed(n + k)
+        a = torch.randn(m, k, generator=gen).to(tensor_dtype)
+        b = (torch.randn(len(sizes), n, k, generator=gen) * 0.05).to(tensor_dtype)
+        ps, eo, _, _ = _grouped_args(sizes, n, k, dev)
+        ad, bd, psd, eod = a.to(dev), b.to(dev), ps.to(dev), eo.to(dev)
+        out = torch.full((m, n), 7.0, dtype=tensor_dtype, device=dev)
+        capi.check(capi.lib().nvf_grouped_mm(ad.data_ptr(), bd.data_ptr(), out.data_ptr(), psd.data_ptr(), eod.data_ptr(), len(sizes),
+                                             m, n, k, dt, None))
+        torch.cuda.synchronize()
+        ref = O.ref_grouped_mm(a, b, ps, eo)
+        rows = sum(sizes)
+        assert (out[rows:] == 7.0).all()
+        scale = ref[:rows].abs().amax(dim=1, keepdim=True).clamp(min=1e-30)
+        assert ((out[:rows].float().cpu() - ref[:rows]).abs() / scale).max().item() <= GEMM_MAX_REL, tensor_dtype
+
+
 def _moe_sizes_top2(tokens, experts, seed):
     gen = torch.Generator().manual_seed(seed)
     logits = torch.randn(tokens, experts, generator=gen) + torch.linspace(-1.5, 1.5, experts)
