@@ -359,6 +359,12 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int6
   // Pick the largest tile that still yields about one work item per compute unit.
   auto tiles = [&](int bm, int bn) { return ceil_div(m_hint, bm) * ceil_div(p.n, bn); };
   const bool dense = p.problem_sizes == nullptr;
+  // grouped NVFP4: does the call count as a prefill (see kPrefillRows)?  Also with fewer rows where the large groups'
+  // launches find a round of 256x256 tiles - with 128 rows per group on average, or two rounds whatever the groups
+  // (8 experts, 1536 rows, N=14336, K=4096: 320 -> 223 us; 16 experts, 3072 rows: 540 -> 394; 128 experts, 5632 rows,
+  // N=7168, K=2048: 460 -> 336; at 96 rows per group and one round the other launches stay faster: 125 against 167 us)
+  const int64_t tiles256 = (m_hint / 256) * (p.n / 256);
+  const bool is_prefill = m_hint >= kPrefillRows || (tiles256 >= cus && m_hint >= 128 * (int64_t)p.groups) || tiles256 >= 2 * (int64_t)cus;
   if constexpr (NVFP4) {
     if (dense && workspace != nullptr) {
       const int skinny_splits = nvfp4_skinny_splits(p.m, p.n, p.k, cus);
@@ -416,21 +422,18 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int6
       // found by rank among the groups of their size (a launch with few workgroups when there are few rows in all).  A
       // 128x256 tile of the persistent kernel walks all of K on one compute unit: with 64 or 256 experts, 512..5600
       // rows and K = 4096..14336 the call is 5-40 % slower that way wherever such groups exist and 0-3 % faster where
-      // none does; with K < 4096 the tiles win from about 2048 rows on.  Kept on the tiles: many groups of near 128
-      // rows against wide weights (64 experts, 5600 rows, N=14336, K=4096: 0.97 against 1.05 ms).
-      const int64_t mid_tiles = std::min<int64_t>(p.groups, m_hint / 33) * (p.n / 256);
-      const bool mid_on_tiles = mid_tiles >= 12 * (int64_t)cus && m_hint >= 80 * (int64_t)p.groups;
-      if (m_hint <= 1024 || (p.k >= 4096 && m_hint < kPrefillRows && !mid_on_tiles)) {
+      // none does; with K < 4096 the tiles win from about 2048 rows on.
+      if (m_hint <= 1024 || (p.k >= 4096 && !is_prefill)) {
         rc = launch_nvfp4_skinny_grouped<4, 8, OUT_BF16, false>(p, 33, 128, stream);
-      } else if ((p.k < 4096 || m_hint < kPrefillRows) && (p.n & 255) == 0 && p.k >= 256) {
+      } else if ((p.k < 4096 || !is_prefill) && (p.n & 255) == 0 && p.k >= 256) {
         // shallow K: one 128x256 tile of the persistent kernel per weight panel converts a group's rows once per 256
         // weight rows; the streaming kernel whose wavefronts own rows converts them once per wavefront.
         Params mid = p;
         mid.rows_lo = 33;
         mid.rows_hi = 128;
-        if (m_hint >= kPrefillRows) mid.min_rows = 129;  // the 256x256 kernel follows: take the ends of its groups along
+        if (is_prefill) mid.min_rows = 129;  // the 256x256 kernel follows: take the ends of its groups along
         tail_done = mid.min_rows != 0;
-        if (m_hint >= kPrefillRows && (p.n & 511) == 0 && p.k >= 1024) {
+        if (is_prefill && (p.n & 511) == 0 && p.k >= 1024) {
           // a prefill: the groups of up to 80 rows on the panel kernel, which multiplies row tiles of 16 (config 5,
           // K=2048: 5376 tiles of 128x256 in 680 us -> 325 us + 1792 tiles in 227 us)
           rc = launch_nvfp4_group_panel<4, 5, 2, OUT_BF16>(p, 33, 80, stream);
@@ -464,7 +467,7 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int6
     // Grouped NVFP4 with room for whole 256-row tiles: those go to the 256x256 kernel (about 1.4 times as
     // fast per flop), the ends of the groups to the 128x128 tile kernel.  The group sizes live on the
     // device, so both kernels are always launched; one that finds no work returns at once.
-    if (!dense && (p.n & 255) == 0 && (p.k & 31) == 0 && p.k >= 256 && m_hint >= kPrefillRows) {
+    if (!dense && (p.n & 255) == 0 && (p.k & 31) == 0 && p.k >= 256 && is_prefill) {
       const int rc = launch_nvfp4_fast<OUT_BF16, true>(p, cus, stream);
       if (rc != NVF_OK || p.tail_done) return rc;
       Params rest = p;

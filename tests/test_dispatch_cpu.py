@@ -175,8 +175,8 @@ def test_config5_nvfp4_grouped(n, k):
     (4096, 2048, 7168, 256, True, 124),   # a short prefill against deep weights
     (4096, 4096, 14336, 64, True, 64),
     (4096, 7168, 2048, 256, False, 0),    # shallow weights from 1025 rows on: 128x256 tiles of the persistent kernel
-    (5600, 14336, 4096, 64, False, 0),    # many groups of near 128 rows against wide weights: tiles
-    (2048, 14336, 4096, 64, True, 62),
+    (3072, 7168, 2048, 32, False, 0),     # 96 rows per group and one round of 256x256 tiles: no prefill yet
+    (1536, 14336, 4096, 64, True, 46),
 ])
 def test_nvfp4_grouped_below_the_prefill_size_streams_the_mid_sized_groups(m, n, k, groups, streams, slots):
     got = plan("nvfp4_scaled_grouped_mm", m, n, k, groups=groups)
@@ -188,6 +188,18 @@ def test_nvfp4_grouped_below_the_prefill_size_streams_the_mid_sized_groups(m, n,
     else:
         assert mid[0].startswith("nvfp4_gemm_256_kernel<grouped=1,TM=2"), got
     assert "nvfp4_group_panel_kernel" not in got, got
+
+
+@pytest.mark.parametrize("m,n,k,groups,prefill", [
+    (65536, 2048, 7168, 256, True), (6144, 2048, 7168, 256, True), (6000, 2048, 7168, 256, False),
+    (1536, 14336, 4096, 8, True),     # a round of 256x256 tiles and 128 rows per group on average
+    (2048, 14336, 4096, 64, False),   # a round, but 32 rows per group
+    (3072, 14336, 4096, 64, True),    # two rounds
+    (4096, 4096, 14336, 8, True), (3072, 4096, 14336, 8, False), (5632, 7168, 2048, 128, True), (4096, 7168, 2048, 256, False),
+])
+def test_nvfp4_grouped_counts_as_a_prefill_by_rows_or_by_rounds_of_256_row_tiles(m, n, k, groups, prefill):
+    got = plan("nvfp4_scaled_grouped_mm", m, n, k, groups=groups)
+    assert ("nvfp4_gemm_256_kernel<grouped=1,TM=4" in got) == prefill, got
 
 
 def test_dry_run_reports_argument_errors_and_touches_no_device():

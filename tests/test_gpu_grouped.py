@@ -285,9 +285,11 @@ def test_nvfp4_grouped_mm_fewer_rows_in_all_than_the_smallest_mid_sized_group(de
                                        ([3700, 2248, 130, 400], 256, 384),
                                        ([40, 64, 2100, 33, 65, 100, 128, 50, 0, 32, 3620], 256, 512),
                                        ([40, 64, 2100, 33, 65, 100, 128, 50, 0, 32, 3620], 384, 256),
-                                       ([600, 0, 256, 255, 1, 1030, 512, 3600], 512, 320), ([3700, 2248, 130, 400], 256, 448)])
+                                       ([600, 0, 256, 255, 1, 1030, 512, 3600], 512, 320), ([3700, 2248, 130, 400], 256, 448),
+                                       ([219, 130, 300, 0, 1, 257, 129, 500], 12288, 256), ([90, 40, 700, 64, 33, 1400, 128, 160, 8, 500], 22528, 256)])
 def test_nvfp4_grouped_mm_whole_tiles_and_group_ends(dev, sizes, n, k):
-    """A prefill-sized call (6144 rows or more), N % 256 == 0 (the last two cases with K % 128 = 64: a short last span): the whole 256-row tiles of every group, and a last tile of
+    """A prefill-sized call (6144 rows or more; the last two cases: fewer rows against weights so wide that the 256-row
+    tiles of the large groups fill a round with 128 rows per group, or two rounds), N % 256 == 0 (the last two cases with K % 128 = 64: a short last span): the whole 256-row tiles of every group, and a last tile of
     more than 128 rows, run on the persistent 256x256 kernel (the rows past such a group read as zero payload
     with whatever the scale padding holds - it is poisoned here - and are not stored), the other group ends
     on the 128x128 tile kernel.  Groups with no whole tile, only whole tiles, one row past a tile, 255 of 256
