@@ -241,7 +241,6 @@ __device__ __forceinline__ void lds_dma16(uint32_t lds_byte_addr, const uint8_t*
 // is not defined - are replaced by 2^0, so that the step adds exact zeros.
 template <int TM, bool OUT_BF16, bool STREAM_OUT, bool RAGGED_K = false, bool RAGGED_M = false>
 __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) {
-  static_assert(!(RAGGED_K && RAGGED_M), "one variant per kind of raggedness");
   constexpr int BM = 64 * TM, BN = 256;
   constexpr int A_UNITS = BM * 8;             // 16-byte units of the A tile (BM rows x 8 chunks)
   constexpr int TILE_UNITS = 2048;            // ... of the B tile
@@ -345,17 +344,17 @@ __global__ __launch_bounds__(256, 1) void mxfp8_gemm_256_kernel(const Params p) 
     const int j = q < 4 * TM ? (q >> 1) : q - 2 * TM;
     const uint32_t l = lds_base + (uint32_t)(buf * BUF_UNITS + (op ? A_UNITS + wave * 512 : wave * (BM * 2))) * 16u + j * 1024u;
     const uint8_t* gp = (op ? lp.b : lp.a) + ((int64_t)l_ks << 7);
+    uint32_t voff = ((j & 1) ? voff_odd : voff_even) + (uint32_t)j * step8;
+    if (RAGGED_M && op == 0) {
+      const uint32_t row = min((uint32_t)(wave * (BM / 4) + j * 8) + (uint32_t)(lane >> 3), (uint32_t)(lp.valid - 1));
+      voff = row * (uint32_t)p.k + (((j & 1) ? voff_odd : voff_even) - row_off);
+    }
     if (RAGGED_K && l_ks == nk - 1) {
-      if ((j & 1) ? tail_odd : tail_even) lds_dma16(l, gp, ((j & 1) ? voff_odd : voff_even) + (uint32_t)j * step8);
+      if ((j & 1) ? tail_odd : tail_even) lds_dma16(l, gp, voff);
       else *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(lds) + (l - lds_base) + lane * 16) = u32x4{0, 0, 0, 0};
       return;
     }
-    if (RAGGED_M && op == 0) {
-      const uint32_t row = min((uint32_t)(wave * (BM / 4) + j * 8) + (uint32_t)(lane >> 3), (uint32_t)(lp.valid - 1));
-      lds_dma16(l, gp, row * (uint32_t)p.k + (((j & 1) ? voff_odd : voff_even) - row_off));
-      return;
-    }
-    lds_dma16(l, gp, ((j & 1) ? voff_odd : voff_even) + (uint32_t)j * step8);
+    lds_dma16(l, gp, voff);
   };
   // After the 16 units: the step's scale loads, then advance the stream (selects only).
   auto issue_step_tail = [&]() {
@@ -568,6 +567,8 @@ int launch_fast(const Params& p, hipStream_t stream) {
   // operand panels out of it (and out of the L2s) on its way to memory, so it leaves with non-temporal stores
   // (8192^3: +5 %, 16384 x 16384 x 2048: +17 %; smaller problems lose 1-5 % that way).
   const bool stream_out = ((int64_t)p.m + p.n) * p.k + 2 * (int64_t)p.m * p.n > (int64_t)224 << 20;
+  if (p.m % (64 * TM) != 0 && (p.k & 127) != 0)
+    return stream_out ? launch_fast_cfg<TM, OUT_BF16, true, true, true>(p, stream) : launch_fast_cfg<TM, OUT_BF16, false, true, true>(p, stream);
   if (p.m % (64 * TM) != 0) return stream_out ? launch_fast_cfg<TM, OUT_BF16, true, false, true>(p, stream) : launch_fast_cfg<TM, OUT_BF16, false, false, true>(p, stream);
   if ((p.k & 127) != 0) return stream_out ? launch_fast_cfg<TM, OUT_BF16, true, true>(p, stream) : launch_fast_cfg<TM, OUT_BF16, false, true>(p, stream);
   return stream_out ? launch_fast_cfg<TM, OUT_BF16, true, false>(p, stream) : launch_fast_cfg<TM, OUT_BF16, false, false>(p, stream);
@@ -881,11 +882,11 @@ Plan mxfp8_plan(int64_t m, int64_t n, int64_t k, int64_t cus, int64_t* ns = null
   if (ns) *ns = INT64_MAX;
   const bool skinny_ok = (k & 31) == 0 && (n & 15) == 0 && k * 64 < (1ll << 31);  // 32-bit lane offsets (a short last chunk is fine)
   // (the persistent kernel takes any K % 32 == 0: its last step may be short)
-  // (a last row tile with fewer rows: the variant that clamps the rows of its activation loads, K % 128 == 0 only;
-  // the tile counts as a whole one.  640 x 14336 x 4096: 280 tiles of 128 rows in 2 rounds 60 us, 168 of 256 rows 43 us)
+  // (a last row tile with fewer rows: the variant that clamps the rows of its activation loads; the tile counts as a
+  // whole one.  640 x 14336 x 4096: 280 tiles of 128 rows in 2 rounds 60 us, 168 of 256 rows 43 us)
   const bool fast_shape = (k & 31) == 0 && k >= 256 && (n & 255) == 0 && k * 256 < (1ll << 31);
-  const bool ok256 = fast_shape && ((m & 255) == 0 || ((k & 127) == 0 && m > 128));
-  const bool ok128 = fast_shape && ((m & 127) == 0 || ((k & 127) == 0 && m > 64));
+  const bool ok256 = fast_shape && ((m & 255) == 0 || m > 128);
+  const bool ok128 = fast_shape && ((m & 127) == 0 || m > 64);
   const int64_t t256 = ok256 ? ceil_div(m, 256) * (n / 256) : 0, t128 = ok128 ? ceil_div(m, 128) * (n / 256) : 0;
   const int64_t cost256 = t256 >= 128 ? 100 * ceil_div(t256, cus) : INT64_MAX;
   const int64_t cost128 = t128 >= 48 ? 61 * ceil_div(t128, cus) : INT64_MAX;

@@ -291,8 +291,8 @@ def test_nvfp4_gemm_many_rows_small_n_deep_k(dev, shape):
                                    (2100, 4096, 2080), (2504, 2048, 2144), (1000, 14336, 2080), (4300, 2048, 2080)])
 def test_dense_gemms_with_m_not_a_multiple_of_128(dev, shape):
     """A prefill of any token count, M > 128 and not a multiple of 128.  K % 128 == 0: one launch of the persistent
-    kernel whose last row tile holds fewer rows.  K % 128 != 0 (the last four shapes; that variant of the kernel wants
-    whole row tiles): cut at a multiple of 128 or 256; the rows before the cut go to the persistent kernel, the 1..255
+    kernel whose last row tile holds fewer rows.  K % 128 != 0 (the last four shapes): MXFP8 the same with a short last
+    K step as well; NVFP4 (that variant of its kernel wants whole row tiles) cut at a multiple of 128 or 256; the rows before the cut go to the persistent kernel, the 1..255
     rows after it to the weight-streaming kernel in a launch of its own, which reads its activation scales a whole
     number of 128-row scale tiles further on.  Both ops, both output types, every element against the oracle, poisoned
     scale padding, rows of the two launches next to the cut compared like all others, run-to-run bit equality."""
@@ -328,8 +328,8 @@ def test_dense_gemms_with_m_not_a_multiple_of_128(dev, shape):
         assert out.shape == (m, n)
         assert ((out.float().cpu() - ref).abs() / scale).max().item() <= GEMM_MAX_REL, (shape, dtype, plans[-1])
         assert torch.equal(out, _run_mxfp8(a8, b8, sa8_p, sb8, 0.75, dtype, dev))
-    if k % 128 != 0:
-        assert all("; " in p and "ragged_k" in p for p in plans), plans
+    if k % 128 != 0:  # NVFP4: the cut; MXFP8: one launch of the variant with a short last K step and a short last row tile
+        assert "; " in plans[0] and "ragged_k" in plans[0] and "ragged_k,ragged_m" in plans[1] and "; " not in plans[1], plans
     elif shape != (1000, 2048, 256):  # (too few tiles for the persistent kernel)
         assert all("ragged_m" in p and "; " not in p for p in plans), plans
 
@@ -802,13 +802,15 @@ def test_mxfp8_gemm_persistent_256_tile_kernel_full_compare(dev, shape):
 
 
 @pytest.mark.parametrize("shape", [(300, 14336, 512), (136, 12288, 512), (80, 28672, 256), (520, 14336, 512), (640, 14336, 1024),
-                                   (700, 12288, 256), (2049, 4096, 512), (390, 8192, 1280), (200, 65536, 256), (130, 65536, 256)])
+                                   (700, 12288, 256), (2049, 4096, 512), (390, 8192, 1280), (200, 65536, 256), (130, 65536, 256),
+                                   (300, 14336, 352), (520, 14336, 288), (700, 12288, 320), (1000, 5632, 2880)])
 def test_mxfp8_gemm_last_row_tile_with_fewer_rows_on_the_persistent_kernel(dev, shape):
     """M no multiple of the tile height, N % 256 == K % 128 == 0 and enough tiles: the persistent kernel's variant whose
     last row tile clamps the rows of its activation loads and stores only the rows that exist.  128-row tiles with 44,
     8 and 80 rows in the last one (one tile row in all for the 80), 256-row tiles with 8 rows (the tile's second scale
     tile does not exist: the last one is read instead), 128 (M % 256 == 128), 188 and 1 row, and a single 256-row tile row
-    with 200 and 130 rows; two to ten K steps.  NaN
+    with 200 and 130 rows; two to ten K steps; the last four shapes with a short last K step as well (K % 128 = 96, 32,
+    64, 64).  NaN
     code in every scale byte of the padding rows, both output types, every element compared, rows are written once
     (a result buffer pre-filled with a pattern keeps it past row M), run-to-run determinism."""
     from fuser_amd import capi
