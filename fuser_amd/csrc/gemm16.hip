@@ -66,6 +66,8 @@ struct Params {
   // layout of [roundUp(m,128), roundUp(n/16,4)], gnorm = the result's global (encode) scale on the device
   uint8_t* out_sf = nullptr;
   const float* gnorm = nullptr;
+  // dense weight-streaming kernel: 0 = 16-bit result, 1 = the block-scaled result above, 2 = the fp32 product itself
+  int stream_result = 0;
   // dense NVFP4 with a 16-bit result: elements between rows of the result; 0: n (a launch that computes some of the
   // columns sets it)
   int ldc = 0;
@@ -527,8 +529,20 @@ int launch_nvfp4_wide(const Params& p, int cus, hipStream_t stream) {
 template <bool FP4>
 int launch_nvfp4_wide_part(const Params& p, int cus, hipStream_t stream) {
   auto tiles = [&](int bm, int bn) { return ceil_div(p.m, bm) * ceil_div(p.n, bn); };
+  // Decode-sized and other shapes that the 16-bit op streams: the same kernel, whose last stage then quantizes the
+  // summed product (or stores it as it is) instead of rounding it to 16 bits (16 x 4096 x 4096: 28 -> 6 us, 128 x 4096 x
+  // 14336: 85 -> 24 us on the tile kernels before).
+  if ((p.k & 127) == 0 && nvfp4_dense_plan(p.m, p.n, p.k, cus).kernel == DensePlan::kStream) {
+    Params q = p;
+    q.stream_result = FP4 ? 1 : 2;
+    return launch_nvfp4_skinny<true>(q, cus, stream);
+  }
   if ((p.n & 255) == 0 && (p.k & 127) == 0 && p.k >= 256) {
     // as for the 16-bit results: persistent 256x256 or 128x256 tiles where they fill the compute units
+    const DensePlan::Kernel like16 = nvfp4_dense_plan(p.m, p.n, p.k, cus).kernel;
+    if (like16 == DensePlan::kTiles256 && (p.m & 255) == 0) return launch_nvfp4_fast<false, false, 4, !FP4, FP4>(p, cus, stream);
+    if ((like16 == DensePlan::kTiles256 || like16 == DensePlan::kTiles128) && (p.m & 127) == 0)
+      return launch_nvfp4_fast<false, false, 2, !FP4, FP4>(p, cus, stream);
     const int64_t t256 = (p.m & 255) == 0 ? tiles(256, 256) : 0, t128 = (p.m & 127) == 0 ? tiles(128, 256) : 0;
     const int64_t cost256 = t256 ? 100 * ceil_div(t256, cus) : INT64_MAX;
     const int64_t cost128 = t128 ? 58 * ceil_div(t128, cus) : INT64_MAX;

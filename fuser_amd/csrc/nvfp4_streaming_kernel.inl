@@ -272,11 +272,40 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
 #pragma unroll
         for (int w = 1; w < W; ++w) s += red[w * units + u];
         const int tok = tt * 16 + (l & 15);
+        if (!GROUPED && p.stream_result == 1) {
+          // Block-scaled result: the quantizer's arithmetic (runtime/block_quantization_kernels.cu:224-263) on alpha *
+          // sum.  The 16 columns of a row's block are this lane's four and those of the lanes 16, 32 and 48 further on.
+          const float gs = p.gnorm[0], decode = 1.0f / gs;
+          const float x0 = s[0] * alpha, x1 = s[1] * alpha, x2 = s[2] * alpha, x3 = s[3] * alpha;
+          float amax = fmaxf(fmaxf(fmaxf(fmaxf(-INFINITY, fabsf(x0)), fabsf(x1)), fabsf(x2)), fabsf(x3));  // NaN ignored
+          const bool nonfinite = !(fabsf(x0) < INFINITY) || !(fabsf(x1) < INFINITY) || !(fabsf(x2) < INFINITY) || !(fabsf(x3) < INFINITY);
+          amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
+          amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+          float rr;
+          const uint32_t q8 = nvfp4_block_scale(amax, true, gs, decode, tok < m_loc, rr);
+          uint32_t w = 0;
+          if (__builtin_amdgcn_ballot_w64(nonfinite) == 0) {
+            w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, x0 * rr, x1 * rr, 1.0f, 0);
+            w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, x2 * rr, x3 * rr, 1.0f, 1);
+          } else {  // explicit NaN rule of the narrow cast
+            w = f32x2_to_e2m1_byte(x0 * rr, x1 * rr) | (f32x2_to_e2m1_byte(x2 * rr, x3 * rr) << 8);
+          }
+          if (tok < m_loc) {
+            const int col4 = n0 + (round * RPR + r2) * 16 + 4 * (l >> 4);
+            *reinterpret_cast<uint16_t*>(static_cast<uint8_t*>(p.out) + (a_row0 + tok) * (int64_t)(p.n >> 1) + (col4 >> 1)) = (uint16_t)w;
+            if ((l >> 4) == 0) p.out_sf[swizzle_128x4(a_row0 + tok, col4 >> 4, (((int64_t)p.n >> 4) + 3) & ~(int64_t)3)] = (uint8_t)q8;
+          }
+        }
         if (tok < m_loc) {
           const int col = n0 + (round * RPR + r2) * 16 + 4 * (l >> 4);
           const int64_t at = (a_row0 + tok) * p.out_pitch() + col;
           if (!GROUPED && p.partial != nullptr) {  // this K range's sums as they are; the reduction applies alpha
             *reinterpret_cast<f32x4*>(p.partial + ((int64_t)blockIdx.z * p.m + a_row0 + tok) * p.n + col) = s;
+          } else if (!GROUPED && p.stream_result == 2) {  // the fp32 product
+            *reinterpret_cast<f32x4*>(static_cast<float*>(p.out) + (a_row0 + tok) * (int64_t)p.n + col) =
+                f32x4{s[0] * alpha, s[1] * alpha, s[2] * alpha, s[3] * alpha};
+          } else if (!GROUPED && p.stream_result == 1) {
+            // (block-scaled result: stored below, outside the test for the row - its shuffles need the whole wavefront)
           } else {
             u32x2 v;
             v[0] = pack2(s[0] * alpha, s[1] * alpha, OUT_BF16);

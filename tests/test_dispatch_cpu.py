@@ -221,7 +221,14 @@ def test_blockscale_is_one_launch_and_ragged_shapes_add_only_the_fill_kernel():
     got = plan("nvfp4_scaled_mm_blockscale", 8192, 8192, 8192)
     assert got.startswith("nvfp4_gemm_256_kernel<") and "fp4_blockscale" in got and ";" not in got, got
     ragged = plan("nvfp4_scaled_mm_blockscale", 200, 160, 512).split("; ")
+    assert len(ragged) == 2 and ragged[0].startswith("zero_fill_kernel") and ragged[1].startswith("nvfp4_skinny_ring_kernel<"), ragged
+    ragged = plan("nvfp4_scaled_mm_blockscale", 600, 160, 512).split("; ")
     assert len(ragged) == 2 and ragged[0].startswith("zero_fill_kernel") and ragged[1].startswith("nvfp4_tile_kernel<"), ragged
+    # decode-sized calls stream the weights like the 16-bit op (one launch; the dump a second run of that kernel)
+    got = plan("nvfp4_scaled_mm_blockscale", 128, 14336, 4096)
+    assert got == plan("nvfp4_scaled_mm", 128, 14336, 4096) and got.startswith("nvfp4_skinny_ring_kernel<RT=4,TT=8>"), got
+    dump = plan("nvfp4_scaled_mm_blockscale", 128, 14336, 4096, ws=4 * 128 * 14336).split("; ")
+    assert len(dump) == 2 and dump[0] == dump[1], dump
     # the optional dump of the fp32 product is a second run of the same kernel
     dump = plan("nvfp4_scaled_mm_blockscale", 8192, 8192, 8192, ws=4 * 8192 * 8192).split("; ")
     assert len(dump) == 2 and "fp4_blockscale" in dump[0] and "f32=1" in dump[1], dump

@@ -83,14 +83,18 @@ def test_nvfp4_gemm_epilogue_reference_shapes(dev, dtype, shape):
 
 
 @pytest.mark.parametrize("shape", [(200, 160, 192), (4096, 3072, 256), (1920, 4096, 384), (1024, 2048, 384), (300, 544, 608), (64, 96, 64),
-                                   (2176, 2048, 256), (4096, 4128, 128), (2100, 4096, 256), (4000 + 77, 2048, 384)])
+                                   (2176, 2048, 256), (4096, 4128, 128), (2100, 4096, 256), (4000 + 77, 2048, 384),
+                                   (16, 4096, 512), (100, 14336, 256), (128, 2048, 1024), (300, 4096, 2048), (48, 1056, 384), (1000, 14336, 256)])
 def test_nvfp4_gemm_epilogue_quantizes_its_own_fp32_product_bit_exactly(dev, shape):
     """Through the C ABI.  The result is quantized in the GEMM's epilogue; with a workspace the call also dumps the
     fp32 product it quantized: that agrees with the oracle product to fp32 summation noise, and payload and scales
     are bit-identical to the oracle quantizer applied to exactly that product (rows not a multiple of 128 and
     padded scale columns on the 64x64, 128x128 and 256x256 tile kernels; shapes on the persistent kernel with
     256x256 and with 128x256 tiles; the last two: M not a multiple of 128, cut into a part for the persistent kernel
-    and the remaining rows for the tile kernels, whose payload and scale tiles follow the first part's)."""
+    and the remaining rows for the tile kernels, whose payload and scale tiles follow the first part's; the last six:
+    shapes that the 16-bit op streams - one to eight activation row tiles, one to four weight tiles per workgroup, one
+    and several slabs, and 104 rows streamed behind 896 on the persistent kernel - where the weight-streaming kernel's
+    last stage quantizes the summed product)."""
     from fuser_amd import capi
 
     m, n, k = shape
