@@ -362,11 +362,11 @@ int launch_sized(const Params& p, int64_t m_hint, int cus, void* workspace, int6
   auto tiles = [&](int bm, int bn) { return ceil_div(m_hint, bm) * ceil_div(p.n, bn); };
   const bool dense = p.problem_sizes == nullptr;
   // grouped NVFP4: does the call count as a prefill (see kPrefillRows)?  Also with fewer rows where the large groups'
-  // launches find a round of 256x256 tiles - with 128 rows per group on average, or two rounds whatever the groups
+  // launches find (nearly) a round of 256x256 tiles - with 128 rows per group on average, or two rounds whatever the groups
   // (8 experts, 1536 rows, N=14336, K=4096: 320 -> 223 us; 16 experts, 3072 rows: 540 -> 394; 128 experts, 5632 rows,
   // N=7168, K=2048: 460 -> 336; at 96 rows per group and one round the other launches stay faster: 125 against 167 us)
   const int64_t tiles256 = (m_hint / 256) * (p.n / 256);
-  const bool is_prefill = m_hint >= kPrefillRows || (tiles256 >= cus && m_hint >= 128 * (int64_t)p.groups) || tiles256 >= 2 * (int64_t)cus;
+  const bool is_prefill = m_hint >= kPrefillRows || (8 * tiles256 >= 7 * (int64_t)cus && m_hint >= 128 * (int64_t)p.groups) || tiles256 >= 2 * (int64_t)cus;
   if constexpr (NVFP4) {
     if (dense && workspace != nullptr) {
       const int skinny_splits = nvfp4_skinny_splits(p.m, p.n, p.k, cus);
