@@ -68,6 +68,8 @@ struct Params {
   const float* gnorm = nullptr;
   // dense weight-streaming kernel: 0 = 16-bit result, 1 = the block-scaled result above, 2 = the fp32 product itself
   int stream_result = 0;
+  // ... with stream_result 1: the kernel also zeroes the padding rows and columns of the scale buffer's last 128x4 tiles
+  int stream_zero_pad = 0;
   // dense NVFP4 with a 16-bit result: elements between rows of the result; 0: n (a launch that computes some of the
   // columns sets it)
   int ldc = 0;
@@ -501,7 +503,11 @@ int launch_nvfp4_wide_part(const Params& p, int cus, hipStream_t stream);
 
 template <bool FP4>
 int launch_nvfp4_wide(const Params& p, int cus, hipStream_t stream) {
-  if (FP4 && ((p.m & 127) != 0 || ((p.n >> 4) & 3) != 0)) {
+  const bool cut_m = (p.n & 255) == 0 && (p.k & 127) == 0 && p.k >= 256 && p.m > 256 && (p.m & 127) != 0 &&
+                     ceil_div(p.m / 128 * 128, 128) * (p.n / 256) >= cus / 2;
+  // (a call that the weight-streaming kernel takes whole zeroes that padding itself: no launch for it at decode sizes)
+  const bool streams_whole = !cut_m && (p.k & 127) == 0 && nvfp4_dense_plan(p.m, p.n, p.k, cus).kernel == DensePlan::kStream;
+  if (FP4 && !streams_whole && ((p.m & 127) != 0 || ((p.n >> 4) & 3) != 0)) {
     // ragged: the padding rows / columns of the scale buffer's last 128x4 tiles are written as zero first
     const int64_t words = round_up(p.m, 128) * round_up(p.n >> 4, 4) / 4;
     if (!note_launch("zero_fill_kernel grid=%lld", (long long)ceil_div(words, 256))) {
@@ -509,7 +515,7 @@ int launch_nvfp4_wide(const Params& p, int cus, hipStream_t stream) {
       if (const int rc = check_launch("zero_fill_kernel")) return rc;
     }
   }
-  if ((p.n & 255) == 0 && (p.k & 127) == 0 && p.k >= 256 && p.m > 256 && (p.m & 127) != 0 && ceil_div(p.m / 128 * 128, 128) * (p.n / 256) >= cus / 2) {
+  if (cut_m) {
     // M not a multiple of 128 and enough rows for the persistent kernel: the rows up to the last multiple of 128 go
     // there, the rest to the tile kernels (their part of the result and of its scale tiles starts a whole number of
     // 128-row tiles further on)
@@ -522,6 +528,11 @@ int launch_nvfp4_wide(const Params& p, int cus, hipStream_t stream) {
     if (FP4) rest.out_sf = p.out_sf + (int64_t)main.m * round_up(p.n >> 4, 4);
     if (const int rc = launch_nvfp4_wide_part<FP4>(main, cus, stream)) return rc;
     return launch_nvfp4_wide_part<FP4>(rest, cus, stream);
+  }
+  if (FP4 && streams_whole) {
+    Params q = p;
+    q.stream_zero_pad = 1;
+    return launch_nvfp4_wide_part<FP4>(q, cus, stream);
   }
   return launch_nvfp4_wide_part<FP4>(p, cus, stream);
 }

@@ -315,6 +315,18 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
         }
       }
     }
+    if (!GROUPED && p.stream_result == 1 && p.stream_zero_pad != 0 && blockIdx.y == gridDim.y - 1) {
+      // block-scaled result: the padding of the scale buffer's last 128x4 tiles is zero - the rows past M (this
+      // workgroup's scale columns; the last slab's workgroups) and the columns past N / 16 (the last workgroup)
+      const int64_t sf_cols = (int64_t)p.n >> 4, padded = (sf_cols + 3) & ~(int64_t)3;
+      const int m_pad = (p.m + 127) & ~127;
+      for (int i = tid; i < (m_pad - p.m) * RT; i += 512)
+        p.out_sf[swizzle_128x4(p.m + i / RT, (n0 >> 4) + i % RT, padded)] = 0;
+      if (blockIdx.x == gridDim.x - 1 && padded != sf_cols) {
+        const int pc = (int)(padded - sf_cols);
+        for (int i = tid; i < m_pad * pc; i += 512) p.out_sf[swizzle_128x4(i / pc, sf_cols + i % pc, padded)] = 0;
+      }
+    }
   };
 
   constexpr int CSTEP = NSPLIT ? 1 : W;  // distance of a wavefront's consecutive chunks
