@@ -503,11 +503,14 @@ int launch_nvfp4_wide_part(const Params& p, int cus, hipStream_t stream);
 
 template <bool FP4>
 int launch_nvfp4_wide(const Params& p, int cus, hipStream_t stream) {
-  const bool cut_m = (p.n & 255) == 0 && (p.k & 127) == 0 && p.k >= 256 && p.m > 256 && (p.m & 127) != 0 &&
+  // A call that one launch of the weight-streaming kernel or of the persistent kernel (whose last row tile may hold
+  // fewer rows) takes whole leaves that padding zero itself: no launch for it.
+  const DensePlan::Kernel like16 = (p.k & 127) == 0 ? nvfp4_dense_plan(p.m, p.n, p.k, cus).kernel : DensePlan::kOther;
+  const bool one_launch = like16 == DensePlan::kStream || like16 == DensePlan::kTiles256 || like16 == DensePlan::kTiles128;
+  const bool cut_m = !one_launch && (p.n & 255) == 0 && (p.k & 127) == 0 && p.k >= 256 && p.m > 256 && (p.m & 127) != 0 &&
                      ceil_div(p.m / 128 * 128, 128) * (p.n / 256) >= cus / 2;
-  // (a call that the weight-streaming kernel takes whole zeroes that padding itself: no launch for it at decode sizes)
-  const bool streams_whole = !cut_m && (p.k & 127) == 0 && nvfp4_dense_plan(p.m, p.n, p.k, cus).kernel == DensePlan::kStream;
-  if (FP4 && !streams_whole && ((p.m & 127) != 0 || ((p.n >> 4) & 3) != 0)) {
+  const bool streams_whole = like16 == DensePlan::kStream;
+  if (FP4 && !one_launch && ((p.m & 127) != 0 || ((p.n >> 4) & 3) != 0)) {
     // ragged: the padding rows / columns of the scale buffer's last 128x4 tiles are written as zero first
     const int64_t words = round_up(p.m, 128) * round_up(p.n >> 4, 4) / 4;
     if (!note_launch("zero_fill_kernel grid=%lld", (long long)ceil_div(words, 256))) {
@@ -551,9 +554,8 @@ int launch_nvfp4_wide_part(const Params& p, int cus, hipStream_t stream) {
   if ((p.n & 255) == 0 && (p.k & 127) == 0 && p.k >= 256) {
     // as for the 16-bit results: persistent 256x256 or 128x256 tiles where they fill the compute units
     const DensePlan::Kernel like16 = nvfp4_dense_plan(p.m, p.n, p.k, cus).kernel;
-    if (like16 == DensePlan::kTiles256 && (p.m & 255) == 0) return launch_nvfp4_fast<false, false, 4, !FP4, FP4>(p, cus, stream);
-    if ((like16 == DensePlan::kTiles256 || like16 == DensePlan::kTiles128) && (p.m & 127) == 0)
-      return launch_nvfp4_fast<false, false, 2, !FP4, FP4>(p, cus, stream);
+    if (like16 == DensePlan::kTiles256) return launch_nvfp4_fast<false, false, 4, !FP4, FP4>(p, cus, stream);
+    if (like16 == DensePlan::kTiles128) return launch_nvfp4_fast<false, false, 2, !FP4, FP4>(p, cus, stream);
     const int64_t t256 = (p.m & 255) == 0 ? tiles(256, 256) : 0, t128 = (p.m & 127) == 0 ? tiles(128, 256) : 0;
     const int64_t cost256 = t256 ? 100 * ceil_div(t256, cus) : INT64_MAX;
     const int64_t cost128 = t128 ? 58 * ceil_div(t128, cus) : INT64_MAX;

@@ -31,14 +31,14 @@
 // RAGGED_K (16-bit result; grouped: the 256x256 tiles): K % 128 = 32, 64 or 96.  A tile's last span is short: the threads whose 32 elements lie
 // past K fetch their row's first piece instead of the next row's bytes, and their scale load runs past the range of its
 // buffer resource on purpose, which makes it return zero - and a zero scale makes a block count as zero.
-// RAGGED_M (dense, 16-bit result): the last row tile holds fewer than BM rows.  As for the last tile of a group, the
+// RAGGED_M (dense): the last row tile holds fewer than BM rows.  As for the last tile of a group, the
 // buffer range of the activations ends with the last row, so the rows past it read as zero, and they are not stored;
 // the scale tile of a 256-row tile's second half may not exist and then reads as zero the same way.
 template <bool OUT_BF16, bool GROUPED, int TM = 4, bool OUT_F32 = false, bool PAIRS = false, bool OUT_FP4 = false, bool RAGGED_K = false,
           bool RAGGED_M = false>
 __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
   static_assert(TM == 4 || TM == 2, "tile height");
-  static_assert(!RAGGED_M || (!GROUPED && !OUT_F32 && !OUT_FP4), "a short last row tile: dense calls with a 16-bit result");
+  static_assert(!RAGGED_M || !GROUPED, "a short last row tile: dense calls (the groups' tiles are always of that kind)");
   constexpr bool PARTIAL = GROUPED || RAGGED_M;  // tiles may hold fewer rows than BM
   constexpr int BM = 64 * TM, BN = 256;
   constexpr int A_UNITS = BM * 8;            // 16-byte units of the A tile (fp16, 64 of K per row)
@@ -452,10 +452,12 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
         }
         asm volatile("" ::: "memory");  // the read below sees the writes above: one wavefront's LDS accesses stay in order
         const u32x4 v = *reinterpret_cast<const u32x4*>(rd);
-        *reinterpret_cast<u32x4*>(obase + (int64_t)(i * 32) * opitch) = v;
+        if (!RAGGED_M || wm * (32 * TM) + i * 32 + (elane >> 1) < cw.valid) *reinterpret_cast<u32x4*>(obase + (int64_t)(i * 32) * opitch) = v;
         asm volatile("" ::: "memory");
       }
-      if (lg == 0) {
+      // (RAGGED_M: the rows past M read as zero, so their scale codes are zero - exactly what the padding rows of the
+      // last 128-row scale tile must hold; a 256-row tile with at most 128 rows has no second scale tile to write)
+      if (lg == 0 && (!RAGGED_M || TM == 2 || wm * 128 < cw.valid)) {
         const int sf_cols4 = p.n >> 6;  // 512-byte scale tiles per 128 rows (N % 256 == 0: no padding columns)
         uint8_t* sfp = p.out_sf + ((cw.m0 >> 7) * (int64_t)sf_cols4 + ((cw.n0 + wn * 64) >> 6)) * 512 + li * 16;
         if constexpr (TM == 4) *reinterpret_cast<u32x4*>(sfp + (int64_t)wm * sf_cols4 * 512) = u32x4{sfw[0], sfw[1], sfw[2], sfw[3]};
@@ -485,7 +487,8 @@ __global__ __launch_bounds__(512) void nvfp4_gemm_256_kernel(const Params p) {
 #pragma unroll
           for (int t = 0; t < 2; ++t) {
             const f32x4 v = *reinterpret_cast<const f32x4*>(rd + t * 1280);
-            *reinterpret_cast<f32x4*>(obase + ((int64_t)(i * 32 + 16 * t) * p.n + jh * 16) * 4 + ooff) = v;
+            if (!RAGGED_M || wm * (32 * TM) + i * 32 + 16 * t + (elane >> 2) < cw.valid)
+              *reinterpret_cast<f32x4*>(obase + ((int64_t)(i * 32 + 16 * t) * p.n + jh * 16) * 4 + ooff) = v;
           }
           asm volatile("" ::: "memory");
         }
@@ -545,8 +548,9 @@ int launch_nvfp4_fast_cfg(const Params& p, int cus, hipStream_t stream) {
   const int64_t tiles = tiles_m * (p.n / 256);
   const unsigned grid = (unsigned)(tiles >= cus ? (cus & ~7) : ((tiles + 7) / 8) * 8);
   if (grid == 0) return NVF_OK;  // fewer rows in the whole call than the smallest group this launch serves: no work
-  if (note_launch("nvfp4_gemm_256_kernel<grouped=%d,TM=%d,f32=%d,pairs=%d%s%s> grid=%u rows=%d..%d min_rows=%d", (int)GROUPED, TM, (int)OUT_F32,
-                  (int)PAIRS, OUT_FP4 ? ",fp4_blockscale" : (RAGGED_M ? ",ragged_m" : ""), RAGGED_K ? ",ragged_k" : "", grid, p.rows_lo, p.rows_hi, p.min_rows))
+  if (note_launch("nvfp4_gemm_256_kernel<grouped=%d,TM=%d,f32=%d,pairs=%d%s%s%s> grid=%u rows=%d..%d min_rows=%d", (int)GROUPED, TM, (int)OUT_F32,
+                  (int)PAIRS, OUT_FP4 ? ",fp4_blockscale" : "", RAGGED_M ? ",ragged_m" : "", RAGGED_K ? ",ragged_k" : "", grid, p.rows_lo, p.rows_hi,
+                  p.min_rows))
     return NVF_OK;
   static std::atomic<uint64_t> configured{0};  // one bit per device
   if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured)) return rc;
@@ -563,7 +567,7 @@ int launch_nvfp4_fast(const Params& p, int cus, hipStream_t stream) {
       return launch_nvfp4_fast_cfg<OUT_BF16, GROUPED, TM, OUT_F32, false, OUT_FP4, true>(p, cus, stream);
     }
   }
-  if constexpr (!GROUPED && !OUT_F32 && !OUT_FP4) {
+  if constexpr (!GROUPED) {
     if (p.m % (64 * TM) != 0) {  // a last row tile with fewer rows
       if (((p.k >> 7) & 1) == 0) return launch_nvfp4_fast_cfg<OUT_BF16, GROUPED, TM, OUT_F32, true, OUT_FP4, false, true>(p, cus, stream);
       return launch_nvfp4_fast_cfg<OUT_BF16, GROUPED, TM, OUT_F32, false, OUT_FP4, false, true>(p, cus, stream);

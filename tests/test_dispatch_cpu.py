@@ -225,6 +225,9 @@ def test_blockscale_is_one_launch_and_ragged_shapes_add_only_the_fill_kernel():
     assert ragged.startswith("nvfp4_skinny_ring_kernel<") and ";" not in ragged, ragged
     ragged = plan("nvfp4_scaled_mm_blockscale", 600, 160, 512).split("; ")
     assert len(ragged) == 2 and ragged[0].startswith("zero_fill_kernel") and ragged[1].startswith("nvfp4_tile_kernel<"), ragged
+    # M no multiple of the tile height: one launch of the persistent kernel's variant with a short last row tile
+    got = plan("nvfp4_scaled_mm_blockscale", 1000, 14336, 4096)
+    assert got.startswith("nvfp4_gemm_256_kernel<grouped=0,TM=4,") and "fp4_blockscale,ragged_m" in got and ";" not in got, got
     # decode-sized calls stream the weights like the 16-bit op (one launch; the dump a second run of that kernel)
     got = plan("nvfp4_scaled_mm_blockscale", 128, 14336, 4096)
     assert got == plan("nvfp4_scaled_mm", 128, 14336, 4096) and got.startswith("nvfp4_skinny_ring_kernel<RT=4,TT=8>"), got
