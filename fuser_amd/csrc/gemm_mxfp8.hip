@@ -579,8 +579,8 @@ int launch_fast(const Params& p, hipStream_t stream) {
 // whole ones side by side in one launch, blockIdx.y = slab), K % 32 == 0, N % (16*RT) == 0.  A slab streams
 // the weight matrix exactly once, so the op is bound by HBM (by the last-level cache for the slabs after the
 // first):
-//   * A workgroup owns 16*RT weight rows for the whole of K and all M activation rows; its 8 wavefronts
-//     split K in interleaved 128-element chunks and their partial sums are added in a fixed order through
+//   * A workgroup owns 16*RT weight rows for the whole of K and all M activation rows; its W = 8 wavefronts
+//     (4 in the form of which two workgroups share a compute unit) split K in interleaved 128-element chunks and their partial sums are added in a fixed order through
 //     LDS (no atomics, no workspace, deterministic).
 //   * v_mfma_scale_f32_16x16x128_f8f6f4, measured operand layout: lane (i, g) = i + 16 g supplies row i,
 //     bytes 0..15 = K [16g, 16g+16) and bytes 16..31 = K [64+16g, 64+16g+16); the scale byte of lane
@@ -596,9 +596,8 @@ int launch_fast(const Params& p, hipStream_t stream) {
 // -------------------------------------------------------------------------------------------------
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-template <int RT, int TT, bool OUT_BF16, int DEPTH, bool RAGGED_K = false>
-__global__ __launch_bounds__(512) void mxfp8_skinny_kernel(const Params p) {
-  constexpr int W = 8;
+template <int RT, int TT, bool OUT_BF16, int DEPTH, bool RAGGED_K = false, int W = 8>
+__global__ __launch_bounds__(W * 64) void mxfp8_skinny_kernel(const Params p) {
   constexpr int NT = RT + TT;
   // activation rows r and r + 32 share their 16-byte scale group, so 32 groups serve any number of tiles
   constexpr int A_SC_BYTES = (TT < 2 ? TT : 2) * 256;
@@ -752,7 +751,7 @@ __global__ __launch_bounds__(512) void mxfp8_skinny_kernel(const Params p) {
     for (int tt = 0; tt < TT; ++tt)
       if (tt < tt_count) red[(wave * tiles + rt * tt_count + tt) * 64 + lane] = acc[rt][tt];
   __syncthreads();
-  for (int u = tid; u < units; u += 512) {
+  for (int u = tid; u < units; u += W * 64) {
     const int l = u & 63, tile = u >> 6;
     const int rt = tile / tt_count, tt = tile - rt * tt_count;
     f32x4 s = red[u];
@@ -769,18 +768,20 @@ __global__ __launch_bounds__(512) void mxfp8_skinny_kernel(const Params p) {
   }
 }
 
-template <int RT, int TT, bool OUT_BF16>
+template <int RT, int TT, bool OUT_BF16, int W = 8>
 int launch_skinny_cfg(const Params& p, hipStream_t stream, int slabs = 1) {
   constexpr int SLOT = (RT + TT) * 2048 + RT * 256 + (TT < 2 ? TT : 2) * 256;
-  constexpr int DEPTH = 8 * 3 * SLOT <= 160 * 1024 ? 3 : (8 * 2 * SLOT <= 160 * 1024 ? 2 : 1);
-  auto kern = (p.k & 127) != 0 ? mxfp8_skinny_kernel<RT, TT, OUT_BF16, DEPTH, true> : mxfp8_skinny_kernel<RT, TT, OUT_BF16, DEPTH>;
-  constexpr int ring = 8 * DEPTH * SLOT, red = 8 * RT * TT * 1024;
+  constexpr int DEPTH = W != 8 ? 1 : 8 * 3 * SLOT <= 160 * 1024 ? 3 : (8 * 2 * SLOT <= 160 * 1024 ? 2 : 1);
+  // (4 wavefronts: K % 128 == 0 only, and a ring of one slot, so that two workgroups share a compute unit's LDS)
+  if (W != 8 && (p.k & 127) != 0) return fail(NVF_ERR_UNSUPPORTED_SHAPE, "mxfp8_skinny_kernel: 4 wavefronts need K % 128 == 0");
+  auto kern = W == 8 && (p.k & 127) != 0 ? mxfp8_skinny_kernel<RT, TT, OUT_BF16, DEPTH, W == 8, W> : mxfp8_skinny_kernel<RT, TT, OUT_BF16, DEPTH, false, W>;
+  constexpr int ring = W * DEPTH * SLOT, red = W * RT * TT * 1024;
   constexpr int lds_bytes = ring > red ? ring : red;
   static_assert(lds_bytes <= 160 * 1024, "LDS");
-  if (note_launch("mxfp8_skinny_kernel<RT=%d,TT=%d> grid=%ux%d m_base=%d", RT, TT, (unsigned)(p.n / (16 * RT)), slabs, p.m_base)) return NVF_OK;
+  if (note_launch("mxfp8_skinny_kernel<RT=%d,TT=%d%s> grid=%ux%d m_base=%d", RT, TT, W == 4 ? ",W=4" : "", (unsigned)(p.n / (16 * RT)), slabs, p.m_base)) return NVF_OK;
   static std::atomic<uint64_t> configured[2] = {{0}, {0}};  // per kernel, one bit per device
   if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured[(p.k & 127) != 0])) return rc;
-  hipLaunchKernelGGL(kern, dim3((unsigned)(p.n / (16 * RT)), (unsigned)slabs), dim3(512), lds_bytes, stream, p);
+  hipLaunchKernelGGL(kern, dim3((unsigned)(p.n / (16 * RT)), (unsigned)slabs), dim3(W * 64), lds_bytes, stream, p);
   return check_launch("mxfp8_skinny_kernel");
 }
 
@@ -803,8 +804,25 @@ int launch_skinny_rt(const Params& p, int rt, hipStream_t stream, int slabs) {
 // (duration: the estimate is compared with another kernel's; then a round of workgroups streams the weight rows it
 // covers, not all of them - with 28672 weight rows a slab takes two rounds, which made the other floor twice the
 // measured time; the choice of the form keeps the floor it was fitted with)
-int64_t mxfp8_skinny_cost(int64_t m, int64_t n, int64_t k, int slab, int rt, int64_t cus, bool duration = false) {
+// (w = 4: the form with 4 wavefronts and a ring of one slot, 64-row slabs x 4 weight tiles.  Two of its workgroups share
+// a compute unit, so up to twice as many as there are compute units run in one round where the form with 8 wavefronts
+// takes two; a wavefront then visits twice the chunks, each 27 % dearer.  Only for that case, and K % 128 == 0.
+// Measured, 8 -> 4 wavefronts: 128 x 14336 x 4096 (448 workgroups) 25.4 -> 19.9 us, 64 x 28672 x 4096 26.0 -> 24.1,
+// 256 x 7168 x 2048 12.7 -> 10.5, 192 x 7168 x 2048 (336) 11.9 -> 9.8; but with one round either way 256 x 4096 x 4096
+// 10.6 -> 12.8 us, 256 x 4096 x 14336 24.9 -> 30.4.  Over the 234 of 2448 shapes (M 33..2048, N 1024..32896, K 512..14336)
+// whose launch the form changes, the time falls by 16 % in the geometric mean, by 28-32 % at K <= 1024, where it also
+// takes over from the persistent kernel: 160 x 8192 x 1024 10.8 -> 6.5 us.)
+int64_t mxfp8_skinny_cost(int64_t m, int64_t n, int64_t k, int slab, int rt, int64_t cus, bool duration = false, int w = 8) {
   if ((slab == 128 && rt != 1) || n % (16 * rt) != 0) return INT64_MAX;
+  if (w == 4) {
+    const int64_t wgs4 = ceil_div(m, 64) * (n / 64);
+    if (slab != 64 || rt != 4 || (n & 63) != 0 || (k & 127) != 0 || m <= 32 || wgs4 <= cus || wgs4 > 2 * cus) return INT64_MAX;
+    // (a deep K makes the second, partly filled round of the other form cheap against its first: 96 x 12288 x 14336,
+    // 384 workgroups, 51 -> 55 us; and many slabs of few columns gain nothing from K = 7168 on: 1024 x 2048 x 7168 28 -> 30 us)
+    if ((k > 8192 && 4 * wgs4 < 7 * cus) || (k > 4096 && m > 8 * 64)) return INT64_MAX;
+    const int64_t per_chunk4 = ((4 + 4) * 145 + 4 * 4 * 10 + 100) * 127 / 100;
+    return std::max(2 * ceil_div(k >> 7, 8) * per_chunk4 + 4 * 4 * 193 + 2493, n * k / 5400);
+  }
   const int64_t slabs = m <= slab ? 1 : ceil_div(m, slab);
   const int tt = m <= slab ? (m <= 16 ? 1 : m <= 32 ? 2 : m <= 64 ? 4 : 8) : slab / 16;
   if (tt == 8 && rt != 1) return INT64_MAX;
@@ -820,23 +838,25 @@ int64_t mxfp8_skinny_cost(int64_t m, int64_t n, int64_t k, int slab, int rt, int
 }
 
 // best form of the skinny kernel for more than 32 rows: estimated duration, slab height and weight tiles per workgroup
-int64_t mxfp8_skinny_best(int64_t m, int64_t n, int64_t k, int64_t cus, int* slab_out, int* rt_out) {
-  int slab = 128, rt = 1;
+int64_t mxfp8_skinny_best(int64_t m, int64_t n, int64_t k, int64_t cus, int* slab_out, int* rt_out, int* w_out) {
+  int slab = 128, rt = 1, w = 8;
   int64_t best = INT64_MAX;
   for (const int s : {32, 64, 128})  // (equal estimates: the lower slab, measured 2-9 % faster)
     for (const int r : {1, 2, 4}) {
       const int64_t c = mxfp8_skinny_cost(m, n, k, s, r, cus);
       if (c < best) best = c, slab = s, rt = r;
     }
+  if (const int64_t c = mxfp8_skinny_cost(m, n, k, 64, 4, cus, false, 4); c < best) best = c, slab = 64, rt = 4, w = 4;
   if (slab_out) *slab_out = slab;
   if (rt_out) *rt_out = rt;
+  if (w_out) *w_out = w;
   return best;
 }
 // estimated duration of the form that mxfp8_skinny_best picks, in ns
 int64_t mxfp8_skinny_ns(int64_t m, int64_t n, int64_t k, int64_t cus) {
-  int slab, rt;
-  if (mxfp8_skinny_best(m, n, k, cus, &slab, &rt) == INT64_MAX) return INT64_MAX;
-  return mxfp8_skinny_cost(m, n, k, slab, rt, cus, true) * 963 / 1000;
+  int slab, rt, w;
+  if (mxfp8_skinny_best(m, n, k, cus, &slab, &rt, &w) == INT64_MAX) return INT64_MAX;
+  return mxfp8_skinny_cost(m, n, k, slab, rt, cus, true, w) * 963 / 1000;
 }
 
 template <bool OUT_BF16>
@@ -847,14 +867,15 @@ int launch_skinny(const Params& p, hipStream_t stream) {
   // (1 with 128-row slabs, whose 8 activation tiles fill the ring), whichever the estimate above prefers
   // (128 x 4096 x 4096: 10.5 us as one slab of 128 rows, 7.6 us as 4 slabs of 32 rows x 4 weight tiles;
   // 256 x 4096 x 14336: 49.9 -> 26.1 us; 128 x 8192 x 7168: 28.0 -> 16.6 us).
-  int slab, rt;
-  mxfp8_skinny_best(p.m, p.n, p.k, cu_count(), &slab, &rt);
+  int slab, rt, w;
+  mxfp8_skinny_best(p.m, p.n, p.k, cu_count(), &slab, &rt, &w);
   // Decode sizes against weight rows a multiple of 8 KiB apart: 2 weight tiles per workgroup stream them slower than
   // 1 or 4 do (measured, 8 rows: 8192 x 8192 15.8 us with 2, 14.3 with 1, 12.6 with 4; 7168 x 8192 13.6 / 12.5 / 11.4;
   // other K: as estimated), so 4 where that still leaves 80 workgroups
   if (p.m <= 32 && rt == 2 && (p.k & 8191) == 0 && (p.n & 63) == 0 && p.n / 64 >= 80) rt = 4;
   const int slabs = p.m <= slab ? 1 : (int)ceil_div(p.m, slab);
   const int rows = p.m <= slab ? p.m : slab;
+  if (w == 4) return launch_skinny_cfg<4, 4, OUT_BF16, 4>(p, stream, slabs);
   return rows <= 16 ? launch_skinny_rt<1, OUT_BF16>(p, rt, stream, slabs)
        : rows <= 32 ? launch_skinny_rt<2, OUT_BF16>(p, rt, stream, slabs)
        : rows <= 64 ? launch_skinny_rt<4, OUT_BF16>(p, rt, stream, slabs)

@@ -68,20 +68,36 @@ def test_deep_k_with_a_workspace_splits_k_only_where_it_wins():
 @pytest.mark.parametrize("m,n,k,kernel", [
     (16, 4096, 4096, "mxfp8_skinny_kernel<RT=1,TT=1> grid=256x1"),
     (128, 4096, 4096, "mxfp8_skinny_kernel<RT=4,TT=2> grid=64x4"),
-    (128, 14336, 4096, "mxfp8_skinny_kernel<RT=4,TT=4> grid=224x2"),
+    (128, 14336, 4096, "mxfp8_skinny_kernel<RT=4,TT=4,W=4> grid=224x2"),
     (128, 4096, 14336, "mxfp8_skinny_kernel<RT=4,TT=2> grid=64x4"),
     (2048, 4096, 4096, "mxfp8_gemm_256_kernel<TM=2,stream_out=0> grid=256"),
     (2048, 14336, 4096, "mxfp8_gemm_256_kernel<TM=4,stream_out=0> grid=256"),
     # streaming or persistent kernel by estimated duration
     (256, 14336, 4096, "mxfp8_gemm_256_kernel<TM=2,stream_out=0> grid=112"),
     (256, 14336, 14336, "mxfp8_gemm_256_kernel<TM=2,stream_out=0> grid=112"),
-    (512, 4096, 7168, "mxfp8_skinny_kernel<RT=4,TT=4> grid=64x8"),
+    (512, 4096, 7168, "mxfp8_skinny_kernel<RT=4,TT=4,W=4> grid=64x8"),
+    (512, 4096, 14336, "mxfp8_skinny_kernel<RT=4,TT=4> grid=64x8"),
     (1024, 2048, 14336, "mxfp8_skinny_kernel<RT=4,TT=4> grid=32x16"),
     (1024, 4096, 4096, "mxfp8_gemm_256_kernel<TM=2,stream_out=0> grid=128"),
     (1024, 8192, 4096, "mxfp8_gemm_256_kernel<TM=2,stream_out=0> grid=256"),
 ])
 def test_mxfp8_llm_and_mid_sized_shapes(m, n, k, kernel):
     assert plan("mxfp8_scaled_mm", m, n, k).startswith(kernel), plan("mxfp8_scaled_mm", m, n, k)
+
+
+def test_mxfp8_streaming_form_with_four_wavefronts_where_it_saves_a_round():
+    """64-row x 64-column workgroups, more than the 256 compute units and at most twice as many: the form of which two
+    share a compute unit (one round instead of two); otherwise, and with K % 128 != 0, the forms with 8 wavefronts."""
+    four = "mxfp8_skinny_kernel<RT=4,TT=4,W=4>"
+    assert plan("mxfp8_scaled_mm", 128, 14336, 4096) == four + " grid=224x2 m_base=0"
+    assert plan("mxfp8_scaled_mm", 64, 28672, 4096) == four + " grid=448x1 m_base=0"
+    assert plan("mxfp8_scaled_mm", 48, 28672, 4096) == four + " grid=448x1 m_base=0"
+    assert plan("mxfp8_scaled_mm", 160, 7168, 2048) == four + " grid=112x3 m_base=0"
+    assert plan("mxfp8_scaled_mm", 256, 8192, 2048) == four + " grid=128x4 m_base=0"
+    for m, n, k in ((128, 7168, 2048), (256, 4096, 4096), (64, 16384, 8192), (128, 14336, 2880), (32, 28672, 4096)):
+        got = plan("mxfp8_scaled_mm", m, n, k)
+        assert got.startswith("mxfp8_skinny_kernel<") and "W=4" not in got, got
+    assert "W=4" not in plan("mxfp8_scaled_mm", 320, 14336, 4096)
 
 
 @pytest.mark.parametrize("m,n,k,kernel", [

@@ -339,7 +339,7 @@ def test_dense_gemms_with_m_not_a_multiple_of_128(dev, shape):
 
 
 @pytest.mark.parametrize("shape", [(2048, 2432, 256), (2100, 2368, 384), (1536, 4128, 256), (640, 4224, 2048), (2048, 4224, 2048),
-                                   (100, 12416, 512), (200, 12352, 512), (200, 32896, 2048)])
+                                   (100, 16512, 512), (200, 12352, 512), (200, 32896, 2048)])
 def test_dense_gemms_with_n_not_a_multiple_of_256(dev, shape):
     """N > 256 and not a multiple of 256: the columns up to the last multiple of 256 go to the persistent kernel, the
     remaining 32..224 columns to a launch of their own (tile kernel or weight-streaming kernel) that writes into the same
@@ -726,6 +726,35 @@ def test_mxfp8_gemm_decode_sized_activations(dev, shape):
         assert out.shape == (m, n)
         assert ((out.float().cpu() - ref).abs() / scale).max().item() <= GEMM_MAX_REL, (shape, dtype)
         assert torch.equal(out, _run_mxfp8(a, b, sa_p, sb, 0.75, dtype, dev))
+
+
+@pytest.mark.parametrize("shape", [(100, 14336, 640), (160, 7168, 2048), (250, 7744, 256), (192, 6144, 128), (48, 28672, 384),
+                                   (128, 14336, 4096)])
+def test_mxfp8_gemm_streaming_form_with_four_wavefronts(dev, shape):
+    """More 64-row x 64-column workgroups than compute units, at most twice as many: the form with 4 wavefronts and a
+    one-slot ring, of which two workgroups share a compute unit, so that one round does.  Ragged last slabs (36, 32 and 58 of
+    64 rows, one slab of 48), K of one and two chunks (wavefronts without any chunk add zeros); every element compared,
+    both output types, NaN codes in all scale padding, run-to-run bit equality."""
+    from fuser_amd import capi
+
+    m, n, k = shape
+    gen = torch.Generator().manual_seed(m + n + k)
+    a, sa = _mxfp8_operand(m, k, gen, 1.0)
+    b, sb = _mxfp8_operand(n, k, gen, 1.0)
+    ref = O.ref_mxfp8_scaled_mm(a, b, sa, sb, 0.75)
+    scale = ref.abs().amax(dim=1, keepdim=True).clamp(min=1e-30)
+    sa_p, sb_p = sa.clone(), sb.clone()
+    sa_p[O.linear_to_swizzled_128_4(torch.ones(m, k // 32, dtype=torch.uint8)) == 0] = 0xFF
+    sb_p[O.linear_to_swizzled_128_4(torch.ones(n, k // 32, dtype=torch.uint8)) == 0] = 0xFF
+    plan = capi.describe_dispatch("mxfp8_scaled_mm", m, n, k)
+    assert plan.startswith("mxfp8_skinny_kernel<RT=4,TT=4,W=4>") and ";" not in plan, plan
+    for dtype in (torch.bfloat16, torch.float16):
+        if dtype == torch.float16 and ref.abs().max() > 6e4:
+            continue
+        out = _run_mxfp8(a, b, sa_p, sb_p, 0.75, dtype, dev)
+        assert out.shape == (m, n) and torch.isfinite(out.float()).all()
+        assert ((out.float().cpu() - ref).abs() / scale).max().item() <= GEMM_MAX_REL, (shape, dtype)
+        assert torch.equal(out, _run_mxfp8(a, b, sa_p, sb_p, 0.75, dtype, dev))
 
 
 @pytest.mark.parametrize("nk", [(1024, 2048), (2048, 4096), (4096, 2048), (6144, 2176), (4096, 7168), (8192, 1152), (14336, 640),
