@@ -50,10 +50,11 @@ __device__ __forceinline__ void dequant_frags(const u32x4 q, uint32_t s2, u32x4 
 // 16*RT weight rows and each walks all of K on its own - a long pipeline per wavefront and no reduction -
 // instead of sharing one block and splitting K.
 // RAGGED_K: K % 128 != 0 (a kernel of its own: the tests for the short chunk cost the others 4-8 %).
-template <int RT, int TT, bool OUT_BF16, int DEPTH, bool GROUPED = false, bool NSPLIT = false, bool RAGGED_K = false>
-__global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) {
+// W: wavefronts per workgroup, 8 or (dense, 4 x 8 tiles) 4; two wavefronts per SIMD in both cases, i.e. at most 256
+// registers, so that two workgroups of 4 fit a compute unit.
+template <int RT, int TT, bool OUT_BF16, int DEPTH, bool GROUPED = false, bool NSPLIT = false, bool RAGGED_K = false, int W = 8>
+__global__ __launch_bounds__(W * 64, 2) void nvfp4_skinny_ring_kernel(const Params p) {
   static_assert(GROUPED || !NSPLIT, "the dense op has too few row blocks to give every wavefront its own");
-  constexpr int W = 8;
   constexpr int NT = RT + TT;
   // Scale blocks (1 KiB) per operand and chunk: one.  A block holds, for a pair of 16-row tiles, the 16-byte pieces of
   // the 128x4 layout with the scale words of rows {row, row+32, row+64, row+96}: the pairs of an operand (rows 32 apart)
@@ -265,7 +266,7 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
         for (int tt = 0; tt < TTC; ++tt)
           if (tt < tt_count) red[(wave * tiles + r2 * tt_count + tt) * 64 + lane] = acc[round * RPR + r2][tt];
       __syncthreads();
-      for (int u = tid; u < units; u += 512) {
+      for (int u = tid; u < units; u += W * 64) {
         const int l = u & 63, tile = u >> 6;
         const int r2 = tile / tt_count, tt = tile - r2 * tt_count;
         f32x4 s = red[u];
@@ -320,11 +321,11 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
       // workgroup's scale columns; the last slab's workgroups) and the columns past N / 16 (the last workgroup)
       const int64_t sf_cols = (int64_t)p.n >> 4, padded = (sf_cols + 3) & ~(int64_t)3;
       const int m_pad = (p.m + 127) & ~127;
-      for (int i = tid; i < (m_pad - p.m) * RT; i += 512)
+      for (int i = tid; i < (m_pad - p.m) * RT; i += W * 64)
         p.out_sf[swizzle_128x4(p.m + i / RT, (n0 >> 4) + i % RT, padded)] = 0;
       if (blockIdx.x == gridDim.x - 1 && padded != sf_cols) {
         const int pc = (int)(padded - sf_cols);
-        for (int i = tid; i < m_pad * pc; i += 512) p.out_sf[swizzle_128x4(i / pc, sf_cols + i % pc, padded)] = 0;
+        for (int i = tid; i < m_pad * pc; i += W * 64) p.out_sf[swizzle_128x4(i / pc, sf_cols + i % pc, padded)] = 0;
       }
     }
   };
@@ -725,25 +726,35 @@ __global__ __launch_bounds__(512) void nvfp4_skinny_ring_kernel(const Params p) 
   }
 }
 
-template <int RT, int TT, bool OUT_BF16>
+template <int RT, int TT, bool OUT_BF16, int W = 8>
 int launch_nvfp4_skinny_ring_cfg(const Params& p, hipStream_t stream, int slabs = 1) {
   constexpr int SLOT_KIB = RT + TT + (RT + 1) / 2 + (TT + 1) / 2;
   // one slot per wavefront also where two would fit (M=16, N=14336, K=4096: 8.0 -> 7.5 us; K=14336: 9.6 -> 9.2 us)
   constexpr int DEPTH = 1;
-  auto kern = (p.k & 127) != 0 ? nvfp4_skinny_ring_kernel<RT, TT, OUT_BF16, DEPTH, false, false, true> : nvfp4_skinny_ring_kernel<RT, TT, OUT_BF16, DEPTH>;
-  // the ring; the reduction reuses it and needs 8 KiB per partial tile of a round
-  constexpr int red_kib = 8 * (RT * TT <= 8 ? RT * TT : TT);
-  constexpr int ring_kib = 8 * DEPTH * SLOT_KIB;
+  // More workgroups than compute units (slabs of 128 rows x blocks of 64 weight rows): 4 wavefronts each, so that two
+  // share a compute unit (72 KiB of LDS each, 2 wavefronts per SIMD either way) and one streams while the other reduces,
+  // stores and starts.  Measured, 8 -> 4 wavefronts: 192 x 14336 x 4096 (448 workgroups) 33.6 -> 28.0 us, 256 x 14336 x 4096
+  // 40.2 -> 36.5, 128 x 28672 x 4096 38.8 -> 35.1, 384 x 16384 x 4096 (768) 58.8 -> 53.1, 512 x 8192 x 8192 66.1 -> 63.6;
+  // but up to one workgroup per compute unit 128 x 14336 x 4096 22.1 -> 27.3.
+  if constexpr (W == 8 && RT == 4 && TT == 8) {
+    if ((p.k & 127) == 0 && p.partial == nullptr && (int64_t)(p.n / 64) * slabs > cu_count())
+      return launch_nvfp4_skinny_ring_cfg<RT, TT, OUT_BF16, 4>(p, stream, slabs);
+  }
+  auto kern = W == 8 && (p.k & 127) != 0 ? nvfp4_skinny_ring_kernel<RT, TT, OUT_BF16, DEPTH, false, false, W == 8, W>
+                                         : nvfp4_skinny_ring_kernel<RT, TT, OUT_BF16, DEPTH, false, false, false, W>;
+  // the ring; the reduction reuses it and needs 1 KiB per wavefront and partial tile of a round
+  constexpr int red_kib = W * (RT * TT <= 8 ? RT * TT : TT);
+  constexpr int ring_kib = W * DEPTH * SLOT_KIB;
   constexpr int lds_bytes = (ring_kib > red_kib ? ring_kib : red_kib) * 1024;
   static_assert(lds_bytes <= 160 * 1024, "LDS");
   const int splits = p.partial != nullptr ? p.splits : 1;
   if (splits > 1 ? note_launch("nvfp4_skinny_ring_kernel<RT=%d,TT=%d> grid=%ux%dx%d split_k + splitk_reduce_kernel", RT, TT,
                                (unsigned)(p.n / (16 * RT)), slabs, splits)
-                 : note_launch("nvfp4_skinny_ring_kernel<RT=%d,TT=%d> grid=%ux%d", RT, TT, (unsigned)(p.n / (16 * RT)), slabs))
+                 : note_launch("nvfp4_skinny_ring_kernel<RT=%d,TT=%d%s> grid=%ux%d", RT, TT, W == 4 ? ",W=4" : "", (unsigned)(p.n / (16 * RT)), slabs))
     return NVF_OK;
   static std::atomic<uint64_t> configured[2] = {{0}, {0}};  // per kernel, one bit per device
   if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured[(p.k & 127) != 0])) return rc;
-  hipLaunchKernelGGL(kern, dim3((unsigned)(p.n / (16 * RT)), (unsigned)slabs, (unsigned)splits), dim3(512), lds_bytes, stream, p);
+  hipLaunchKernelGGL(kern, dim3((unsigned)(p.n / (16 * RT)), (unsigned)slabs, (unsigned)splits), dim3(W * 64), lds_bytes, stream, p);
   if (const int rc = check_launch("nvfp4_skinny_ring_kernel")) return rc;
   if (p.partial == nullptr) return NVF_OK;
   const int64_t mn = (int64_t)p.m * p.n;

@@ -104,9 +104,9 @@ def test_mxfp8_streaming_form_with_four_wavefronts_where_it_saves_a_round():
     # streaming, persistent (256x256 / 128x256 tiles) or tile kernel by estimated duration
     (512, 4096, 4096, "nvfp4_skinny_ring_kernel<RT=4,TT=8> grid=64x4"),
     (1024, 2048, 4096, "nvfp4_skinny_ring_kernel<RT=4,TT=8> grid=32x8"),
-    (640, 8192, 4096, "nvfp4_skinny_ring_kernel<RT=4,TT=8> grid=128x5"),
-    (1024, 4096, 14336, "nvfp4_skinny_ring_kernel<RT=4,TT=8> grid=64x8"),
-    (256, 14336, 4096, "nvfp4_skinny_ring_kernel<RT=4,TT=8> grid=224x2"),
+    (640, 8192, 4096, "nvfp4_skinny_ring_kernel<RT=4,TT=8,W=4> grid=128x5"),
+    (1024, 4096, 14336, "nvfp4_skinny_ring_kernel<RT=4,TT=8,W=4> grid=64x8"),
+    (256, 14336, 4096, "nvfp4_skinny_ring_kernel<RT=4,TT=8,W=4> grid=224x2"),
     (1024, 8192, 4096, "nvfp4_gemm_256_kernel<grouped=0,TM=2,f32=0,pairs=1> grid=256"),
     (512, 14336, 4096, "nvfp4_gemm_256_kernel<grouped=0,TM=2,f32=0,pairs=1> grid=224"),
     (768, 14336, 4096, "nvfp4_gemm_256_kernel<grouped=0,TM=4,f32=0,pairs=1> grid=168"),

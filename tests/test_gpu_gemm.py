@@ -84,17 +84,18 @@ def test_nvfp4_gemm_epilogue_reference_shapes(dev, dtype, shape):
 
 @pytest.mark.parametrize("shape", [(200, 160, 192), (4096, 3072, 256), (1920, 4096, 384), (1024, 2048, 384), (300, 544, 608), (64, 96, 64),
                                    (2176, 2048, 256), (4096, 4128, 128), (2100, 4096, 256), (4000 + 77, 2048, 384),
-                                   (16, 4096, 512), (100, 14336, 256), (128, 2048, 1024), (300, 4096, 2048), (48, 1056, 384), (1000, 14336, 256)])
+                                   (16, 4096, 512), (100, 14336, 256), (128, 2048, 1024), (300, 4096, 2048), (48, 1056, 384), (1000, 14336, 256),
+                                   (200, 14336, 256), (100, 28672, 128)])
 def test_nvfp4_gemm_epilogue_quantizes_its_own_fp32_product_bit_exactly(dev, shape):
     """Through the C ABI.  The result is quantized in the GEMM's epilogue; with a workspace the call also dumps the
     fp32 product it quantized: that agrees with the oracle product to fp32 summation noise, and payload and scales
     are bit-identical to the oracle quantizer applied to exactly that product (rows not a multiple of 128 and
     padded scale columns on the 64x64, 128x128 and 256x256 tile kernels; shapes on the persistent kernel with
     256x256 and with 128x256 tiles; the last two: M not a multiple of 128, cut into a part for the persistent kernel
-    and the remaining rows for the tile kernels, whose payload and scale tiles follow the first part's; the last six:
+    and the remaining rows for the tile kernels, whose payload and scale tiles follow the first part's; the six before the last two:
     shapes that the 16-bit op streams - one to eight activation row tiles, one to four weight tiles per workgroup, one
     and several slabs, and 104 rows streamed behind 896 on the persistent kernel - where the weight-streaming kernel's
-    last stage quantizes the summed product)."""
+    last stage quantizes the summed product; the two after those: the same on its form with 4 wavefronts)."""
     from fuser_amd import capi
 
     m, n, k = shape
@@ -240,6 +241,30 @@ def test_nvfp4_gemm_decode_sized_activations(dev, shape):
     for dtype in (torch.bfloat16, torch.float16):
         out = _run_nvfp4(a, b, sa_p, sb, alpha, dtype, dev)
         assert out.shape == (m, n) and max_rel(out, ref) <= GEMM_MAX_REL, (shape, dtype)
+        assert torch.equal(out, _run_nvfp4(a, b, sa_p, sb, alpha, dtype, dev))
+
+
+@pytest.mark.parametrize("shape", [(200, 14336, 256), (100, 28672, 128), (256, 14336, 640), (300, 8256, 512), (256, 16384, 4096)])
+def test_nvfp4_gemm_streaming_form_with_four_wavefronts(dev, shape):
+    """More workgroups (128-row slabs x 64 weight rows) than compute units: the streaming kernel runs with 4 wavefronts
+    per workgroup, two workgroups to a compute unit.  Ragged last slabs (72, 100 and 44 of 128 rows), K of one to five
+    chunks (wavefronts without any chunk add zeros) and 32; every element compared, both output types, NaN codes in the
+    scale padding of the activations, run-to-run bit equality."""
+    from fuser_amd import capi
+
+    m, n, k = shape
+    gen = torch.Generator().manual_seed(m + n + k)
+    a, sa, ga = _nvfp4_operand(m, k, 1.0, gen)
+    b, sb, gb = _nvfp4_operand(n, k, 0.02, gen)
+    alpha = 1.0 / (ga * gb)
+    ref = O.ref_nvfp4_scaled_mm(a, b, sa, sb, alpha)
+    sa_p = sa.clone()
+    sa_p[O.linear_to_swizzled_128_4(torch.ones(m, k // 16, dtype=torch.uint8)) == 0] = 0x7F
+    plan = capi.describe_dispatch("nvfp4_scaled_mm", m, n, k)
+    assert plan.startswith("nvfp4_skinny_ring_kernel<RT=4,TT=8,W=4>") and ";" not in plan, plan
+    for dtype in (torch.bfloat16, torch.float16):
+        out = _run_nvfp4(a, b, sa_p, sb, alpha, dtype, dev)
+        assert out.shape == (m, n) and max_rel_rowwise(out, ref) <= GEMM_MAX_REL, (shape, dtype)
         assert torch.equal(out, _run_nvfp4(a, b, sa_p, sb, alpha, dtype, dev))
 
 
