@@ -176,8 +176,15 @@ int launch_nvfp4_tile(const Params& p, int grid, hipStream_t stream) {
 // two to a compute unit: 68 per such round, 45 for a last round of one tile per compute unit, and 22..47 when there
 // is no more than that in all (all measured: M = 128..1024, N = 2048..14336, K = 4096 and 14336).
 // the streaming kernel's cost estimate is in ns within 0.8 (K = 2048) .. 1.1 (K = 14336)
+// (the form with 4 wavefronts: its discount in the cost holds among the streaming forms; against the tiles it made 26 of
+// 91 changed picks slower, at K = 2048 and 7168, and 43 faster, so there only 4 % of it stay, for 3072 <= K < 6144:
+// 1536 x 11008 x 4096 162 -> 139 us, 160 x 29568 x 4096 58 -> 46)
 int64_t nvfp4_stream_ns(int64_t m, int64_t n, int64_t k, int cus) {
-  return nvfp4_skinny_best(m, n, k, cus, nullptr, nullptr) * (k < 3072 ? 82 : k < 6144 ? 96 : k < 10240 ? 103 : 110) / 100;
+  int slab, rt;
+  int64_t cost = nvfp4_skinny_best(m, n, k, cus, &slab, &rt);
+  if (slab == 128 && rt == 4 && m > 64 && (k & 127) == 0 && ceil_div(m, 128) * (n / 64) > cus)
+    cost = cost * (k >= 3072 && k < 6144 ? 96 : 100) / nvfp4_four_wavefront_percent(k);
+  return cost * (k < 3072 ? 82 : k < 6144 ? 96 : k < 10240 ? 103 : 110) / 100;
 }
 struct DensePlan {
   enum Kernel { kStream, kTiles256, kTiles128, kOther } kernel;

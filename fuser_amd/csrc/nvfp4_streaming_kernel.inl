@@ -809,6 +809,7 @@ int launch_nvfp4_skinny_rt(const Params& p, int rt, hipStream_t stream, int slab
 // the nine (slab, rt) forms over M = 48..256, N = 1024..14336, K = 2048..14336 (144 shapes: the form picked is within
 // 8 % of the fastest for 134 of them, 1.8 % off on average; a fixed rule by N alone was 13 % off); for 1..32 rows
 // (112 shapes) its pick of rt is 0.2 % off the fastest on average.
+inline int nvfp4_four_wavefront_percent(int64_t k) { return k < 768 ? 73 : k < 1536 ? 78 : k < 3072 ? 85 : k < 6144 ? 89 : k < 10240 ? 92 : 95; }
 int64_t nvfp4_skinny_cost(int64_t m, int64_t n, int64_t k, int slab, int rt, int cus) {
   if (n % (16 * rt) != 0) return INT64_MAX;
   const int64_t slabs = m <= slab ? 1 : ceil_div(m, slab);
@@ -824,6 +825,9 @@ int64_t nvfp4_skinny_cost(int64_t m, int64_t n, int64_t k, int slab, int rt, int
   const int64_t rounds = ceil_div(wgs, cus * per_cu);
   const int64_t per_chunk = (rt + tt) * 183 + rt * tt * 18 + 100;
   const int64_t wg_time = chunks * per_chunk * (100 + 73 * (resident - 1)) / 100 + rt * tt * 110 + 5070;
+  // (4 x 8 tiles with more workgroups than compute units run as workgroups of 4 wavefronts, two to a compute unit:
+  // measured 27 % (K = 512) .. 5 % (K = 14336) faster than the rounds of one workgroup per compute unit)
+  if (rt == 4 && tt == 8 && (k & 127) == 0 && wgs > cus) return rounds * wg_time * nvfp4_four_wavefront_percent(k) / 100;
   return rounds * wg_time;
 }
 
