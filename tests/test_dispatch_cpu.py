@@ -85,6 +85,20 @@ def test_mxfp8_llm_and_mid_sized_shapes(m, n, k, kernel):
     assert plan("mxfp8_scaled_mm", m, n, k).startswith(kernel), plan("mxfp8_scaled_mm", m, n, k)
 
 
+def test_nvfp4_streaming_form_with_four_wavefronts_with_more_workgroups_than_compute_units():
+    """128-row slabs x 64 weight rows, K % 128 == 0, more workgroups than the 256 compute units: workgroups of 4 wavefronts,
+    two to a compute unit.  The form's measured gain is part of the streaming estimate among the streaming forms (160
+    rows: two slabs of 128 rows instead of five of 32), and for 3072 <= K < 6144, by 4 %, against the persistent tiles."""
+    four = "nvfp4_skinny_ring_kernel<RT=4,TT=8,W=4>"
+    assert plan("nvfp4_scaled_mm", 256, 14336, 4096) == four + " grid=224x2"
+    assert plan("nvfp4_scaled_mm", 160, 29568, 14336) == four + " grid=462x2"
+    assert plan("nvfp4_scaled_mm", 160, 32896, 1024) == four + " grid=514x2"
+    assert plan("nvfp4_scaled_mm", 1536, 12288, 4096) == four + " grid=192x12"
+    assert plan("nvfp4_scaled_mm", 1536, 12288, 2048).startswith("nvfp4_gemm_256_kernel<grouped=0,TM=2")
+    assert plan("nvfp4_scaled_mm", 128, 14336, 4096) == "nvfp4_skinny_ring_kernel<RT=4,TT=8> grid=224x1"
+    assert plan("nvfp4_scaled_mm", 256, 14336, 2880) == "nvfp4_skinny_ring_kernel<RT=4,TT=8> grid=224x2"
+
+
 def test_mxfp8_streaming_form_with_four_wavefronts_where_it_saves_a_round():
     """64-row x 64-column workgroups, more than the 256 compute units and at most twice as many: the form of which two
     share a compute unit (one round instead of two); otherwise, and with K % 128 != 0, the forms with 8 wavefronts."""
