@@ -763,17 +763,17 @@ int launch_nvfp4_skinny_ring_cfg(const Params& p, hipStream_t stream, int slabs 
   return check_launch("splitk_reduce_kernel");
 }
 
-template <int RT, int TT, bool OUT_BF16, bool NSPLIT>
+template <int RT, int TT, bool OUT_BF16, bool NSPLIT, int W = 8>
 int launch_nvfp4_skinny_grouped(const Params& p0, int rows_lo, int rows_hi, hipStream_t stream) {
   constexpr int SLOT_KIB = RT + TT + (RT + 1) / 2 + (TT + 1) / 2;
   // One slot per wavefront also where two would fit: measured faster for the groups of up to 32 rows (512 rows
   // over 256 experts, K=7168: 401 -> 375 us; K=2048: 432 -> 413 us).  Forcing the registers down to two
   // workgroups per compute unit on top of that costs more than it gains (450 us).
   constexpr int DEPTH = 1;
-  auto kern = (p0.k & 127) != 0 ? nvfp4_skinny_ring_kernel<RT, TT, OUT_BF16, DEPTH, true, NSPLIT, true>
-                                : nvfp4_skinny_ring_kernel<RT, TT, OUT_BF16, DEPTH, true, NSPLIT>;
-  constexpr int red_kib = NSPLIT ? 0 : 8 * (RT * TT <= 8 ? RT * TT : TT);
-  constexpr int ring_kib = 8 * DEPTH * SLOT_KIB;
+  auto kern = W == 8 && (p0.k & 127) != 0 ? nvfp4_skinny_ring_kernel<RT, TT, OUT_BF16, DEPTH, true, NSPLIT, W == 8, W>
+                                          : nvfp4_skinny_ring_kernel<RT, TT, OUT_BF16, DEPTH, true, NSPLIT, false, W>;
+  constexpr int red_kib = NSPLIT ? 0 : W * (RT * TT <= 8 ? RT * TT : TT);
+  constexpr int ring_kib = W * DEPTH * SLOT_KIB;
   constexpr int lds_bytes = (ring_kib > red_kib ? ring_kib : red_kib) * 1024;
   static_assert(lds_bytes <= 160 * 1024, "LDS");
   Params p = p0;
@@ -785,13 +785,19 @@ int launch_nvfp4_skinny_grouped(const Params& p0, int rows_lo, int rows_hi, hipS
   if (rows_lo > 1) p.class_slots = (int)std::min<int64_t>(p.groups, p.m / rows_lo);
   if (rows_lo > 1 && p.class_slots == 0) return NVF_OK;  // fewer rows in all than one such group has
   const int64_t wgs = (int64_t)(p.class_slots ? p.class_slots : p.groups) * (p.n / (16 * RT * (NSPLIT ? 8 : 1)));
+  // (groups of 33-128 rows, more workgroups than compute units: 4 wavefronts each and two to a compute unit, as in the
+  // dense launch; 8 experts x 64 rows, N=14336, K=4096: 111 -> 86 us, 32 x 40 rows, N=7168: 180 -> 142, 64 x 64 rows,
+  // N=2048, K=7168: 187 -> 164)
+  if constexpr (W == 8 && RT == 4 && TT == 8 && !NSPLIT) {
+    if ((p.k & 127) == 0 && wgs > cu_count()) return launch_nvfp4_skinny_grouped<RT, TT, OUT_BF16, NSPLIT, 4>(p0, rows_lo, rows_hi, stream);
+  }
   if (wgs >= ((int64_t)1 << 31)) return fail(NVF_ERR_UNSUPPORTED_SHAPE, "too many (group, row block) pairs for one launch");
-  if (note_launch("nvfp4_skinny_ring_kernel<RT=%d,TT=%d,grouped,nsplit=%d> grid=%lld rows=%d..%d", RT, TT, (int)NSPLIT, (long long)wgs, rows_lo,
-                  rows_hi))
+  if (note_launch("nvfp4_skinny_ring_kernel<RT=%d,TT=%d,grouped,nsplit=%d%s> grid=%lld rows=%d..%d", RT, TT, (int)NSPLIT, W == 4 ? ",W=4" : "", (long long)wgs,
+                  rows_lo, rows_hi))
     return NVF_OK;
   static std::atomic<uint64_t> configured[2] = {{0}, {0}};  // per kernel, one bit per device
   if (const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured[(p.k & 127) != 0])) return rc;
-  hipLaunchKernelGGL(kern, dim3((unsigned)wgs), dim3(512), lds_bytes, stream, p);
+  hipLaunchKernelGGL(kern, dim3((unsigned)wgs), dim3(W * 64), lds_bytes, stream, p);
   return check_launch("nvfp4_skinny_ring_kernel (grouped)");
 }
 

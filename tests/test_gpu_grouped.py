@@ -422,13 +422,15 @@ def test_nvfp4_grouped_mm_mid_sized_groups_of_a_prefill(dev, n, k):
         assert torch.equal(out[:rows], nvf_cutlass.nvfp4_scaled_grouped_mm(*args, dtype)[:rows])
 
 
-@pytest.mark.parametrize("n,k,few_rows", [(256, 4096, False), (128, 4224, False), (256, 512, False), (256, 512, True), (128, 4096, True)])
+@pytest.mark.parametrize("n,k,few_rows", [(256, 4096, False), (128, 4224, False), (256, 512, False), (256, 512, True), (128, 4096, True),
+                                          (1024, 4096, False), (2048, 512, True)])
 def test_nvfp4_grouped_mm_mid_sized_groups_below_the_prefill_size(dev, n, k, few_rows):
     """300 experts, most of them with 0..3 rows, a few with 33..128 at indices on both sides of the borders at which
     the streaming kernel counts the groups of a size class (63 | 64, 255 | 256, the last one), two large ones.  Up to
     1024 rows in all, or below 6144 with K >= 4096, the mid-sized groups stream their weights from a launch with one
     block of workgroups per group of 33 rows that the call could hold (the block finds its group by rank); otherwise
-    they run as 128x256 tiles of the persistent kernel.  A different alpha per group, poisoned padding of the activation
+    they run as 128x256 tiles of the persistent kernel.  The last two shapes give that launch more workgroups than compute
+    units: workgroups of 4 wavefronts, two to a compute unit.  A different alpha per group, poisoned padding of the activation
     scale slabs; every element compared, rows after the last group untouched, run-to-run bit equality."""
     from fuser_amd import capi, nvf_cutlass
 
@@ -446,6 +448,7 @@ def test_nvfp4_grouped_mm_mid_sized_groups_below_the_prefill_size(dev, n, k, few
     got = capi.describe_dispatch("nvfp4_scaled_grouped_mm", m, n, k, groups=g)
     mid = [part for part in got.split("; ") if "rows=33..128" in part]
     assert len(mid) == 1 and mid[0].startswith("nvfp4_skinny_ring_kernel<" if few_rows or k >= 4096 else "nvfp4_gemm_256_kernel<grouped=1,TM=2"), got
+    assert (",W=4>" in mid[0]) == (n >= 1024), got
     gen = torch.Generator().manual_seed(n + k + few_rows)
     x = torch.randn(m, k, generator=gen).bfloat16()
     w = (torch.randn(8, n, k, generator=gen) * 0.05).bfloat16()  # eight different experts, repeated
