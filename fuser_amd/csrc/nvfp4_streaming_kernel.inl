@@ -833,7 +833,17 @@ int64_t nvfp4_skinny_cost(int64_t m, int64_t n, int64_t k, int slab, int rt, int
   const int64_t wg_time = chunks * per_chunk * (100 + 73 * (resident - 1)) / 100 + rt * tt * 110 + 5070;
   // (4 x 8 tiles with more workgroups than compute units run as workgroups of 4 wavefronts, two to a compute unit:
   // measured 27 % (K = 512) .. 5 % (K = 14336) faster than the rounds of one workgroup per compute unit)
-  if (rt == 4 && tt == 8 && (k & 127) == 0 && wgs > cus) return rounds * wg_time * nvfp4_four_wavefront_percent(k) / 100;
+  if (rt == 4 && tt == 8 && (k & 127) == 0 && wgs > cus) {
+    // (two workgroups share a compute unit and a short one makes room early: the workgroups of a last slab with fewer
+    // row tiles count by their share of a full one's time - 320 x 11008 x 2048: 2.6 slabs x 172 in 2 rounds, not 3)
+    int64_t rounds4 = rounds;
+    const int tt_last = m > slab ? (int)ceil_div(m % slab, 16) : 0;
+    if (tt_last != 0) {
+      const int64_t wg_last = chunks * ((rt + tt_last) * 183 + rt * tt_last * 18 + 100) + rt * tt_last * 110 + 5070;
+      rounds4 = ceil_div((slabs - 1) * (n / 64) * wg_time + (n / 64) * wg_last, wg_time * cus);
+    }
+    return rounds4 * wg_time * nvfp4_four_wavefront_percent(k) / 100;
+  }
   return rounds * wg_time;
 }
 
