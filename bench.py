@@ -43,6 +43,8 @@ def parse():
                     "(counter runs attribute a replayed graph's kernels poorly)")
     ap.add_argument("--only", default="", help="profiling aid: run just this extra workload "
                     "(quant | fused | nvfp4 | llm | grouped | gnvfp4) and print its line")
+    ap.add_argument("--shapes", default="", help="profiling aid: time dense GEMMs of these shapes only and print their "
+                    "launches, e.g. mxfp8:128x14336x4096,nvfp4:160x28672x14336 (bf16 result, N(0,1) activations)")
     return ap.parse_args()
 
 
@@ -81,6 +83,26 @@ def main():
         torch.cuda.synchronize()
         wall = (time.perf_counter() - t0) * 1e3 / steps
         return e0.elapsed_time(e1) / steps, wall
+
+    if args.shapes:
+        res = {}
+        gen = torch.Generator(device=dev).manual_seed(0)
+        for spec in args.shapes.split(","):
+            op, dims = spec.split(":")
+            m, n, k = (int(v) for v in dims.split("x"))
+            x = torch.randn(m, k, device=dev, generator=gen).bfloat16()
+            w = (torch.randn(n, k, device=dev, generator=gen) * 0.02).bfloat16()
+            if op == "mxfp8":
+                (qx, sx), (qw, sw) = (ops.nv_block_quantize(t, None, True, 32, torch.float8_e4m3fn) for t in (x, w))
+                fn, name = (lambda: nvf_cutlass.mxfp8_scaled_mm(qx, qw, sx, sw, one, torch.bfloat16)), "mxfp8_scaled_mm"
+            else:
+                (qx, sx), (qw, sw) = (ops.nv_block_quantize(t, None, True, 16) for t in (x, w))
+                fn, name = (lambda: nvf_cutlass.nvfp4_scaled_mm(qx, qw, sx, sw, one, torch.bfloat16)), "nvfp4_scaled_mm"
+            ms, _ = timed(fn, args.steps, args.warmup)
+            res[spec] = {"us": round(ms * 1e3, 2), "TFLOP/s": round(2.0 * m * n * k / ms / 1e9, 1),
+                         "launches": capi.describe_dispatch(name, m, n, k)}
+        print(json.dumps({"shapes": res}))
+        return
 
     def timed_graph(calls, replays=20):
         if args.no_graph:
